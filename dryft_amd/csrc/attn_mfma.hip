@@ -1,0 +1,308 @@
+// bfloat16 attention on the matrix cores (v_mfma_f32_16x16x32_bf16), reading keys and values from
+// the paged cache: a causal kernel for steps that bring many rows per sequence, and a split
+// kernel plus a combine for steps that bring one row per sequence. They stand where the reference
+// uses a library's flash attention for prompts (engine/dryft_qwen3/model.py:172-177) and its
+// split-KV kernel for decoding (kernels/attn_decode.py:36-118). Scores, running maximum, exponentials,
+// row sums and the output accumulator are float; probabilities are rounded to bfloat16 for the
+// second product (attn_decode.py:12-14, 89).
+//
+// A wave owns 16 query rows. It forms transposed tiles so that no operand has to be moved between
+// lanes:   S^T[key, row] = K[key, :] . Q[row, :]        (A = K from its page, B = Q from registers)
+//          O^T[d, row]  += V^T[d, key] * P^T[key, row]  (A = V^T from its page, B = P^T = S^T's own layout)
+// In the 16x16 result layout lane l holds column l%16 and rows 4*(l/16)..+3, while a B operand of the
+// 32-deep product wants 8 consecutive contraction indices per lane. Since a sum does not care about the
+// order of its terms, contraction index 8*(l/16)+i of the second product stands for key 4*(l/16)+i of the
+// first 16-key tile when i < 4 and for key 16+4*(l/16)+(i-4) of the second tile otherwise; V^T is fetched
+// in the same order.
+#include "common.h"
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+#define MFMA16(a, b, c) __builtin_amdgcn_mfma_f32_16x16x32_bf16((a), (b), (c), 0, 0, 0)
+
+__device__ __forceinline__ bf16x8 zero8() {
+  bf16x8 z;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) z[i] = (__bf16)0.f;
+  return z;
+}
+
+__device__ __forceinline__ bf16x8 load8(const bf16_t* p) { return *(const bf16x8*)p; }
+
+__device__ __forceinline__ __bf16 to_bf16(float f) {
+  bf16_t b = float_to_bf16(f);
+  return __builtin_bit_cast(__bf16, b.bits);
+}
+
+// State of one wave's 16 rows while it walks over pages of keys.
+template <int KB>  // KB = ceil(head_dim / 32)
+struct RowBlock {
+  bf16x8 q[KB];          // B operand of the first product, per 32 features
+  f32x4 o[2 * KB];       // O^T tiles of 16 features each
+  float m, l;            // running maximum and sum of the lane's own row (l % 16)
+};
+
+// One page (64 keys) for one wave. `key0` is the position of the page's first key; the lane's row sees
+// keys j with lo_row <= j <= hi_row. K page: [64][head_dim]; V^T page: [head_dim][64].
+template <int KB>
+__device__ __forceinline__ void attend_page(RowBlock<KB>& st, const bf16_t* __restrict__ k_page,
+                                            const bf16_t* __restrict__ v_page, int head_dim, float scale, int key0,
+                                            int lo_row, int hi_row) {
+  const int lane = threadIdx.x % WAVE, c = lane % 16, g = lane / 16;
+  f32x4 s[4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    s[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int kb = 0; kb < KB; ++kb) {
+      const int d = 32 * kb + 8 * g;
+      const bf16x8 a = d < head_dim ? load8(k_page + (16 * t + c) * head_dim + d) : zero8();
+      s[t] = MFMA16(a, st.q[kb], s[t]);
+    }
+  }
+  float tile_max = -INFINITY;
+#pragma unroll
+  for (int t = 0; t < 4; ++t)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int j = key0 + 16 * t + 4 * g + i;
+      const float v = (j >= lo_row && j <= hi_row) ? s[t][i] * scale : -INFINITY;
+      s[t][i] = v;
+      tile_max = fmaxf(tile_max, v);
+    }
+  tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, WAVE));
+  tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, WAVE));
+  const float m_new = fmaxf(st.m, tile_max);
+  const float m_safe = m_new == -INFINITY ? 0.f : m_new;   // a row that has seen no key yet stays empty
+  const float alpha = expf(st.m - m_safe);                  // exp(-inf) = 0 for such a row
+  float sum = 0.f;
+#pragma unroll
+  for (int t = 0; t < 4; ++t)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float p = expf(s[t][i] - m_safe);
+      s[t][i] = p;
+      sum += p;
+    }
+  sum += __shfl_xor(sum, 16, WAVE);
+  sum += __shfl_xor(sum, 32, WAVE);
+  st.l = st.l * alpha + sum;
+  st.m = m_new;
+  bf16x8 p[2];
+#pragma unroll
+  for (int h = 0; h < 2; ++h)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      p[h][i] = to_bf16(s[2 * h][i]);
+      p[h][4 + i] = to_bf16(s[2 * h + 1][i]);
+    }
+#pragma unroll
+  for (int dt = 0; dt < 2 * KB; ++dt) {
+    if (16 * dt >= head_dim) break;
+    st.o[dt] *= alpha;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const bf16_t* vp = v_page + (16 * dt + c) * PAGE_TOKENS + 32 * h + 4 * g;
+      const bf16x4 v0 = *(const bf16x4*)vp;
+      const bf16x4 v1 = *(const bf16x4*)(vp + 16);
+      bf16x8 a;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        a[i] = v0[i];
+        a[4 + i] = v1[i];
+      }
+      st.o[dt] = MFMA16(a, p[h], st.o[dt]);
+    }
+  }
+}
+
+template <int KB>
+__device__ __forceinline__ void init_rows(RowBlock<KB>& st, const bf16_t* q_row, bool row_valid, int head_dim) {
+  const int g = (threadIdx.x % WAVE) / 16;
+#pragma unroll
+  for (int kb = 0; kb < KB; ++kb) {
+    const int d = 32 * kb + 8 * g;
+    st.q[kb] = (row_valid && d < head_dim) ? load8(q_row + d) : zero8();
+  }
+#pragma unroll
+  for (int dt = 0; dt < 2 * KB; ++dt) st.o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  st.m = -INFINITY;
+  st.l = 0.f;
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Many rows per sequence. Grid: (64-row query tiles, query heads); 4 waves of 16 rows each.
+template <int KB>
+__global__ __launch_bounds__(256) void attn_causal_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
+    const int* __restrict__ page_table, int max_pages, const int* __restrict__ seq_slot,
+    const int* __restrict__ cu_rows, const int* __restrict__ tile_cu, const int* __restrict__ seq_start, int n_seqs,
+    bf16_t* __restrict__ out, int n_heads, int n_kv, int head_dim, float scale, int window) {
+  const int tile = blockIdx.x, head = blockIdx.y;
+  if (tile >= tile_cu[n_seqs]) return;
+  int lo = 0, hi = n_seqs;  // the sequence whose tiles include `tile`
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (tile_cu[mid] <= tile) lo = mid; else hi = mid;
+  }
+  while (lo + 1 < n_seqs && tile_cu[lo + 1] <= tile) ++lo;
+  const int seq = lo, slot = seq_slot[seq];
+  if (slot < 0) return;
+  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE, c = lane % 16, g = lane / 16;
+  const int q_len = cu_rows[seq + 1] - cu_rows[seq];
+  const int first = (tile - tile_cu[seq]) * 64 + 16 * wave;   // first of the wave's rows within the sequence
+  if (first >= q_len) return;
+  const int rows = min(16, q_len - first);
+  const bool row_valid = c < rows;
+  const int64_t row = (int64_t)cu_rows[seq] + first + c;
+  const int kvh = head / (n_heads / n_kv);
+  RowBlock<KB> st;
+  init_rows<KB>(st, q + (row * n_heads + head) * head_dim, row_valid, head_dim);
+  const int pos0 = seq_start[seq] + first;                    // position of the wave's first row
+  const int pos_row = row_valid ? pos0 + c : -1;              // an absent row sees nothing
+  const int lo_row = window > 0 ? max(0, pos_row - window + 1) : 0;
+  const int lo_wave = window > 0 ? max(0, pos0 - window + 1) : 0;
+  const int hi_wave = pos0 + rows - 1;
+  for (int pg = lo_wave / PAGE_TOKENS; pg <= hi_wave / PAGE_TOKENS; ++pg) {
+    const int page = page_table[(int64_t)slot * max_pages + pg];
+    if (page < 0) continue;
+    const int64_t base = ((int64_t)page * n_kv + kvh) * PAGE_TOKENS * head_dim;
+    attend_page<KB>(st, k_pages + base, v_pages + base, head_dim, scale, pg * PAGE_TOKENS, lo_row, pos_row);
+  }
+  if (!row_valid) return;
+  const float inv = 1.f / st.l;
+  bf16_t* o = out + (row * n_heads + head) * head_dim;
+#pragma unroll
+  for (int dt = 0; dt < 2 * KB; ++dt) {
+    if (16 * dt >= head_dim) break;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o[16 * dt + 4 * g + i] = float_to_bf16(st.o[dt][i] * inv);
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------
+// One row per sequence. Grid: (sequences, kv heads * head blocks, splits); one wave each. The wave's 16
+// "rows" are up to 16 query heads that share the kv head. Each split writes an unnormalised partial
+// (o, m, l); the combine kernel merges them in a fixed order, so results do not depend on timing.
+template <int KB>
+__global__ __launch_bounds__(64) void attn_split_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
+    const int* __restrict__ page_table, int max_pages, const int* __restrict__ seq_slot,
+    const int* __restrict__ cu_rows, const int* __restrict__ kv_len, float* __restrict__ part_o,
+    float* __restrict__ part_ml, int n_heads, int n_kv, int head_dim, float scale, int window, int n_splits) {
+  const int seq = blockIdx.x, split = blockIdx.z;
+  const int group = n_heads / n_kv, blocks = (group + 15) / 16;
+  const int kvh = blockIdx.y / blocks, hb = blockIdx.y % blocks;
+  const int lane = threadIdx.x, c = lane % 16, g = lane / 16;
+  const int slot = seq_slot[seq];
+  const int head = kvh * group + hb * 16 + c;
+  const bool row_valid = hb * 16 + c < group;
+  const int64_t row = cu_rows[seq];
+  float* po = part_o + (((int64_t)seq * n_heads + head) * n_splits + split) * head_dim;
+  float* pml = part_ml + (((int64_t)seq * n_heads + head) * n_splits + split) * 2;
+  RowBlock<KB> st;
+  init_rows<KB>(st, q + (row * n_heads + head) * head_dim, row_valid && slot >= 0, head_dim);
+  if (slot >= 0) {
+    const int pos = kv_len[seq] - 1;                           // the row's own position; its key is cached
+    const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+    const int pg_lo = lo / PAGE_TOKENS, pg_hi = pos / PAGE_TOKENS;
+    const int per = (pg_hi - pg_lo + n_splits) / n_splits;     // ceil(pages / splits)
+    const int pg0 = pg_lo + split * per, pg1 = min(pg_hi, pg0 + per - 1);
+    for (int pg = pg0; pg <= pg1; ++pg) {
+      const int page = page_table[(int64_t)slot * max_pages + pg];
+      if (page < 0) continue;
+      const int64_t base = ((int64_t)page * n_kv + kvh) * PAGE_TOKENS * head_dim;
+      attend_page<KB>(st, k_pages + base, v_pages + base, head_dim, scale, pg * PAGE_TOKENS, lo, pos);
+    }
+  }
+  if (!row_valid) return;
+#pragma unroll
+  for (int dt = 0; dt < 2 * KB; ++dt) {
+    if (16 * dt >= head_dim) break;
+    *(f32x4*)(po + 16 * dt + 4 * g) = st.o[dt];
+  }
+  if (g == 0) {
+    pml[0] = st.m;
+    pml[1] = st.l;
+  }
+}
+
+// out[seq_row, head, :] = sum_s w_s o_s / sum_s w_s l_s,  w_s = exp(m_s - max m)  (attn_decode.py:102-118)
+__global__ void attn_combine_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                    const int* __restrict__ seq_slot, const int* __restrict__ cu_rows,
+                                    bf16_t* __restrict__ out, int n_heads, int head_dim, int n_splits) {
+  const int seq = blockIdx.x, head = blockIdx.y;
+  const int64_t row = cu_rows[seq];
+  bf16_t* o = out + (row * n_heads + head) * head_dim;
+  const float* ml = part_ml + ((int64_t)seq * n_heads + head) * n_splits * 2;
+  const float* po = part_o + ((int64_t)seq * n_heads + head) * n_splits * head_dim;
+  const bool live = seq_slot[seq] >= 0;
+  float m = -INFINITY;
+  if (live)
+    for (int s = 0; s < n_splits; ++s) m = fmaxf(m, ml[2 * s]);
+  for (int d = threadIdx.x; d < head_dim; d += blockDim.x) {
+    float num = 0.f, den = 0.f;
+    if (live && m != -INFINITY)
+      for (int s = 0; s < n_splits; ++s) {
+        const float ms = ml[2 * s];
+        if (ms == -INFINITY) continue;   // a split that saw no key
+        const float w = expf(ms - m);
+        num += w * po[s * head_dim + d];
+        den += w * ml[2 * s + 1];
+      }
+    o[d] = float_to_bf16(den > 0.f ? num / den : 0.f);
+  }
+}
+
+#define DISPATCH_KB(KBV, CALL)                                                      \
+  switch (KBV) {                                                                    \
+    case 1: { constexpr int KB = 1; CALL; } break;                                  \
+    case 2: { constexpr int KB = 2; CALL; } break;                                  \
+    case 3: { constexpr int KB = 3; CALL; } break;                                  \
+    case 4: { constexpr int KB = 4; CALL; } break;                                  \
+    case 5: { constexpr int KB = 5; CALL; } break;                                  \
+    case 6: { constexpr int KB = 6; CALL; } break;                                  \
+    case 7: { constexpr int KB = 7; CALL; } break;                                  \
+    case 8: { constexpr int KB = 8; CALL; } break;                                  \
+    default: return -1;                                                             \
+  }
+
+static int head_shape_ok(int n_heads, int n_kv, int head_dim) {
+  return head_dim > 0 && head_dim % 16 == 0 && head_dim <= 256 && n_kv > 0 && n_heads % n_kv == 0;
+}
+
+DRYFT_API int dryft_attn_causal_bf16(const void* q, const void* k_pages, const void* v_pages, const int* page_table,
+                                     int max_pages, const int* seq_slot, const int* cu_rows, const int* tile_cu,
+                                     const int* seq_start, int n_seqs, int max_tiles, void* out, int n_heads,
+                                     int n_kv, int head_dim, float scale, int window, hipStream_t stream) {
+  if (n_seqs <= 0 || max_tiles <= 0) return 0;
+  if (!head_shape_ok(n_heads, n_kv, head_dim)) return -1;
+  dim3 grid(max_tiles, n_heads), block(256);
+  DISPATCH_KB((head_dim + 31) / 32,
+              hipLaunchKernelGGL(attn_causal_kernel<KB>, grid, block, 0, stream, (const bf16_t*)q,
+                                 (const bf16_t*)k_pages, (const bf16_t*)v_pages, page_table, max_pages, seq_slot,
+                                 cu_rows, tile_cu, seq_start, n_seqs, (bf16_t*)out, n_heads, n_kv, head_dim, scale,
+                                 window));
+  return DRYFT_LAUNCH_CHECK();
+}
+
+DRYFT_API int dryft_attn_split_bf16(const void* q, const void* k_pages, const void* v_pages, const int* page_table,
+                                    int max_pages, const int* seq_slot, const int* cu_rows, const int* kv_len,
+                                    int n_seqs, float* part_o, float* part_ml, int n_splits, void* out, int n_heads,
+                                    int n_kv, int head_dim, float scale, int window, hipStream_t stream) {
+  if (n_seqs <= 0) return 0;
+  if (!head_shape_ok(n_heads, n_kv, head_dim) || n_splits < 1) return -1;
+  const int group = n_heads / n_kv, blocks = (group + 15) / 16;
+  dim3 grid(n_seqs, n_kv * blocks, n_splits), block(64);
+  DISPATCH_KB((head_dim + 31) / 32,
+              hipLaunchKernelGGL(attn_split_kernel<KB>, grid, block, 0, stream, (const bf16_t*)q,
+                                 (const bf16_t*)k_pages, (const bf16_t*)v_pages, page_table, max_pages, seq_slot,
+                                 cu_rows, kv_len, part_o, part_ml, n_heads, n_kv, head_dim, scale, window, n_splits));
+  int rc = DRYFT_LAUNCH_CHECK();
+  if (rc) return rc;
+  hipLaunchKernelGGL(attn_combine_kernel, dim3(n_seqs, n_heads), dim3(64), 0, stream, part_o, part_ml, seq_slot,
+                     cu_rows, (bf16_t*)out, n_heads, head_dim, n_splits);
+  return DRYFT_LAUNCH_CHECK();
+}

@@ -1,0 +1,56 @@
+// Turns a step's per-sequence facts into per-row facts, on the device, so that
+// a captured decode step can be replayed at any position: everything that
+// varies is read from memory (the reference keeps positions in a device
+// tensor for the same reason, engine/dryft_qwen3/cache.py:8-10).
+#include "common.h"
+
+// One block. Inputs: seq_slot[B] (-1 = not taking part), q_len[B] (new tokens of
+// each sequence), lengths[slots] (cached tokens per slot). Outputs: cu_rows[B+1],
+// tile_cu[B+1] (prefix sums of rows and of 64-row query tiles), kv_len[B] (cached
+// tokens after this step), row_seq/row_slot/row_pos[n_rows]. Advances lengths.
+__global__ void prepare_batch_kernel(const int* __restrict__ seq_slot, const int* __restrict__ q_len,
+                                     int* __restrict__ lengths, int n_seqs, int n_rows,
+                                     int* __restrict__ cu_rows, int* __restrict__ tile_cu,
+                                     int* __restrict__ kv_len, int* __restrict__ seq_start,
+                                     int* __restrict__ row_seq, int* __restrict__ row_slot,
+                                     int* __restrict__ row_pos) {
+  if (threadIdx.x == 0) {
+    int rows = 0, tiles = 0;
+    for (int s = 0; s < n_seqs; ++s) {
+      cu_rows[s] = rows;
+      tile_cu[s] = tiles;
+      const int slot = seq_slot[s];
+      const int q = slot >= 0 ? q_len[s] : 0;
+      const int past = slot >= 0 ? lengths[slot] : 0;
+      seq_start[s] = past;
+      kv_len[s] = past + q;
+      rows += q_len[s];                         // rows of a sequence that sits out still occupy their places
+      tiles += (q + 63) / 64;
+      if (slot >= 0) lengths[slot] = past + q;
+    }
+    cu_rows[n_seqs] = rows;
+    tile_cu[n_seqs] = tiles;
+  }
+  __syncthreads();
+  for (int r = threadIdx.x; r < n_rows; r += blockDim.x) {
+    int lo = 0, hi = n_seqs;                      // last s with cu_rows[s] <= r
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) >> 1;
+      if (cu_rows[mid] <= r) lo = mid; else hi = mid;
+    }
+    // skip over empty sequences that share the same start
+    while (lo + 1 < n_seqs && cu_rows[lo + 1] <= r) ++lo;
+    const int slot = (r < cu_rows[n_seqs]) ? seq_slot[lo] : -1;
+    row_seq[r] = lo;
+    row_slot[r] = slot;
+    row_pos[r] = slot >= 0 ? seq_start[lo] + (r - cu_rows[lo]) : 0;
+  }
+}
+
+DRYFT_API int dryft_prepare_batch(const int* seq_slot, const int* q_len, int* lengths, int n_seqs, int n_rows,
+                                  int* cu_rows, int* tile_cu, int* kv_len, int* seq_start, int* row_seq,
+                                  int* row_slot, int* row_pos, hipStream_t stream) {
+  hipLaunchKernelGGL(prepare_batch_kernel, dim3(1), dim3(256), 0, stream, seq_slot, q_len, lengths, n_seqs, n_rows,
+                     cu_rows, tile_cu, kv_len, seq_start, row_seq, row_slot, row_pos);
+  return DRYFT_LAUNCH_CHECK();
+}

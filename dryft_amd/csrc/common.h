@@ -1,0 +1,91 @@
+// Shared device helpers for the gfx950 kernels: storage types, exact
+// float <-> bfloat16 conversion, wave and block reductions.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#define DRYFT_API extern "C" __attribute__((visibility("default")))
+#define WAVE 64
+#define PAGE_TOKENS 64
+
+// bfloat16 kept as its 16 bits; arithmetic is always done in float.
+struct bf16_t {
+  uint16_t bits;
+};
+
+__device__ __forceinline__ float bf16_to_float(bf16_t v) { return __uint_as_float(((uint32_t)v.bits) << 16); }
+
+// round to nearest, ties to even; NaN stays NaN
+__device__ __forceinline__ bf16_t float_to_bf16(float f) {
+  uint32_t u = __float_as_uint(f);
+  bf16_t r;
+  if ((u & 0x7fffffffu) > 0x7f800000u) {
+    r.bits = (uint16_t)((u >> 16) | 0x0040u);
+  } else {
+    u += 0x7fffu + ((u >> 16) & 1u);
+    r.bits = (uint16_t)(u >> 16);
+  }
+  return r;
+}
+
+template <typename T> __device__ __forceinline__ float load_as_float(const T* p);
+template <> __device__ __forceinline__ float load_as_float<float>(const float* p) { return *p; }
+template <> __device__ __forceinline__ float load_as_float<bf16_t>(const bf16_t* p) { return bf16_to_float(*p); }
+
+template <typename T> __device__ __forceinline__ void store_from_float(T* p, float v);
+template <> __device__ __forceinline__ void store_from_float<float>(float* p, float v) { *p = v; }
+template <> __device__ __forceinline__ void store_from_float<bf16_t>(bf16_t* p, float v) { *p = float_to_bf16(v); }
+
+// The value a float takes when it is stored as T and read back: the rounding
+// boundaries of the bfloat16 path; the identity in the float32 path.
+template <typename T> __device__ __forceinline__ float rounded_as(float v);
+template <> __device__ __forceinline__ float rounded_as<float>(float v) { return v; }
+template <> __device__ __forceinline__ float rounded_as<bf16_t>(float v) { return bf16_to_float(float_to_bf16(v)); }
+
+// A vector whose dtype is only known at run time (norm weights: bfloat16, or float32 if stored so).
+__device__ __forceinline__ float load_vector(const void* p, int i, int is_f32) {
+  return is_f32 ? ((const float*)p)[i] : bf16_to_float(((const bf16_t*)p)[i]);
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = WAVE / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
+  return v;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = WAVE / 2; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, WAVE));
+  return v;
+}
+
+// Sum over a block of up to 1024 threads; every thread gets the result.
+// `scratch` holds at least 16 floats of LDS; the call synchronises the block.
+__device__ __forceinline__ float block_sum(float v, float* scratch) {
+  v = wave_sum(v);
+  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE, waves = (blockDim.x + WAVE - 1) / WAVE;
+  __syncthreads();
+  if (lane == 0) scratch[wave] = v;
+  __syncthreads();
+  float t = 0.f;
+  for (int w = 0; w < waves; ++w) t += scratch[w];
+  return t;
+}
+
+__device__ __forceinline__ float block_max(float v, float* scratch) {
+  v = wave_max(v);
+  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE, waves = (blockDim.x + WAVE - 1) / WAVE;
+  __syncthreads();
+  if (lane == 0) scratch[wave] = v;
+  __syncthreads();
+  float t = scratch[0];
+  for (int w = 1; w < waves; ++w) t = fmaxf(t, scratch[w]);
+  return t;
+}
+
+// Where position `pos` of the sequence in `slot` lives: index of its page, or -1.
+__device__ __forceinline__ int page_of(const int* page_table, int max_pages, int slot, int pos) {
+  return page_table[(int64_t)slot * max_pages + pos / PAGE_TOKENS];
+}
+
+#define DRYFT_LAUNCH_CHECK() (int)hipGetLastError()

@@ -1,0 +1,240 @@
+// Matrix products y[M,N] = x[M,K] . W[N,K]^T (weights in their checkpoint layout [out, in], no bias;
+// reference: F.linear at engine/dryft_qwen3/model.py:153, 179-180, 237, 258-261).
+//
+//  * gemm_tiled:  any M, N, K, float accumulation by plain fused multiply-adds. With float inputs it
+//    is the true 32-bit product (no reduced-precision matrix mode); with bfloat16 inputs it takes the
+//    sizes the matrix-core kernel refuses.
+//  * gemm_skinny: bfloat16, M <= 64 rows (decoding, output head): every weight is read once, from
+//    global memory straight into the A operand of v_mfma_f32_16x16x32_bf16; the four waves of a
+//    workgroup split K, and further workgroups may split K again into float partial sums that the
+//    consumer adds in a fixed order.
+#include "common.h"
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+// ------------------------------------------------------------------------------------------ tiled
+#define TILE 64
+#define TILE_K 16
+
+template <typename T, typename O>
+__global__ __launch_bounds__(256) void gemm_tiled_kernel(const T* __restrict__ x, int64_t x_stride,
+                                                         const T* __restrict__ w, O* __restrict__ y, int M, int N,
+                                                         int K) {
+  __shared__ float xs[TILE_K][TILE + 1];
+  __shared__ float ws[TILE_K][TILE + 1];
+  const int tid = threadIdx.x, tx = tid % 16, ty = tid / 16;
+  const int m0 = blockIdx.y * TILE, n0 = blockIdx.x * TILE;
+  float acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+  const int lr = tid / 4, lk = (tid % 4) * 4;   // this thread stages row lr, k lk..lk+3 of both tiles
+  for (int k0 = 0; k0 < K; k0 += TILE_K) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int k = k0 + lk + i;
+      const int m = m0 + lr, n = n0 + lr;
+      xs[lk + i][lr] = (m < M && k < K) ? load_as_float(x + (int64_t)m * x_stride + k) : 0.f;
+      ws[lk + i][lr] = (n < N && k < K) ? load_as_float(w + (int64_t)n * K + k) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < TILE_K; ++k) {
+      float a[4], b[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) a[i] = xs[k][ty * 4 + i];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) b[j] = ws[k][tx * 4 + j];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int m = m0 + ty * 4 + i;
+    if (m >= M) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int n = n0 + tx * 4 + j;
+      if (n < N) store_from_float(y + (int64_t)m * N + n, acc[i][j]);
+    }
+  }
+}
+
+// out_f32: the result is stored as float whatever the inputs are (logits)
+DRYFT_API int dryft_gemm_tiled(const void* x, int64_t x_stride, const void* w, void* y, int M, int N, int K,
+                               int is_f32, int out_f32, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (K <= 0) return -1;
+  dim3 grid((N + TILE - 1) / TILE, (M + TILE - 1) / TILE), block(256);
+  if (grid.y > 65535) return -1;
+  if (is_f32)
+    hipLaunchKernelGGL((gemm_tiled_kernel<float, float>), grid, block, 0, stream, (const float*)x, x_stride,
+                       (const float*)w, (float*)y, M, N, K);
+  else if (out_f32)
+    hipLaunchKernelGGL((gemm_tiled_kernel<bf16_t, float>), grid, block, 0, stream, (const bf16_t*)x, x_stride,
+                       (const bf16_t*)w, (float*)y, M, N, K);
+  else
+    hipLaunchKernelGGL((gemm_tiled_kernel<bf16_t, bf16_t>), grid, block, 0, stream, (const bf16_t*)x, x_stride,
+                       (const bf16_t*)w, (bf16_t*)y, M, N, K);
+  return DRYFT_LAUNCH_CHECK();
+}
+
+// ----------------------------------------------------------------------------------------- skinny
+__device__ __forceinline__ bf16x8 zero8g() {
+  bf16x8 z;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) z[i] = (__bf16)0.f;
+  return z;
+}
+
+// A wave computes C^T[n, m] = W[n, :] . x[m, :] for NTW tiles of 16 weight rows and MT tiles of 16
+// activation rows, over its share of K. Per 64 values of K a lane reads 32 contiguous bytes of its
+// weight row (4 lanes cover one 128-byte line) and the same 32 bytes' worth of its activation row; the
+// two halves feed two 32-deep products. Both operands use the same order of K, so the order itself
+// does not matter.
+template <int MT, int NTW, typename O>
+__global__ __launch_bounds__(256) void gemm_skinny_kernel(const bf16_t* __restrict__ x, int64_t x_stride,
+                                                          const bf16_t* __restrict__ w, O* __restrict__ y,
+                                                          float* __restrict__ partials, int M, int N, int K) {
+  __shared__ f32x4 red[4][MT * NTW][WAVE];
+  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE, c = lane % 16, g = lane / 16;
+  const int n0 = blockIdx.x * 16 * NTW;
+  const int splits = gridDim.y, units = splits * 4, unit = blockIdx.y * 4 + wave;
+  const int kblocks = (K + 63) / 64, per = (kblocks + units - 1) / units;
+  const int kb0 = unit * per, kb1 = min(kblocks, kb0 + per);
+  f32x4 acc[NTW][MT];
+#pragma unroll
+  for (int nt = 0; nt < NTW; ++nt)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[nt][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const bf16_t* wp[NTW];
+  bool w_ok[NTW];
+#pragma unroll
+  for (int nt = 0; nt < NTW; ++nt) {
+    const int n = n0 + 16 * nt + c;
+    w_ok[nt] = n < N;
+    wp[nt] = w + (int64_t)(w_ok[nt] ? n : 0) * K;
+  }
+  const bf16_t* xp[MT];
+  bool x_ok[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int m = 16 * mt + c;
+    x_ok[mt] = m < M;
+    xp[mt] = x + (int64_t)(x_ok[mt] ? m : 0) * x_stride;
+  }
+  for (int kb = kb0; kb < kb1; ++kb) {
+    const int k = kb * 64 + 16 * g;
+    const bool k0_ok = k < K, k1_ok = k + 8 < K;
+    bf16x8 a[NTW][2], b[MT][2];
+#pragma unroll
+    for (int nt = 0; nt < NTW; ++nt) {
+      a[nt][0] = (w_ok[nt] && k0_ok) ? *(const bf16x8*)(wp[nt] + k) : zero8g();
+      a[nt][1] = (w_ok[nt] && k1_ok) ? *(const bf16x8*)(wp[nt] + k + 8) : zero8g();
+    }
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      b[mt][0] = (x_ok[mt] && k0_ok) ? *(const bf16x8*)(xp[mt] + k) : zero8g();
+      b[mt][1] = (x_ok[mt] && k1_ok) ? *(const bf16x8*)(xp[mt] + k + 8) : zero8g();
+    }
+#pragma unroll
+    for (int nt = 0; nt < NTW; ++nt)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[nt][0], b[mt][0], acc[nt][mt], 0, 0, 0);
+        acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[nt][1], b[mt][1], acc[nt][mt], 0, 0, 0);
+      }
+  }
+#pragma unroll
+  for (int nt = 0; nt < NTW; ++nt)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) red[wave][nt * MT + mt][lane] = acc[nt][mt];
+  __syncthreads();
+  // tile t is summed (waves in order 0..3) and stored by wave t % 4
+#pragma unroll
+  for (int t = 0; t < MT * NTW; ++t) {
+    if (t % 4 != wave) continue;
+    f32x4 s = red[0][t][lane];
+    s += red[1][t][lane];
+    s += red[2][t][lane];
+    s += red[3][t][lane];
+    const int nt = t / MT, mt = t % MT;
+    const int m = 16 * mt + c;
+    if (m >= M) continue;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int n = n0 + 16 * nt + 4 * g + i;
+      if (n >= N) continue;
+      if (splits > 1)
+        partials[((int64_t)blockIdx.y * M + m) * N + n] = s[i];
+      else
+        store_from_float(y + (int64_t)m * N + n, s[i]);
+    }
+  }
+}
+
+template <int MT, int NTW>
+static int launch_skinny(const void* x, int64_t x_stride, const void* w, void* y, float* partials, int M, int N, int K,
+                         int splits, int out_f32, hipStream_t stream) {
+  dim3 grid((N + 16 * NTW - 1) / (16 * NTW), splits), block(256);
+  if (out_f32)
+    hipLaunchKernelGGL((gemm_skinny_kernel<MT, NTW, float>), grid, block, 0, stream, (const bf16_t*)x, x_stride,
+                       (const bf16_t*)w, (float*)y, partials, M, N, K);
+  else
+    hipLaunchKernelGGL((gemm_skinny_kernel<MT, NTW, bf16_t>), grid, block, 0, stream, (const bf16_t*)x, x_stride,
+                       (const bf16_t*)w, (bf16_t*)y, partials, M, N, K);
+  return DRYFT_LAUNCH_CHECK();
+}
+
+// splits > 1: float partial sums go to partials[splits, M, N] and y is not written.
+DRYFT_API int dryft_gemm_skinny_bf16(const void* x, int64_t x_stride, const void* w, void* y, float* partials, int M,
+                                     int N, int K, int ntw, int splits, int out_f32, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (M > 64 || K <= 0 || K % 8 || x_stride % 8 || splits < 1 || splits > 64) return -1;
+  if (splits > 1 && partials == nullptr) return -1;
+  const int mt = (M + 15) / 16;
+#define SK(MTV, NTWV) return launch_skinny<MTV, NTWV>(x, x_stride, w, y, partials, M, N, K, splits, out_f32, stream)
+  switch (mt * 10 + ntw) {
+    case 11: SK(1, 1);
+    case 12: SK(1, 2);
+    case 14: SK(1, 4);
+    case 21: SK(2, 1);
+    case 22: SK(2, 2);
+    case 24: SK(2, 4);
+    case 31: SK(3, 1);
+    case 32: SK(3, 2);
+    case 34: SK(3, 4);
+    case 41: SK(4, 1);
+    case 42: SK(4, 2);
+    case 44: SK(4, 4);
+    default: return -1;
+  }
+#undef SK
+}
+
+// y = T(sum_s partials[s]) in the order s = 0, 1, ...
+template <typename O>
+__global__ void sum_partials_kernel(const float* __restrict__ partials, O* __restrict__ y, int64_t n, int splits) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  float s = 0.f;
+  for (int p = 0; p < splits; ++p) s += partials[p * n + i];
+  store_from_float(y + i, s);
+}
+
+DRYFT_API int dryft_sum_partials(const float* partials, void* y, int64_t n, int splits, int out_f32,
+                                 hipStream_t stream) {
+  if (n <= 0) return 0;
+  dim3 grid((unsigned)((n + 255) / 256)), block(256);
+  if (out_f32)
+    hipLaunchKernelGGL(sum_partials_kernel<float>, grid, block, 0, stream, partials, (float*)y, n, splits);
+  else
+    hipLaunchKernelGGL(sum_partials_kernel<bf16_t>, grid, block, 0, stream, partials, (bf16_t*)y, n, splits);
+  return DRYFT_LAUNCH_CHECK();
+}

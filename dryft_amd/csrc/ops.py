@@ -1,0 +1,354 @@
+"""Python faces of the HIP kernels: argument checks, then one ctypes call each.
+
+Every function checks on the host that the operands have the dtypes, shapes and
+strides its kernel assumes, and raises rather than launch a kernel that would read
+outside its operands. Kernels run on torch's current stream, so they can be
+recorded into a graph like any other work on it. There is no CPU path: tensors
+must live on the GPU, and a missing library is compiled or the call fails.
+"""
+
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_float, c_int, c_int64, c_void_p
+
+import torch
+
+from . import build
+
+_P, _I, _L, _F = c_void_p, c_int, c_int64, c_float
+_SIGNATURES = {
+    "batch": {"dryft_prepare_batch": [_P, _P, _P, _I, _I, _P, _P, _P, _P, _P, _P, _P, _P]},
+    "embed": {"dryft_embed_rows": [_P, _P, _P, _I, _I, _I, _I, _P]},
+    "norm": {"dryft_add_rmsnorm": [_P, _P, _I, _I, _L, _P, _I, _P, _P, _I, _I, _F, _I, _P],
+             "dryft_add_rows": [_P, _P, _P, _L, _I, _P]},
+    "activation": {"dryft_silu_mul": [_P, _P, _I, _I, _L, _I, _P]},
+    "rope_kv": {"dryft_qk_norm_rope_kv": [_P, _L, _P, _P, _I, _I, _F, _P, _P, _I, _P, _P, _P, _P, _P, _P, _I, _I,
+                                          _I, _I, _I, _I, _I, _P]},
+    "attn_rows": {"dryft_attn_rows": [_P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _F, _I, _I, _P]},
+    "attn_mfma": {"dryft_attn_causal_bf16": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _P, _I, _I, _I, _F, _I, _P],
+                  "dryft_attn_split_bf16": [_P, _P, _P, _P, _I, _P, _P, _P, _I, _P, _P, _I, _P, _I, _I, _I, _F, _I,
+                                            _P]},
+    "gemm": {"dryft_gemm_tiled": [_P, _L, _P, _P, _I, _I, _I, _I, _I, _P],
+             "dryft_gemm_skinny_bf16": [_P, _L, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
+             "dryft_sum_partials": [_P, _P, _L, _I, _I, _P]},
+    "sampling": {"dryft_argmax_rows": [_P, _I, _I, _L, _P, _P],
+                 "dryft_sample_rows": [_P, _I, _I, _L, _F, _P, _P, _P]},
+}
+_functions: dict[str, object] = {}
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def _fn(module: str, name: str):
+    f = _functions.get(name)
+    if f is None:
+        lib = build.load(module)
+        f = getattr(lib, name)
+        f.argtypes = _SIGNATURES[module][name]
+        f.restype = c_int
+        _functions[name] = f
+    return f
+
+
+def preload(modules) -> None:
+    build.ensure(list(modules))
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _check(rc: int, what: str) -> None:
+    if rc == -1:
+        raise KernelError(f"{what}: the kernel refuses these sizes")
+    if rc != 0:
+        raise KernelError(f"{what}: launch failed with HIP error {rc}")
+
+
+def _require(cond: bool, msg: str) -> None:
+    if not cond:
+        raise KernelError(msg)
+
+
+def _gpu(t: torch.Tensor, name: str, dtype=None) -> None:
+    _require(isinstance(t, torch.Tensor) and t.is_cuda, f"{name}: must be a GPU tensor (there is no CPU path)")
+    if dtype is not None:
+        _require(t.dtype == dtype, f"{name}: expected {dtype}, got {t.dtype}")
+
+
+def _float_flag(t: torch.Tensor, name: str) -> int:
+    _require(t.dtype in (torch.float32, torch.bfloat16), f"{name}: expected float32 or bfloat16, got {t.dtype}")
+    return 1 if t.dtype == torch.float32 else 0
+
+
+def _ptr(t) -> int:
+    return 0 if t is None else t.data_ptr()
+
+
+# ------------------------------------------------------------------------------------------- batch
+def prepare_batch(seq_slot, q_len, lengths, n_seqs: int, n_rows: int, cu_rows, tile_cu, kv_len, seq_start,
+                  row_seq, row_slot, row_pos) -> None:
+    for name, t, n in (("seq_slot", seq_slot, n_seqs), ("q_len", q_len, n_seqs), ("cu_rows", cu_rows, n_seqs + 1),
+                       ("tile_cu", tile_cu, n_seqs + 1), ("kv_len", kv_len, n_seqs), ("seq_start", seq_start, n_seqs),
+                       ("row_seq", row_seq, n_rows), ("row_slot", row_slot, n_rows), ("row_pos", row_pos, n_rows),
+                       ("lengths", lengths, 1)):
+        _gpu(t, name, torch.int32)
+        _require(t.is_contiguous() and t.numel() >= n, f"{name}: needs {n} contiguous entries, has {t.numel()}")
+    _check(_fn("batch", "dryft_prepare_batch")(
+        _ptr(seq_slot), _ptr(q_len), _ptr(lengths), n_seqs, n_rows, _ptr(cu_rows), _ptr(tile_cu), _ptr(kv_len),
+        _ptr(seq_start), _ptr(row_seq), _ptr(row_slot), _ptr(row_pos), _stream()), "prepare_batch")
+
+
+# ------------------------------------------------------------------------------------------- embed
+def embed_rows(tokens: torch.Tensor, table: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    _gpu(tokens, "tokens", torch.int32)
+    _gpu(table, "table")
+    _gpu(out, "out", table.dtype)
+    n, (vocab, hidden) = tokens.numel(), table.shape
+    _require(table.is_contiguous() and out.is_contiguous() and tokens.is_contiguous(), "embed_rows: contiguous operands")
+    _require(out.shape == (n, hidden), f"embed_rows: out is {tuple(out.shape)}, expected {(n, hidden)}")
+    _check(_fn("embed", "dryft_embed_rows")(_ptr(tokens), _ptr(table), _ptr(out), n, hidden, vocab,
+                                            _float_flag(table, "table"), _stream()), "embed_rows")
+    return out
+
+
+# -------------------------------------------------------------------------------------------- norm
+def add_rmsnorm(res: torch.Tensor, delta, weight: torch.Tensor, eps: float, res_out, y: torch.Tensor,
+                n_partials: int = 1) -> None:
+    """``res_out = res + delta`` (when ``delta`` is given) and ``y = rmsnorm(res_out) * weight``.
+
+    ``delta`` is ``[rows, width]`` in the dtype of ``res``, or ``[n_partials, rows, width]`` float32
+    partial sums. Without ``delta`` nothing is added and ``res_out`` is ignored.
+    """
+    _gpu(res, "res")
+    rows, width = res.shape
+    is_f32 = _float_flag(res, "res")
+    _gpu(weight, "weight")
+    w_f32 = _float_flag(weight, "weight")
+    _require(weight.shape == (width,) and weight.is_contiguous(), f"add_rmsnorm: weight must be [{width}]")
+    _gpu(y, "y", res.dtype)
+    _require(res.is_contiguous() and y.is_contiguous() and y.shape == res.shape, "add_rmsnorm: res and y contiguous, same shape")
+    kind, stride = 0, 0
+    if delta is not None:
+        _gpu(delta, "delta")
+        _gpu(res_out, "res_out", res.dtype)
+        _require(res_out.shape == res.shape and res_out.is_contiguous(), "add_rmsnorm: res_out like res")
+        _require(delta.is_contiguous(), "add_rmsnorm: delta contiguous")
+        if delta.dim() == 3:
+            _require(delta.dtype == torch.float32 and delta.shape[1:] == res.shape and delta.shape[0] >= n_partials,
+                     "add_rmsnorm: partial sums must be float32 [n, rows, width]")
+            kind, stride = 2, rows * width
+        else:
+            _require(delta.dtype == res.dtype and delta.shape == res.shape, "add_rmsnorm: delta like res")
+            kind, n_partials, stride = 1, 1, rows * width
+    else:
+        n_partials = 0
+    _check(_fn("norm", "dryft_add_rmsnorm")(_ptr(res), _ptr(delta), kind, n_partials, stride, _ptr(weight), w_f32,
+                                            _ptr(res_out), _ptr(y), rows, width, float(eps), is_f32, _stream()),
+           "add_rmsnorm")
+
+
+def add_rows(a: torch.Tensor, b: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    _gpu(a, "a")
+    _gpu(b, "b", a.dtype)
+    _gpu(out, "out", a.dtype)
+    _require(a.shape == b.shape == out.shape and a.is_contiguous() and b.is_contiguous() and out.is_contiguous(),
+             "add_rows: contiguous operands of one shape")
+    _check(_fn("norm", "dryft_add_rows")(_ptr(a), _ptr(b), _ptr(out), a.numel(), _float_flag(a, "a"), _stream()),
+           "add_rows")
+    return out
+
+
+# -------------------------------------------------------------------------------------- activation
+def silu_mul(gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    _gpu(gate_up, "gate_up")
+    _gpu(out, "out", gate_up.dtype)
+    rows, two_i = gate_up.shape
+    _require(two_i % 2 == 0 and out.shape == (rows, two_i // 2), "silu_mul: out must be [rows, width / 2]")
+    _require(gate_up.stride(1) == 1 and out.is_contiguous(), "silu_mul: unit stride along the width")
+    _check(_fn("activation", "dryft_silu_mul")(_ptr(gate_up), _ptr(out), rows, two_i // 2, gate_up.stride(0),
+                                               _float_flag(gate_up, "gate_up"), _stream()), "silu_mul")
+    return out
+
+
+# ----------------------------------------------------------------------------------------- rope_kv
+def qk_norm_rope_kv(qkv: torch.Tensor, q_weight, k_weight, eps: float, cos, sin, rot: int, row_slot, row_pos,
+                    q_out: torch.Tensor, k_pages, v_pages, page_table, write_kv: bool, n_heads: int, n_kv: int,
+                    head_dim: int) -> None:
+    _gpu(qkv, "qkv")
+    is_f32 = _float_flag(qkv, "qkv")
+    rows = qkv.shape[0]
+    need_cols = (n_heads + (2 * n_kv if write_kv else 0)) * head_dim
+    _require(qkv.dim() == 2 and qkv.stride(1) == 1 and qkv.shape[1] >= need_cols,
+             f"qk_norm_rope_kv: qkv needs {need_cols} columns, has {tuple(qkv.shape)}")
+    has_norm = q_weight is not None
+    w_f32 = 0
+    if has_norm:
+        for name, w in (("q_weight", q_weight), ("k_weight", k_weight)):
+            _gpu(w, name)
+            _require(w.shape == (head_dim,) and w.is_contiguous(), f"{name}: must be [{head_dim}]")
+        _require(q_weight.dtype == k_weight.dtype, "q_weight and k_weight must share a dtype")
+        w_f32 = _float_flag(q_weight, "q_weight")
+    if rot:
+        _require(rot % 2 == 0 and rot <= head_dim, f"rotary width {rot} must be even and at most {head_dim}")
+        for name, t in (("cos", cos), ("sin", sin)):
+            _gpu(t, name, qkv.dtype)
+            _require(t.dim() == 2 and t.shape[1] == rot // 2 and t.is_contiguous(), f"{name}: must be [positions, {rot // 2}]")
+    for name, t in (("row_slot", row_slot), ("row_pos", row_pos)):
+        _gpu(t, name, torch.int32)
+        _require(t.numel() >= rows and t.is_contiguous(), f"{name}: needs {rows} entries")
+    _gpu(q_out, "q_out", qkv.dtype)
+    _require(q_out.is_contiguous() and q_out.numel() == rows * n_heads * head_dim, "q_out: must be [rows, heads, head_dim]")
+    max_pages = 0
+    if write_kv:
+        _check_pages(k_pages, v_pages, page_table, n_kv, head_dim, qkv.dtype)
+        max_pages = page_table.shape[1]
+    _check(_fn("rope_kv", "dryft_qk_norm_rope_kv")(
+        _ptr(qkv), qkv.stride(0), _ptr(q_weight), _ptr(k_weight), w_f32, int(has_norm), float(eps), _ptr(cos),
+        _ptr(sin), int(rot), _ptr(row_slot), _ptr(row_pos), _ptr(q_out), _ptr(k_pages), _ptr(v_pages),
+        _ptr(page_table), max_pages, int(write_kv), rows, n_heads, n_kv, head_dim, is_f32, _stream()),
+        "qk_norm_rope_kv")
+
+
+def _check_pages(k_pages, v_pages, page_table, n_kv: int, head_dim: int, dtype) -> None:
+    for name, t in (("k_pages", k_pages), ("v_pages", v_pages)):
+        _gpu(t, name, dtype)
+        _require(t.dim() == 4 and t.shape[1] == n_kv and t.shape[2] * t.shape[3] == 64 * head_dim and t.is_contiguous(),
+                 f"{name}: must be contiguous [pages, {n_kv}, 64, {head_dim}], got {tuple(t.shape)}")
+    _gpu(page_table, "page_table", torch.int32)
+    _require(page_table.dim() == 2 and page_table.is_contiguous(), "page_table: must be contiguous [slots, pages]")
+
+
+# --------------------------------------------------------------------------------------- attention
+def attn_rows(q, k_pages, v_pages, page_table, row_slot, row_pos, out, n_heads: int, n_kv: int, head_dim: int,
+              scale: float, window: int) -> None:
+    _gpu(q, "q")
+    is_f32 = _float_flag(q, "q")
+    rows = q.numel() // (n_heads * head_dim)
+    _require(q.is_contiguous() and q.numel() == rows * n_heads * head_dim, "attn_rows: q must be [rows, heads, head_dim]")
+    _gpu(out, "out", q.dtype)
+    _require(out.is_contiguous() and out.numel() == q.numel(), "attn_rows: out like q")
+    _check_pages(k_pages, v_pages, page_table, n_kv, head_dim, q.dtype)
+    for name, t in (("row_slot", row_slot), ("row_pos", row_pos)):
+        _gpu(t, name, torch.int32)
+        _require(t.numel() >= rows, f"{name}: needs {rows} entries")
+    _require(n_heads <= 65535, "attn_rows: too many heads")
+    _check(_fn("attn_rows", "dryft_attn_rows")(
+        _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(page_table), page_table.shape[1], _ptr(row_slot), _ptr(row_pos),
+        _ptr(out), rows, n_heads, n_kv, head_dim, float(scale), int(window), is_f32, _stream()), "attn_rows")
+
+
+def attn_causal_bf16(q, k_pages, v_pages, page_table, seq_slot, cu_rows, tile_cu, seq_start, n_seqs: int,
+                     max_tiles: int, out, n_heads: int, n_kv: int, head_dim: int, scale: float, window: int) -> None:
+    _gpu(q, "q", torch.bfloat16)
+    _gpu(out, "out", torch.bfloat16)
+    _require(q.is_contiguous() and out.is_contiguous() and out.numel() == q.numel(), "attn_causal: q and out contiguous")
+    _check_pages(k_pages, v_pages, page_table, n_kv, head_dim, torch.bfloat16)
+    for name, t, n in (("seq_slot", seq_slot, n_seqs), ("cu_rows", cu_rows, n_seqs + 1),
+                       ("tile_cu", tile_cu, n_seqs + 1), ("seq_start", seq_start, n_seqs)):
+        _gpu(t, name, torch.int32)
+        _require(t.numel() >= n, f"{name}: needs {n} entries")
+    _require(n_heads <= 65535, "attn_causal: too many heads")
+    _check(_fn("attn_mfma", "dryft_attn_causal_bf16")(
+        _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(page_table), page_table.shape[1], _ptr(seq_slot), _ptr(cu_rows),
+        _ptr(tile_cu), _ptr(seq_start), n_seqs, max_tiles, _ptr(out), n_heads, n_kv, head_dim, float(scale),
+        int(window), _stream()), "attn_causal_bf16")
+
+
+def attn_split_bf16(q, k_pages, v_pages, page_table, seq_slot, cu_rows, kv_len, n_seqs: int, part_o, part_ml,
+                    n_splits: int, out, n_heads: int, n_kv: int, head_dim: int, scale: float, window: int) -> None:
+    _gpu(q, "q", torch.bfloat16)
+    _gpu(out, "out", torch.bfloat16)
+    _require(q.is_contiguous() and out.is_contiguous() and out.numel() == q.numel(), "attn_split: q and out contiguous")
+    _check_pages(k_pages, v_pages, page_table, n_kv, head_dim, torch.bfloat16)
+    for name, t, n in (("seq_slot", seq_slot, n_seqs), ("cu_rows", cu_rows, n_seqs + 1), ("kv_len", kv_len, n_seqs)):
+        _gpu(t, name, torch.int32)
+        _require(t.numel() >= n, f"{name}: needs {n} entries")
+    _gpu(part_o, "part_o", torch.float32)
+    _gpu(part_ml, "part_ml", torch.float32)
+    _require(part_o.numel() >= n_seqs * n_heads * n_splits * head_dim and part_ml.numel() >= n_seqs * n_heads * n_splits * 2,
+             "attn_split: partial buffers too small")
+    _require(n_splits <= 65535 and n_kv * ((n_heads // n_kv + 15) // 16) <= 65535, "attn_split: grid too large")
+    _check(_fn("attn_mfma", "dryft_attn_split_bf16")(
+        _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(page_table), page_table.shape[1], _ptr(seq_slot), _ptr(cu_rows),
+        _ptr(kv_len), n_seqs, _ptr(part_o), _ptr(part_ml), n_splits, _ptr(out), n_heads, n_kv, head_dim, float(scale),
+        int(window), _stream()), "attn_split_bf16")
+
+
+# -------------------------------------------------------------------------------------------- gemm
+def gemm_tiled(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """``out = x @ w.T`` with float accumulation by plain multiply-adds (any sizes)."""
+    _gpu(x, "x")
+    _gpu(w, "w", x.dtype)
+    is_f32 = _float_flag(x, "x")
+    m, k = x.shape
+    n = w.shape[0]
+    _require(w.shape == (n, k) and w.is_contiguous() and x.stride(1) == 1, "gemm_tiled: x [M,K] row-major, w [N,K] contiguous")
+    _gpu(out, "out")
+    out_f32 = 1 if out.dtype == torch.float32 else 0
+    _require(out.shape == (m, n) and out.is_contiguous() and (out.dtype == x.dtype or out_f32),
+             f"gemm_tiled: out must be [{m},{n}] in the input dtype or float32")
+    for m0 in range(0, m, 65535 * 64):                      # the row tiles ride on grid.y
+        m1 = min(m, m0 + 65535 * 64)
+        _check(_fn("gemm", "dryft_gemm_tiled")(_ptr(x[m0:m1]), x.stride(0), _ptr(w), _ptr(out[m0:m1]), m1 - m0, n, k,
+                                               is_f32, out_f32, _stream()), "gemm_tiled")
+    return out
+
+
+def gemm_skinny_bf16(x, w, out, partials=None, ntw: int = 1, splits: int = 1) -> None:
+    """``x [M<=64, K] @ w[N, K].T``; with ``splits > 1`` the result is left as ``partials[splits, M, N]``."""
+    _gpu(x, "x", torch.bfloat16)
+    _gpu(w, "w", torch.bfloat16)
+    m, k = x.shape
+    n = w.shape[0]
+    _require(w.shape == (n, k) and w.is_contiguous() and x.stride(1) == 1, "gemm_skinny: x [M,K] row-major, w [N,K] contiguous")
+    _require(m <= 64 and k % 8 == 0 and x.stride(0) % 8 == 0, f"gemm_skinny: needs M <= 64 and K % 8 == 0, got M={m} K={k}")
+    _require(x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0, "gemm_skinny: operands must be 16-byte aligned")
+    out_f32 = 0
+    if splits > 1:
+        _gpu(partials, "partials", torch.float32)
+        _require(partials.numel() >= splits * m * n and partials.is_contiguous(), "gemm_skinny: partials too small")
+    else:
+        _gpu(out, "out")
+        out_f32 = 1 if out.dtype == torch.float32 else 0
+        _require(out.shape == (m, n) and out.is_contiguous() and out.dtype in (torch.float32, torch.bfloat16),
+                 f"gemm_skinny: out must be contiguous [{m},{n}]")
+    _check(_fn("gemm", "dryft_gemm_skinny_bf16")(_ptr(x), x.stride(0), _ptr(w), _ptr(out), _ptr(partials), m, n, k,
+                                                 int(ntw), int(splits), out_f32, _stream()), "gemm_skinny_bf16")
+
+
+def sum_partials(partials: torch.Tensor, out: torch.Tensor, splits: int) -> torch.Tensor:
+    _gpu(partials, "partials", torch.float32)
+    _gpu(out, "out")
+    _require(out.is_contiguous() and partials.is_contiguous() and partials.numel() >= splits * out.numel(),
+             "sum_partials: partials must hold splits * out.numel() values")
+    _require(out.dtype in (torch.float32, torch.bfloat16), "sum_partials: out must be float32 or bfloat16")
+    _check(_fn("gemm", "dryft_sum_partials")(_ptr(partials), _ptr(out), out.numel(), splits,
+                                             1 if out.dtype == torch.float32 else 0, _stream()), "sum_partials")
+    return out
+
+
+# ---------------------------------------------------------------------------------------- sampling
+def argmax_rows(logits: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    _gpu(logits, "logits", torch.float32)
+    _gpu(out, "out", torch.int32)
+    rows, vocab = logits.shape
+    _require(logits.stride(1) == 1 and out.numel() >= rows and out.is_contiguous(), "argmax_rows: bad operands")
+    _check(_fn("sampling", "dryft_argmax_rows")(_ptr(logits), rows, vocab, logits.stride(0), _ptr(out), _stream()),
+           "argmax_rows")
+    return out
+
+
+def sample_rows(logits: torch.Tensor, temperature: float, uniforms: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    _gpu(logits, "logits", torch.float32)
+    _gpu(uniforms, "uniforms", torch.float32)
+    _gpu(out, "out", torch.int32)
+    rows, vocab = logits.shape
+    _require(temperature > 0, "sample_rows: temperature must be positive (use argmax_rows for greedy)")
+    _require(logits.stride(1) == 1 and out.numel() >= rows and uniforms.numel() >= rows, "sample_rows: bad operands")
+    _check(_fn("sampling", "dryft_sample_rows")(_ptr(logits), rows, vocab, logits.stride(0), float(temperature),
+                                                _ptr(uniforms), _ptr(out), _stream()), "sample_rows")
+    return out

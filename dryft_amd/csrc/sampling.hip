@@ -1,0 +1,102 @@
+// Choosing the next token from float logits, one workgroup per row.
+//  * greedy: the largest logit, the lowest index among equals (reference: logits.argmax at
+//    engine/dryft_qwen3/model.py:187, 262; tie rule AGENTS.md:174-175).
+//  * temperature: p = softmax(logits / T); the token is the first index whose running sum of p
+//    reaches u * sum(p), u in [0,1) given per row by the caller. The reference has no temperature
+//    sampling; this is this library's own.
+#include "common.h"
+
+#define SAMPLE_THREADS 1024
+
+__global__ __launch_bounds__(SAMPLE_THREADS) void argmax_rows_kernel(const float* __restrict__ logits, int vocab,
+                                                                     int64_t row_stride, int* __restrict__ out) {
+  __shared__ float best_v[SAMPLE_THREADS / WAVE];
+  __shared__ int best_i[SAMPLE_THREADS / WAVE];
+  const float* row = logits + blockIdx.x * row_stride;
+  float v = -INFINITY;
+  int idx = 0x7fffffff;
+  for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
+    const float x = row[i];
+    if (x > v || (x == v && i < idx)) {  // a NaN never wins a comparison
+      v = x;
+      idx = i;
+    }
+  }
+#pragma unroll
+  for (int o = WAVE / 2; o > 0; o >>= 1) {
+    const float ov = __shfl_xor(v, o, WAVE);
+    const int oi = __shfl_xor(idx, o, WAVE);
+    if (ov > v || (ov == v && oi < idx)) { v = ov; idx = oi; }
+  }
+  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+  if (lane == 0) { best_v[wave] = v; best_i[wave] = idx; }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < SAMPLE_THREADS / WAVE; ++w)
+      if (best_v[w] > v || (best_v[w] == v && best_i[w] < idx)) { v = best_v[w]; idx = best_i[w]; }
+    out[blockIdx.x] = idx < vocab ? idx : 0;
+  }
+}
+
+__global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(const float* __restrict__ logits, int vocab,
+                                                                     int64_t row_stride, float inv_temperature,
+                                                                     const float* __restrict__ uniforms,
+                                                                     int* __restrict__ out) {
+  __shared__ float scratch[16];
+  __shared__ float seg_sum[SAMPLE_THREADS];
+  __shared__ int chosen;
+  const float* row = logits + blockIdx.x * row_stride;
+  const int tid = threadIdx.x;
+  float mx = -INFINITY;
+  for (int i = tid; i < vocab; i += blockDim.x) mx = fmaxf(mx, row[i]);
+  mx = block_max(mx, scratch);
+  // each thread owns one contiguous segment, so that running sums follow the index order
+  const int seg = (vocab + SAMPLE_THREADS - 1) / SAMPLE_THREADS;
+  const int i0 = min(vocab, tid * seg), i1 = min(vocab, i0 + seg);
+  float s = 0.f;
+  for (int i = i0; i < i1; ++i) s += expf((row[i] - mx) * inv_temperature);
+  seg_sum[tid] = s;
+  if (tid == 0) chosen = vocab - 1;
+  __syncthreads();
+  if (tid == 0) {
+    float total = 0.f;
+    for (int t = 0; t < SAMPLE_THREADS; ++t) total += seg_sum[t];
+    const float target = uniforms[blockIdx.x] * total;
+    float run = 0.f;
+    int t = 0;
+    for (; t < SAMPLE_THREADS - 1; ++t) {
+      if (run + seg_sum[t] > target) break;
+      run += seg_sum[t];
+    }
+    // walk the segment that holds the target
+    const int a = min(vocab, t * seg), b = min(vocab, a + seg);
+    int pick = -1;
+    for (int i = a; i < b; ++i) {
+      run += expf((row[i] - mx) * inv_temperature);
+      if (run > target) { pick = i; break; }
+    }
+    if (pick < 0) {  // rounding left the target just beyond the sum: take the last token with weight
+      pick = vocab - 1;
+      while (pick > 0 && !(expf((row[pick] - mx) * inv_temperature) > 0.f)) --pick;
+    }
+    chosen = pick;
+  }
+  __syncthreads();
+  if (tid == 0) out[blockIdx.x] = chosen;
+}
+
+DRYFT_API int dryft_argmax_rows(const float* logits, int n_rows, int vocab, int64_t row_stride, int* out,
+                                hipStream_t stream) {
+  if (n_rows <= 0) return 0;
+  hipLaunchKernelGGL(argmax_rows_kernel, dim3(n_rows), dim3(SAMPLE_THREADS), 0, stream, logits, vocab, row_stride, out);
+  return DRYFT_LAUNCH_CHECK();
+}
+
+DRYFT_API int dryft_sample_rows(const float* logits, int n_rows, int vocab, int64_t row_stride, float temperature,
+                                const float* uniforms, int* out, hipStream_t stream) {
+  if (n_rows <= 0) return 0;
+  if (!(temperature > 0.f)) return -1;
+  hipLaunchKernelGGL(sample_rows_kernel, dim3(n_rows), dim3(SAMPLE_THREADS), 0, stream, logits, vocab, row_stride,
+                     1.f / temperature, uniforms, out);
+  return DRYFT_LAUNCH_CHECK();
+}

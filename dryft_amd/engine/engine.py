@@ -1,0 +1,156 @@
+"""The Python entry point, in the manner of the reference's ``Engine``.
+
+``Engine(model_path).generate(input_ids, max_new_tokens)`` yields one list of token ids
+per step, one id per sequence (reference: engine/engine.py:28-29, 138-140). What differs:
+any model folder whose ``config.json`` names a registered architecture is accepted rather
+than one pinned checkpoint; prompts of unequal length run in one step; sampling may use
+a temperature; stop tokens may end sequences early; capacities are constructor arguments
+instead of a global settings object (engine/dryft_qwen3/config.py:161-196), and a request
+beyond them is an error rather than a fallback to a freshly allocated cache
+(engine/engine.py:153-165).
+"""
+
+from __future__ import annotations
+
+import sys
+import time
+from typing import Any, Iterator, Sequence
+
+import torch
+
+from ..cache.store import CacheStore
+from ..config.base import read_config_json
+from ..models import resolve_architecture
+from ..sampling import Sampler
+from ..weights.loader import load_tensors
+from ..weights.random_init import random_tensors
+from . import generate as loop
+from .graph import DecodeGraph
+from .model import DecoderModel
+from .step import SeqStep, Stepper
+
+DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32}
+
+
+def log(*parts: object) -> None:
+    """Diagnostics go to stderr, as the reference's do (engine/dryft_qwen3/config.py:228-230)."""
+    print("[engine]", *parts, file=sys.stderr, flush=True)
+
+
+def require_gpu(device) -> torch.device:
+    device = torch.device(device)
+    if device.type != "cuda" or not torch.cuda.is_available():
+        raise RuntimeError("dryft_amd computes on an AMD GPU only (there is no CPU path); no GPU is visible")
+    return device
+
+
+class Engine:
+    def __init__(self, model_path: str | None = None, *, config: dict[str, Any] | None = None,
+                 seed: int | None = None, norm_std: float = 0.0, dtype: str = "bfloat16", max_batch: int = 32,
+                 max_len: int = 8192, max_tokens: int | None = None, use_graph: bool = True,
+                 device: str = "cuda:0", verbose: bool = False):
+        t0 = time.time()
+        self.device = require_gpu(device)
+        torch.cuda.set_device(self.device)
+        if dtype not in DTYPES:
+            raise ValueError(f"dtype must be one of {sorted(DTYPES)}, got {dtype!r}")
+        self.dtype = DTYPES[dtype]
+        if (model_path is None) == (config is None):
+            raise ValueError("give either model_path (a folder with config.json and safetensors) or config and seed")
+        raw = read_config_json(model_path) if model_path is not None else config
+        arch = resolve_architecture(raw)
+        self.config = arch.config_class.from_dict(raw)
+        self.model = DecoderModel(arch.plan(self.config), self.dtype, self.device)
+        specs = self.model.tensor_specs()
+        if model_path is not None:
+            tensors = load_tensors(model_path, specs, self.dtype, self.device, ignore=self.model.optional_names())
+        else:
+            if seed is None:
+                raise ValueError("random weights need a seed")
+            tensors = random_tensors(specs, seed, self.dtype, norm_std=norm_std, device=self.device)
+        self.model.load(tensors)
+        del tensors
+        self.max_batch, self.max_len = int(max_batch), int(max_len)
+        per_seq = -(-self.max_len // 64) * 64
+        self.max_tokens = int(max_tokens) if max_tokens is not None else self.max_batch * per_seq
+        self.cache = CacheStore(self.model.cache_needs(), max_tokens=self.max_tokens, n_slots=self.max_batch,
+                                max_len=self.max_len, dtype=self.dtype, device=self.device)
+        self.stepper = Stepper(self.model, self.cache)
+        self.use_graph = bool(use_graph)
+        self._graphs: dict[int, DecodeGraph] = {}
+        self._sampler = Sampler()
+        if verbose:
+            log(f"{arch.name} ready in {time.time() - t0:.1f}s: weights {self.model.weight_bytes() / 2**30:.2f} GiB, "
+                f"cache {self.cache.bytes() / 2**30:.2f} GiB for {self.max_tokens} tokens")
+
+    # ------------------------------------------------------------------ the step function
+    def step(self, seqs: list[SeqStep]) -> torch.Tensor:
+        return self.stepper.step(seqs)
+
+    # ------------------------------------------------------------------ StepBackend
+    def acquire(self, n: int) -> list[int]:
+        return self.cache.acquire(n)
+
+    def release(self, slots: list[int]) -> None:
+        self.cache.release(slots)
+
+    def reserve(self, slots: list[int], lengths: list[int]) -> None:
+        self.cache.reserve(slots, lengths)
+
+    def start(self, slots: list[int], prompts: list[list[int]], step_index: int) -> list[int]:
+        logits = self.stepper.step([SeqStep(s, p, [len(p) - 1]) for s, p in zip(slots, prompts)])
+        return self._choose(logits, len(slots))
+
+    def advance(self, slots: list[int], tokens: list[int], step_index: int) -> list[int]:
+        n = len(slots)
+        graph = self._graph_for(n)
+        if graph is not None:
+            live = [s for s in slots if s >= 0]
+            self.cache.begin_step(live, [1] * len(live))
+            logits = graph.replay(slots, tokens)
+            self.cache.end_step(live, [1] * len(live))
+        else:
+            # dead sequences keep their row so that rows and sequences stay aligned
+            logits = self.stepper.step([SeqStep(s, [t], [0]) for s, t in zip(slots, tokens)])
+            if len(logits) != n:
+                full = torch.zeros((n, logits.shape[1]), dtype=logits.dtype, device=logits.device)
+                idx = torch.tensor([i for i, s in enumerate(slots) if s >= 0], dtype=torch.long, device=logits.device)
+                full[idx] = logits
+                logits = full
+        return self._choose(logits, n)
+
+    def _choose(self, logits: torch.Tensor, n: int) -> list[int]:
+        uniforms = None if self._sampler.greedy else self._sampler.draw(n)
+        return self._sampler.choose(logits, uniforms).tolist()
+
+    def _graph_for(self, batch: int) -> DecodeGraph | None:
+        if not self.use_graph:
+            return None
+        g = self._graphs.get(batch)
+        if g is None:
+            g = DecodeGraph(self.stepper, batch)
+            g.capture()
+            self._graphs[batch] = g
+        return g
+
+    # ------------------------------------------------------------------ generation
+    def generate(self, input_ids: Sequence[Sequence[int]], max_new_tokens: int, *, temperature: float = 0.0,
+                 sample_seed: int = 0, stop_token_ids: Sequence[int] = ()) -> Iterator[list[int]]:
+        """Yields one list of ``len(input_ids)`` token ids per step; ``-1`` marks an ended sequence."""
+        prompts = [list(map(int, p)) for p in input_ids]
+        if not prompts or max_new_tokens <= 0:
+            return
+        self._sampler = Sampler(temperature, sample_seed)
+        if len(prompts) <= self.max_batch:
+            yield from loop.generate_batch(self, prompts, max_new_tokens, stop_token_ids)
+            return
+        # more requests than one batch holds: batches run one after another, then the steps are handed out
+        per_request = loop.generate_all(self, prompts, max_new_tokens, stop_token_ids)
+        for t in range(max(len(r) for r in per_request)):
+            yield [r[t] if t < len(r) else loop.FILL for r in per_request]
+
+    def generate_all(self, input_ids: Sequence[Sequence[int]], max_new_tokens: int, *, temperature: float = 0.0,
+                     sample_seed: int = 0, stop_token_ids: Sequence[int] = ()) -> list[list[int]]:
+        """Per request the list of tokens generated for it (a stop token included)."""
+        self._sampler = Sampler(temperature, sample_seed)
+        return loop.generate_all(self, [list(map(int, p)) for p in input_ids], max_new_tokens, stop_token_ids)

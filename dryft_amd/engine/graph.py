@@ -1,0 +1,60 @@
+"""A decoding step captured once per batch size and replayed.
+
+The reference captures one graph per (batch bucket, length bucket) after three warm
+runs on a side stream and checks a replay against eager (engine/dryft_qwen3/graphs.py:108-135,
+146-169). Here every quantity that changes from step to step (tokens, slots, positions,
+lengths, page tables) is read from device memory, so one graph per batch size serves
+every position and length. Warm runs and the capture itself run with every row marked
+dead (slot -1), which launches the same kernels but writes to no cache slot and advances
+no length.
+"""
+
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+from ..parts.base import StepContext
+from .step import BatchBuffers, Stepper
+
+
+class DecodeGraph:
+    def __init__(self, stepper: Stepper, batch_size: int):
+        self.stepper, self.batch = stepper, int(batch_size)
+        dev = stepper.device
+        self.buf = BatchBuffers(self.batch, self.batch, dev)
+        self.buf.q_len.fill_(1)
+        self.ctx: StepContext = stepper.context(self.buf, self.batch, self.batch, max_q_len=1, max_tiles=self.batch,
+                                                max_kv_len=stepper.cache.max_len, host=None)
+        self.logits: torch.Tensor | None = None
+        self.graph: torch.cuda.CUDAGraph | None = None
+        self._stage = torch.zeros(2 * self.batch, dtype=torch.int32).pin_memory()
+
+    def _body(self) -> torch.Tensor:
+        hidden = self.stepper.run(self.buf, self.ctx)
+        return self.stepper.model.logits(hidden, None)
+
+    def capture(self, warm_runs: int = 2) -> None:
+        self.buf.seq_slot.fill_(-1)
+        side = torch.cuda.Stream(device=self.stepper.device)
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(warm_runs):
+                self._body()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            self.logits = self._body()
+        self.graph = graph
+
+    def replay(self, slots: list[int], tokens: list[int]) -> torch.Tensor:
+        """Logits ``[batch, vocab]`` of one more token each; rows of dead sequences hold nothing of use."""
+        n = self.batch
+        stage = self._stage
+        stage[:n] = torch.from_numpy(np.asarray(tokens, dtype=np.int32))
+        stage[n:] = torch.from_numpy(np.asarray(slots, dtype=np.int32))
+        self.buf.tokens.copy_(stage[:n], non_blocking=True)
+        self.buf.seq_slot.copy_(stage[n:], non_blocking=True)
+        self.graph.replay()
+        return self.logits

@@ -1,0 +1,49 @@
+"""The one registry from an architecture's name to its configuration and plan.
+
+``config.json["architectures"][0]`` selects the entry. The reference never
+reads that key (it serves one pinned checkpoint, engine/dryft_qwen3/config.py:55-70);
+here it is the only place where a model is chosen.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Any, Callable
+
+from ..config.base import ConfigError
+from ..config.plan import ModelPlan
+
+
+@dataclass(frozen=True)
+class Architecture:
+    name: str
+    config_class: Any                       # has from_dict(raw) and to_dict()
+    plan: Callable[[Any], ModelPlan]        # typed config -> ModelPlan
+
+
+_REGISTRY: dict[str, Architecture] = {}
+
+
+def register_architecture(name: str, config_class: Any, plan: Callable[[Any], ModelPlan]) -> None:
+    if name in _REGISTRY:
+        raise ValueError(f"architecture {name!r} is already registered")
+    _REGISTRY[name] = Architecture(name, config_class, plan)
+
+
+def known_architectures() -> list[str]:
+    return sorted(_REGISTRY)
+
+
+def resolve_architecture(raw_config: dict[str, Any]) -> Architecture:
+    names = raw_config.get("architectures")
+    if not isinstance(names, list) or not names or not isinstance(names[0], str):
+        raise ConfigError("config.json", [
+            f"architectures: expected a list naming the model class, got {names!r}; known: {known_architectures()}"])
+    arch = _REGISTRY.get(names[0])
+    if arch is None:
+        raise ConfigError("config.json", [
+            f"architectures: {names[0]!r} is not registered; known: {known_architectures()}"])
+    return arch
+
+
+from . import qwen3 as _qwen3  # noqa: E402,F401  (registers Qwen3ForCausalLM)

@@ -1,0 +1,113 @@
+"""Grouped-query attention over the paged cache.
+
+Per row: ``q, k, v`` from one fused projection (reference: engine/dryft_qwen3/weights.py:93-96);
+optional RMSNorm over each q and k head (one weight per head width, before the rotation,
+model.py:165-166); optional rotary positions; append k and v to the cache line (model.py:170-171);
+causal scores ``(q . k) / sqrt(head_dim)`` against every cached key of the sequence up to the row's
+own position (or the last ``window`` of them), query head ``h`` reading kv head ``h // group``
+(model.py:172-177, 254-257); output projection (model.py:179). No biases.
+
+The part knows nothing of the model around it: sizes and constants are constructor arguments, the
+position encoding is looked up by name in the step context, and its storage is the cache line it
+is handed.
+"""
+
+from __future__ import annotations
+
+import math
+
+import torch
+
+from ..cache.spec import KVNeed
+from ..cache.store import KVLine
+from ..csrc import ops
+from ..weights.spec import VECTOR
+from . import register_part
+from .base import Mixer, StepContext, matrix
+from .linear import linear
+
+_SPLIT_TARGET_WAVES = 1024
+_MAX_SPLITS = 32
+
+
+class GQAAttention(Mixer):
+    def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
+                 qk_norm_eps: float | None = None, positions: str | None = None, rotary_dim: int | None = None,
+                 window: int | None = None, scale: float | None = None):
+        if num_heads % num_kv_heads:
+            raise ValueError(f"{num_heads} query heads cannot share {num_kv_heads} kv heads evenly")
+        if head_dim % 16 or head_dim > 256:
+            raise ValueError(f"head_dim must be a multiple of 16 up to 256, got {head_dim}")
+        self.hidden, self.n_heads, self.n_kv, self.head_dim = int(hidden_size), int(num_heads), int(num_kv_heads), int(head_dim)
+        self.qk_norm_eps = qk_norm_eps
+        self.positions = positions
+        self.rotary_dim = int(rotary_dim if rotary_dim is not None else head_dim) if positions else 0
+        self.window = int(window) if window else None
+        self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(head_dim)   # model.py:65
+        self.q_dim, self.kv_dim = self.n_heads * self.head_dim, self.n_kv * self.head_dim
+        self.w_qkv = self.w_o = self.q_norm = self.k_norm = None
+
+    def tensor_specs(self):
+        specs = {"q_proj": matrix((self.q_dim, self.hidden)), "k_proj": matrix((self.kv_dim, self.hidden)),
+                 "v_proj": matrix((self.kv_dim, self.hidden)), "o_proj": matrix((self.hidden, self.q_dim))}
+        if self.qk_norm_eps is not None:
+            specs["q_norm"] = ((self.head_dim,), VECTOR, "ones")
+            specs["k_norm"] = ((self.head_dim,), VECTOR, "ones")
+        return specs
+
+    def load(self, tensors):
+        self.w_qkv = torch.cat([tensors["q_proj"], tensors["k_proj"], tensors["v_proj"]], dim=0).contiguous()
+        self.w_o = tensors["o_proj"]
+        if self.qk_norm_eps is not None:
+            self.q_norm, self.k_norm = tensors["q_norm"], tensors["k_norm"]
+            if self.q_norm.dtype != self.k_norm.dtype:          # one kernel argument says how both are stored
+                self.q_norm, self.k_norm = self.q_norm.float(), self.k_norm.float()
+
+    def cache_need(self):
+        return KVNeed(self.n_kv, self.head_dim, self.window)
+
+    def kernel_modules(self, dtype):
+        return ("gemm", "rope_kv", "attn_rows") + (("attn_mfma",) if dtype == torch.bfloat16 else ())
+
+    def forward(self, h: torch.Tensor, ctx: StepContext, line: KVLine, writes_cache: bool):
+        rows = h.shape[0]
+        qkv = linear(h, self.w_qkv)
+        cos = sin = None
+        if self.positions:
+            table = ctx.positions[self.positions]
+            cos, sin = table.cos, table.sin
+            if ctx.max_kv_len > table.n_positions:
+                raise ValueError(f"position tables cover {table.n_positions} positions, the step reaches {ctx.max_kv_len}")
+        q = torch.empty((rows, self.n_heads, self.head_dim), dtype=h.dtype, device=h.device)
+        ops.qk_norm_rope_kv(qkv, self.q_norm, self.k_norm, self.qk_norm_eps or 0.0, cos, sin, self.rotary_dim,
+                            ctx.row_slot, ctx.row_pos, q, line.k, line.v, line.page_table, writes_cache,
+                            self.n_heads, self.n_kv, self.head_dim)
+        out = torch.empty_like(q)
+        window = self.window or 0
+        if h.dtype == torch.bfloat16:
+            if ctx.max_q_len == 1:
+                splits = self.decode_splits(ctx.n_seqs, ctx.max_kv_len)
+                part_o = torch.empty((ctx.n_seqs, self.n_heads, splits, self.head_dim), dtype=torch.float32, device=h.device)
+                part_ml = torch.empty((ctx.n_seqs, self.n_heads, splits, 2), dtype=torch.float32, device=h.device)
+                ops.attn_split_bf16(q, line.k, line.v, line.page_table, ctx.seq_slot, ctx.cu_rows, ctx.kv_len,
+                                    ctx.n_seqs, part_o, part_ml, splits, out, self.n_heads, self.n_kv, self.head_dim,
+                                    self.scale, window)
+            else:
+                ops.attn_causal_bf16(q, line.k, line.v, line.page_table, ctx.seq_slot, ctx.cu_rows, ctx.tile_cu,
+                                     ctx.seq_start, ctx.n_seqs, ctx.max_tiles, out, self.n_heads, self.n_kv,
+                                     self.head_dim, self.scale, window)
+        else:
+            ops.attn_rows(q, line.k, line.v, line.page_table, ctx.row_slot, ctx.row_pos, out, self.n_heads, self.n_kv,
+                          self.head_dim, self.scale, window)
+        return linear(out.view(rows, self.q_dim), self.w_o, allow_partials=True)
+
+    def decode_splits(self, n_seqs: int, max_kv_len: int) -> int:
+        """How many ways each sequence's keys are split so the chip has enough waves to hide latency."""
+        blocks = self.n_kv * ((self.n_heads // self.n_kv + 15) // 16)
+        want = (_SPLIT_TARGET_WAVES + n_seqs * blocks - 1) // (n_seqs * blocks)
+        span = self.window if self.window else max_kv_len
+        pages = max(1, (span + 63) // 64)
+        return max(1, min(want, _MAX_SPLITS, pages))
+
+
+register_part("gqa_attention", GQAAttention)

@@ -1,0 +1,113 @@
+"""What a part is, and what it is told about a step.
+
+A part (mixer, feed-forward, norm, position encoding, embedding, head) is built
+from sizes and constants alone, names the tensors it needs by logical name, and
+computes on packed rows. It never learns which model it is in: the model plan
+maps logical tensor names to checkpoint names and wires the parts together.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Any
+
+import torch
+
+from ..weights.spec import MATRIX
+
+
+@dataclass
+class HostBatch:
+    """The step as the host knows it (absent while a captured graph is replayed)."""
+
+    slots: list[int]      # cache slot of each sequence, -1 for a sequence that sits out
+    q_lens: list[int]     # rows each sequence occupies in this step
+    starts: list[int]     # tokens each sequence had cached before the step
+
+
+@dataclass
+class StepContext:
+    """Per-step facts shared by all parts. Index tensors are int32 on the device.
+
+    Rows are the step's tokens, packed sequence after sequence. Row ``r`` belongs to
+    sequence ``row_seq[r]`` in cache slot ``row_slot[r]`` (-1: takes no part) at
+    position ``row_pos[r]``. ``cu_rows``/``tile_cu`` are prefix sums over sequences of
+    rows and of 64-row tiles; ``kv_len`` is each sequence's cached length after this
+    step, ``seq_start`` before it.
+    """
+
+    n_rows: int
+    n_seqs: int
+    dtype: torch.dtype
+    device: torch.device
+    row_seq: torch.Tensor
+    row_slot: torch.Tensor
+    row_pos: torch.Tensor
+    cu_rows: torch.Tensor
+    tile_cu: torch.Tensor
+    seq_slot: torch.Tensor
+    q_len: torch.Tensor
+    kv_len: torch.Tensor
+    seq_start: torch.Tensor
+    max_q_len: int                      # host bound on rows per sequence; 1 means a decoding step
+    max_tiles: int                      # host bound on 64-row tiles in the step
+    max_kv_len: int                     # host bound on any sequence's cached length after the step
+    host: HostBatch | None = None
+    positions: dict[str, Any] = field(default_factory=dict)   # name -> position encoding, tables ready
+
+
+@dataclass
+class Partials:
+    """A matrix product left as ``count`` float32 partial sums ``[count, rows, width]``."""
+
+    data: torch.Tensor
+    count: int
+
+
+class Part:
+    """Base of all parts. ``tensor_specs`` maps logical names to (shape, role, init)."""
+
+    def tensor_specs(self) -> dict[str, tuple[tuple[int, ...], str, str]]:
+        return {}
+
+    def load(self, tensors: dict[str, torch.Tensor]) -> None:
+        """Receives the tensors named by ``tensor_specs`` (on the device, in their held dtype)."""
+
+    def kernel_modules(self, dtype: torch.dtype) -> tuple[str, ...]:
+        """The kernel libraries this part will call, so they can be compiled together up front."""
+        return ()
+
+
+class Norm(Part):
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        raise NotImplementedError
+
+    def add_forward(self, res: torch.Tensor, delta) -> tuple[torch.Tensor, torch.Tensor]:
+        """``(res + delta, norm(res + delta))``; ``delta`` is a tensor like ``res`` or ``Partials``."""
+        raise NotImplementedError
+
+
+class Mixer(Part):
+    """Mixes information across positions of a sequence; owns one cache line per run."""
+
+    def cache_need(self):
+        """A ``KVNeed``, a ``StateNeed`` or None."""
+        return None
+
+    def forward(self, h: torch.Tensor, ctx: StepContext, line, writes_cache: bool):
+        """``h`` is ``[rows, hidden]``; returns a tensor of the same shape or ``Partials``."""
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, h: torch.Tensor, ctx: StepContext):
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    def prepare(self, n_positions: int, dtype: torch.dtype, device) -> None:
+        """Build whatever tables are needed for positions ``0..n_positions-1``."""
+
+
+def matrix(shape) -> tuple[tuple[int, ...], str, str]:
+    return (tuple(shape), MATRIX, "normal")

@@ -1,0 +1,77 @@
+"""``y = x @ W.T`` for weights in checkpoint layout ``[out, in]`` (no bias).
+
+The reference hands every projection to a vendor library (F.linear,
+engine/dryft_qwen3/model.py:153, 179-180, 237, 258-261). Here:
+
+* float32: this library's own kernel, plain multiply-adds, so the 32-bit path has no
+  reduced-precision matrix mode anywhere;
+* bfloat16, at most 64 rows (decoding and the output head): this library's
+  weight-streaming matrix-core kernel, which can leave its result as float32 partial
+  sums over K for the consumer to add;
+* bfloat16, many rows (prompts): the vendor library through ``torch.mm``, as in the
+  reference; sizes it or the skinny kernel cannot take go to the plain kernel.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from ..csrc import ops
+from .base import Partials
+
+SKINNY_ROWS = 64
+_TARGET_WORKGROUPS = 512   # about two per compute unit
+
+
+def skinny_plan(m: int, n: int, k: int) -> tuple[int, int]:
+    """(weight tiles per wave, splits of K across workgroups) for the skinny kernel."""
+    tiles = (n + 15) // 16
+    m_tiles = (m + 15) // 16
+    ntw = 1
+    if m_tiles >= 2 and tiles >= 1024:
+        ntw = 2
+    if m_tiles >= 3 and tiles >= 4096:
+        ntw = 4
+    workgroups = (tiles + ntw - 1) // ntw
+    k_blocks = (k + 63) // 64
+    splits = max(1, min((_TARGET_WORKGROUPS + workgroups - 1) // workgroups, k_blocks // 8, 16))
+    return ntw, splits
+
+
+def _skinny_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
+    return x.shape[1] % 8 == 0 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0
+
+
+def linear(x: torch.Tensor, w: torch.Tensor, *, out_dtype: torch.dtype | None = None, allow_partials: bool = False):
+    """Returns ``[rows, out]`` in ``out_dtype`` (default: the dtype of ``x``), or ``Partials``."""
+    m, k = x.shape
+    n = w.shape[0]
+    out_dtype = out_dtype or x.dtype
+    if x.dtype == torch.float32:
+        return ops.gemm_tiled(x, w, torch.empty((m, n), dtype=torch.float32, device=x.device))
+    if m <= SKINNY_ROWS and _skinny_ok(x, w):
+        ntw, splits = skinny_plan(m, n, k)
+        if splits > 1:
+            partials = torch.empty((splits, m, n), dtype=torch.float32, device=x.device)
+            ops.gemm_skinny_bf16(x, w, None, partials, ntw, splits)
+            if allow_partials:
+                return Partials(partials, splits)
+            return ops.sum_partials(partials, torch.empty((m, n), dtype=out_dtype, device=x.device), splits)
+        out = torch.empty((m, n), dtype=out_dtype, device=x.device)
+        ops.gemm_skinny_bf16(x, w, out, None, ntw, 1)
+        return out
+    if out_dtype == torch.float32:
+        out = torch.empty((m, n), dtype=torch.float32, device=x.device)
+        if _skinny_ok(x, w):
+            ntw, _ = skinny_plan(SKINNY_ROWS, n, k)
+            for m0 in range(0, m, SKINNY_ROWS):
+                ops.gemm_skinny_bf16(x[m0:m0 + SKINNY_ROWS], w, out[m0:m0 + SKINNY_ROWS], None, ntw, 1)
+            return out
+        return ops.gemm_tiled(x, w, out)
+    if k % 8 == 0 and n % 8 == 0 and x.is_contiguous():
+        return torch.mm(x, w.t())
+    return ops.gemm_tiled(x, w, torch.empty((m, n), dtype=x.dtype, device=x.device))
+
+
+def linear_modules(dtype: torch.dtype) -> tuple[str, ...]:
+    return ("gemm",)

@@ -1,0 +1,391 @@
+"""Each HIP kernel alone against a plain float32 reference of the same operation, at sizes other
+than the engine's tiny models use. Shapes and tolerances follow the reference's kernel self-tests
+(kernels/rmsnorm.py:106-132, rope_qknorm.py:172-227, attn_decode.py:180-226, silu_mul.py:53-63)."""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import bf16_tolerance, build_pages
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+def ops():
+    from dryft_amd.csrc import ops as o
+    return o
+
+
+def close(got, want, dtype, ulps=2.0, floor=0.0, what=""):
+    got, want = got.float().cpu(), want.float().cpu()
+    assert torch.isfinite(got).all(), f"{what}: non-finite output"
+    tol = bf16_tolerance(want, ulps, floor) if dtype == torch.bfloat16 else 2e-5 * float(want.abs().max()) + 1e-6
+    diff = float((got - want).abs().max())
+    assert diff <= tol, f"{what}: max diff {diff} > {tol}"
+
+
+# ------------------------------------------------------------------------------------------- embed
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_embed_rows(dtype):
+    torch.manual_seed(0)
+    table = torch.randn(331, 100).to(dtype)
+    tokens = torch.tensor([0, 330, 5, 5, 17, 200, 1], dtype=torch.int32)
+    out = torch.empty(7, 100, dtype=dtype, device=DEV)
+    ops().embed_rows(tokens.to(DEV), table.to(DEV), out)
+    assert torch.equal(out.cpu(), table[tokens.long()])
+
+
+# -------------------------------------------------------------------------------------------- norm
+def rmsnorm_ref(x, w, eps, dtype):
+    xf = x.float()
+    n = (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)).to(dtype).float()
+    return (n * w.float()).to(dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rows,width", [(1, 2560), (7, 2560), (33, 128), (1000, 128), (5, 100), (3, 9), (2, 5120)])
+def test_rmsnorm_and_add(dtype, rows, width):
+    torch.manual_seed(rows * 1000 + width)
+    res = (3 * torch.randn(rows, width)).to(dtype)
+    x = (3 * torch.randn(rows, width)).to(dtype)
+    w = (1 + 0.1 * torch.randn(width)).to(dtype)
+    eps = 1e-6
+    o = ops()
+    y = torch.empty(rows, width, dtype=dtype, device=DEV)
+    o.add_rmsnorm(res.to(DEV), None, w.to(DEV), eps, None, y)
+    close(y, rmsnorm_ref(res, w, eps, dtype), dtype, what="rmsnorm")
+    # weights stored in 32-bit are taken as they are
+    o.add_rmsnorm(res.to(DEV), None, w.float().to(DEV), eps, None, y)
+    close(y, rmsnorm_ref(res, w, eps, dtype), dtype, what="rmsnorm with float32 weight")
+    # residual add: the sum is rounded once and must be bit-equal to the library's add
+    res_d, y2 = res.to(DEV).clone(), torch.empty(rows, width, dtype=dtype, device=DEV)
+    o.add_rmsnorm(res_d, x.to(DEV), w.to(DEV), eps, res_d, y2)
+    want_res = (res.float() + x.float()).to(dtype)
+    assert torch.equal(res_d.cpu(), want_res), "residual sum differs"
+    close(y2, rmsnorm_ref(want_res, w, eps, dtype), dtype, what="add_rmsnorm")
+    # partial sums in float32 are added in order
+    parts = torch.randn(3, rows, width)
+    res_d = res.to(DEV).clone()
+    o.add_rmsnorm(res_d, parts.to(DEV), w.to(DEV), eps, res_d, y2, n_partials=3)
+    want_res = (res.float() + ((parts[0] + parts[1]) + parts[2])).to(dtype)
+    close(res_d, want_res, dtype, ulps=1.0, what="residual + partials")
+    close(y2, rmsnorm_ref(res_d.cpu(), w, eps, dtype), dtype, what="norm after partials")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_add_rows(dtype):
+    torch.manual_seed(1)
+    a, b = torch.randn(37, 96).to(dtype), torch.randn(37, 96).to(dtype)
+    out = torch.empty(37, 96, dtype=dtype, device=DEV)
+    ops().add_rows(a.to(DEV), b.to(DEV), out)
+    assert torch.equal(out.cpu(), (a.float() + b.float()).to(dtype))
+
+
+# -------------------------------------------------------------------------------------- activation
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rows,inter", [(1, 9728), (7, 9728), (3, 2048), (5, 224), (2, 37)])
+def test_silu_mul(dtype, rows, inter):
+    torch.manual_seed(rows + inter)
+    gu = (3 * torch.randn(rows, 2 * inter)).to(dtype)
+    g, u = gu[:, :inter].float(), gu[:, inter:].float()
+    want = (torch.nn.functional.silu(g).to(dtype).float() * u).to(dtype)
+    out = torch.empty(rows, inter, dtype=dtype, device=DEV)
+    ops().silu_mul(gu.to(DEV), out)
+    close(out, want, dtype, what="silu_mul")
+
+
+# ----------------------------------------------------------------------------------------- rope_kv
+def rope_ref(x, cos, sin, dtype):
+    """x [rows, heads, D] float; cos/sin [rows, D/2] (already in dtype); rounding as the bf16 path does."""
+    half = x.shape[-1] // 2
+    c, s = cos.float()[:, None, :], sin.float()[:, None, :]
+    x1, x2 = x[..., :half], x[..., half:]
+    r = lambda t: t.to(dtype).float()
+    return torch.cat((r(r(x1 * c) - r(x2 * s)), r(r(x2 * c) + r(x1 * s))), dim=-1)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("n_heads,n_kv,D,theta", [(32, 8, 128, 5e6), (6, 3, 48, 1e4), (4, 2, 16, 1e6), (5, 1, 256, 1e5)])
+def test_qk_norm_rope_kv(dtype, n_heads, n_kv, D, theta):
+    torch.manual_seed(D)
+    rows, n_slots, max_pages, n_pages = 23, 7, 6, 42
+    L = max_pages * 64
+    eps = 1e-6
+    qkv = (2 * torch.randn(rows, (n_heads + 2 * n_kv) * D)).to(dtype)
+    wq = (1 + 0.1 * torch.randn(D)).to(dtype)
+    wk = (1 + 0.1 * torch.randn(D)).to(dtype)
+    inv = 1.0 / (theta ** (torch.arange(0, D, 2).float() / D))
+    ang = torch.arange(L).float()[:, None] * inv[None]
+    cos, sin = ang.cos().to(dtype), ang.sin().to(dtype)
+    rng = np.random.default_rng(D)
+    # rows spread over slots at distinct (slot, position) places; one row is dead
+    places = rng.permutation(n_slots * L)[:rows]
+    row_slot = torch.tensor(places // L, dtype=torch.int32)
+    row_pos = torch.tensor(places % L, dtype=torch.int32)
+    row_slot[5] = -1
+    table = torch.tensor(rng.permutation(n_pages).reshape(n_slots, max_pages), dtype=torch.int32)
+    k_pages = torch.zeros(n_pages, n_kv, 64, D, dtype=dtype, device=DEV)
+    v_pages = torch.zeros(n_pages, n_kv, D, 64, dtype=dtype, device=DEV)
+    q_out = torch.full((rows, n_heads, D), 7.0, dtype=dtype, device=DEV)
+    ops().qk_norm_rope_kv(qkv.to(DEV), wq.to(DEV), wk.to(DEV), eps, cos.to(DEV), sin.to(DEV), D, row_slot.to(DEV),
+                          row_pos.to(DEV), q_out, k_pages, v_pages, table.to(DEV), True, n_heads, n_kv, D)
+    q = qkv[:, : n_heads * D].view(rows, n_heads, D)
+    k = qkv[:, n_heads * D: (n_heads + n_kv) * D].view(rows, n_kv, D)
+    v = qkv[:, (n_heads + n_kv) * D:].view(rows, n_kv, D)
+
+    def norm(x, w):
+        xf = x.float()
+        n = (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)).to(dtype).float()
+        return (n * w.float()).to(dtype).float()
+
+    pos = row_pos.long()
+    q_want = rope_ref(norm(q, wq), cos[pos], sin[pos], dtype)
+    k_want = rope_ref(norm(k, wk), cos[pos], sin[pos], dtype)
+    live = row_slot >= 0
+    close(q_out[live.to(DEV)], q_want[live], dtype, what="q")
+    assert not q_out[5].any(), "a dead row's q must be zero"
+    kp, vp = k_pages.cpu(), v_pages.cpu()
+    for r in range(rows):
+        if not live[r]:
+            continue
+        page = int(table[row_slot[r], row_pos[r] // 64])
+        at = int(row_pos[r]) % 64
+        close(kp[page, :, at], k_want[r], dtype, what=f"k row {r}")
+        assert torch.equal(vp[page, :, :, at], v[r]), f"v row {r} must be copied unchanged"
+        kp[page, :, at] = 0
+        vp[page, :, :, at] = 0
+    assert not kp.any() and not vp.any(), "the kernel wrote outside the rows' places"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_rope_partial_width_and_no_norm(dtype):
+    """Rotation over the first `rot` lanes only, no q/k norm, and a run that writes no cache."""
+    torch.manual_seed(3)
+    rows, n_heads, n_kv, D, rot = 9, 4, 2, 64, 32
+    qkv = torch.randn(rows, (n_heads + 2 * n_kv) * D).to(dtype)
+    ang = torch.arange(128).float()[:, None] * (1.0 / (1e4 ** (torch.arange(0, rot, 2).float() / rot)))[None]
+    cos, sin = ang.cos().to(dtype), ang.sin().to(dtype)
+    row_slot = torch.zeros(rows, dtype=torch.int32)
+    row_pos = torch.arange(10, 10 + rows, dtype=torch.int32)
+    q_out = torch.empty(rows, n_heads, D, dtype=dtype, device=DEV)
+    ops().qk_norm_rope_kv(qkv.to(DEV), None, None, 0.0, cos.to(DEV), sin.to(DEV), rot, row_slot.to(DEV),
+                          row_pos.to(DEV), q_out, None, None, None, False, n_heads, n_kv, D)
+    q = qkv[:, : n_heads * D].view(rows, n_heads, D).float()
+    want = q.clone()
+    want[..., :rot] = rope_ref(q[..., :rot], cos[row_pos.long()], sin[row_pos.long()], dtype)
+    close(q_out, want, dtype, what="partial rotary")
+
+
+# --------------------------------------------------------------------------------------- attention
+def attention_ref(q, k, v, lengths, q_pos, scale, window=None):
+    """q [B, Tq, nH, D] at positions q_pos [B, Tq]; k, v [B, L, nKV, D] float32; float64 softmax."""
+    B, Tq, n_heads, D = q.shape
+    group = n_heads // k.shape[2]
+    out = torch.zeros(B, Tq, n_heads, D, dtype=torch.float64)
+    for b in range(B):
+        kk = k[b].double().repeat_interleave(group, dim=1)
+        vv = v[b].double().repeat_interleave(group, dim=1)
+        for t in range(Tq):
+            p = int(q_pos[b, t])
+            if p < 0:
+                continue
+            lo = 0 if window is None else max(0, p - window + 1)
+            s = torch.einsum("hd,jhd->hj", q[b, t].double(), kk[lo: p + 1]) * scale
+            out[b, t] = torch.einsum("hj,jhd->hd", torch.softmax(s, -1), vv[lo: p + 1])
+    return out.float()
+
+
+CASES = [  # n_heads, n_kv, D, lengths (cached tokens incl. the rows'), q rows per sequence
+    (32, 8, 128, [1, 513, 300, 64], 1),
+    (32, 8, 128, [700], 1),
+    (8, 2, 32, [5, 130, 31, 64, 65, 1], 1),
+    (6, 3, 48, [100, 129], 1),
+    (4, 2, 16, [17, 9, 200], 1),
+    (20, 1, 64, [77, 140], 1),          # 20 heads on one kv head: two blocks of 16 rows
+    (32, 8, 128, [150, 64, 209], 70),   # prompts continuing after cached tokens
+    (8, 2, 32, [31, 13, 6, 1], 31),
+    (6, 3, 48, [129, 90], 64),
+    (4, 2, 16, [300], 300),
+]
+
+
+def run_attention_case(kind, dtype, n_heads, n_kv, D, lengths, tq, window=None, seed=0):
+    torch.manual_seed(seed + D + len(lengths))
+    B, L = len(lengths), max(lengths)
+    n_slots, n_pages = B + 2, sum((n + 63) // 64 for n in lengths) + 3
+    k = torch.randn(B, L, n_kv, D).to(dtype)
+    v = torch.randn(B, L, n_kv, D).to(dtype)
+    q_lens = [min(tq, n) for n in lengths]
+    q_pos = torch.full((B, max(q_lens)), -1, dtype=torch.long)
+    for b, (n, ql) in enumerate(zip(lengths, q_lens)):
+        q_pos[b, :ql] = torch.arange(n - ql, n)
+    q = torch.randn(B, max(q_lens), n_heads, D).to(dtype)
+    # make one far key stand out for the last row of each sequence, so a lost key shows
+    for b, n in enumerate(lengths):
+        far = 0 if window is None else max(0, n - window)
+        k[b, far, :, :] = (4.0 * q[b, q_lens[b] - 1].float().view(n_kv, -1, D).mean(1)).to(dtype)
+    scale = 1.0 / math.sqrt(D)
+    want = attention_ref(q.float(), k.float(), v.float(), lengths, q_pos, scale, window)
+    k_pages, v_pages, table, slots = build_pages(k, v, lengths, n_pages, n_slots, seed=seed, poison=1e4)
+    rows = sum(q_lens)
+    q_packed = torch.cat([q[b, :ql] for b, ql in enumerate(q_lens)]).contiguous()
+    want_packed = torch.cat([want[b, :ql] for b, ql in enumerate(q_lens)])
+    row_slot = torch.tensor([slots[b] for b, ql in enumerate(q_lens) for _ in range(ql)], dtype=torch.int32)
+    row_pos = torch.tensor([int(p) for b, ql in enumerate(q_lens) for p in q_pos[b, :ql]], dtype=torch.int32)
+    cu = np.concatenate([[0], np.cumsum(q_lens)]).astype(np.int32)
+    tiles = np.concatenate([[0], np.cumsum([(ql + 63) // 64 for ql in q_lens])]).astype(np.int32)
+    d = lambda t: t.to(DEV)
+    out = torch.zeros(rows, n_heads, D, dtype=dtype, device=DEV)
+    o = ops()
+    w = window or 0
+    if kind == "rows":
+        o.attn_rows(d(q_packed), d(k_pages), d(v_pages), d(table), d(row_slot), d(row_pos), out, n_heads, n_kv, D, scale, w)
+    elif kind == "causal":
+        o.attn_causal_bf16(d(q_packed), d(k_pages), d(v_pages), d(table), d(torch.tensor(slots, dtype=torch.int32)),
+                           d(torch.from_numpy(cu)), d(torch.from_numpy(tiles)),
+                           d(torch.tensor([n - ql for n, ql in zip(lengths, q_lens)], dtype=torch.int32)), B,
+                           int(tiles[-1]) + 1, out, n_heads, n_kv, D, scale, w)
+    else:
+        splits = kind
+        part_o = torch.empty(B * n_heads * splits * D, dtype=torch.float32, device=DEV)
+        part_ml = torch.empty(B * n_heads * splits * 2, dtype=torch.float32, device=DEV)
+        o.attn_split_bf16(d(q_packed), d(k_pages), d(v_pages), d(table), d(torch.tensor(slots, dtype=torch.int32)),
+                          d(torch.from_numpy(cu)), d(torch.tensor(lengths, dtype=torch.int32)), B, part_o, part_ml,
+                          splits, out, n_heads, n_kv, D, scale, w)
+    close(out, want_packed, dtype, ulps=4.0, floor=1e-3, what=f"attention {kind} {n_heads}/{n_kv}/{D} {lengths} tq={tq}")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("case", CASES)
+def test_attn_rows(dtype, case):
+    run_attention_case("rows", dtype, *case)
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_attn_causal_bf16(case):
+    run_attention_case("causal", torch.bfloat16, *case)
+
+
+@pytest.mark.parametrize("splits", [1, 2, 5, 32])
+@pytest.mark.parametrize("case", [c for c in CASES if c[4] == 1])
+def test_attn_split_bf16(case, splits):
+    run_attention_case(splits, torch.bfloat16, *case)
+
+
+@pytest.mark.parametrize("kind", ["rows", "causal", 3])
+def test_attention_window(kind):
+    tq = 1 if kind == 3 else 90
+    run_attention_case(kind, torch.bfloat16, 8, 2, 32, [200, 70, 130], tq, window=70)
+    if kind == "rows":
+        run_attention_case(kind, torch.float32, 8, 2, 32, [200, 70, 130], tq, window=70)
+
+
+# -------------------------------------------------------------------------------------------- gemm
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("m,n,k", [(1, 256, 64), (5, 384, 96), (37, 331, 80), (64, 224, 96), (130, 100, 36), (3, 17, 5)])
+def test_gemm_tiled(dtype, m, n, k):
+    torch.manual_seed(m * n + k)
+    x, w = torch.randn(m, k).to(dtype), torch.randn(n, k).to(dtype)
+    want = x.double() @ w.double().T
+    out = torch.empty(m, n, dtype=dtype, device=DEV)
+    ops().gemm_tiled(x.to(DEV), w.to(DEV), out)
+    close(out, want, dtype, what="gemm_tiled")
+    if dtype == torch.bfloat16:
+        out32 = torch.empty(m, n, dtype=torch.float32, device=DEV)
+        ops().gemm_tiled(x.to(DEV), w.to(DEV), out32)
+        close(out32, want, torch.float32, what="gemm_tiled float32 out")
+
+
+@pytest.mark.parametrize("m", [1, 8, 16, 17, 33, 64])
+@pytest.mark.parametrize("n,k", [(2560, 2560), (384, 96), (331, 80), (256, 9728), (48, 136)])
+@pytest.mark.parametrize("ntw,splits", [(1, 1), (2, 1), (4, 1), (1, 3), (2, 4)])
+def test_gemm_skinny(m, n, k, ntw, splits):
+    torch.manual_seed(m + n + k)
+    x, w = torch.randn(m, k).to(torch.bfloat16), (torch.randn(n, k) / math.sqrt(k)).to(torch.bfloat16)
+    want = x.double() @ w.double().T
+    o = ops()
+    if splits == 1:
+        out = torch.empty(m, n, dtype=torch.float32, device=DEV)
+        o.gemm_skinny_bf16(x.to(DEV), w.to(DEV), out, None, ntw, 1)
+        close(out, want, torch.float32, what="skinny float32 out")
+        outb = torch.empty(m, n, dtype=torch.bfloat16, device=DEV)
+        o.gemm_skinny_bf16(x.to(DEV), w.to(DEV), outb, None, ntw, 1)
+        close(outb, want, torch.bfloat16, ulps=1.0, what="skinny bfloat16 out")
+    else:
+        parts = torch.full((splits, m, n), float("nan"), dtype=torch.float32, device=DEV)
+        o.gemm_skinny_bf16(x.to(DEV), w.to(DEV), None, parts, ntw, splits)
+        out = o.sum_partials(parts, torch.empty(m, n, dtype=torch.float32, device=DEV), splits)
+        close(out, want, torch.float32, what="skinny split-K")
+
+
+def test_linear_dispatch_matches_everywhere():
+    """The same product through every route the linear helper can take."""
+    from dryft_amd.parts.linear import linear
+    from dryft_amd.parts.base import Partials
+    torch.manual_seed(5)
+    w = (torch.randn(384, 96) / 10).to(torch.bfloat16).to(DEV)
+    for m in (1, 7, 64, 65, 300):
+        x = torch.randn(m, 96).to(torch.bfloat16).to(DEV)
+        want = x.double().cpu() @ w.double().cpu().T
+        close(linear(x, w), want, torch.bfloat16, ulps=1.0, what=f"linear m={m}")
+        close(linear(x, w, out_dtype=torch.float32), want, torch.float32, what=f"linear m={m} float32 out")
+        got = linear(x, w, allow_partials=True)
+        if isinstance(got, Partials):
+            got = got.data[: got.count].sum(0)
+        close(got, want, torch.bfloat16, ulps=1.0, what=f"linear partials m={m}")
+        close(linear(x.float(), w.float()), want, torch.float32, what=f"linear float32 m={m}")
+
+
+# ---------------------------------------------------------------------------------------- sampling
+def test_argmax_rows_ties_to_lowest_index():
+    torch.manual_seed(0)
+    logits = torch.randn(5, 151936)
+    logits[0, 777] = logits[0, 150000] = 50.0
+    logits[1, 151935] = 60.0
+    logits[2, 0] = 60.0
+    logits[3, :] = 1.0
+    out = torch.empty(5, dtype=torch.int32, device=DEV)
+    ops().argmax_rows(logits.to(DEV), out)
+    assert out.tolist() == [777, 151935, 0, 0, int(torch.argmax(logits[4]))]
+
+
+@pytest.mark.parametrize("vocab", [331, 151936])
+def test_sample_rows_follows_inverse_cdf(vocab):
+    torch.manual_seed(1)
+    rows, temperature = 64, 0.8
+    logits = 3 * torch.randn(rows, vocab)
+    u = torch.rand(rows)
+    u[0], u[1] = 0.0, 0.999999
+    out = torch.empty(rows, dtype=torch.int32, device=DEV)
+    ops().sample_rows(logits.to(DEV), temperature, u.to(DEV), out)
+    p = torch.softmax(logits.double() / temperature, -1)
+    cdf = torch.cumsum(p, -1)
+    for r, tok in enumerate(out.tolist()):
+        want = min(int(torch.searchsorted(cdf[r], u[r].double(), right=True)), vocab - 1)
+        if tok != want:  # only a draw that falls on a boundary may differ, and then by one place
+            assert float((cdf[r] - u[r].double()).abs().min()) < 1e-5, f"row {r}: got {tok}, want {want}"
+            assert abs(tok - want) <= 1
+
+
+# ------------------------------------------------------------------------------------------- batch
+def test_prepare_batch():
+    o = ops()
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=DEV)
+    lengths = i32([0, 10, 64, 7, 0, 3])
+    seq_slot, q_len = i32([3, -1, 1, 5]), i32([70, 1, 1, 130])
+    n_seqs, n_rows = 4, 202
+    z = lambda n: torch.full((n,), -7, dtype=torch.int32, device=DEV)
+    cu, tiles, kv, start, rseq, rslot, rpos = z(5), z(5), z(4), z(4), z(n_rows), z(n_rows), z(n_rows)
+    o.prepare_batch(seq_slot, q_len, lengths, n_seqs, n_rows, cu, tiles, kv, start, rseq, rslot, rpos)
+    assert cu.tolist() == [0, 70, 71, 72, 202]
+    assert tiles.tolist() == [0, 2, 2, 3, 6]
+    assert kv.tolist() == [77, 0, 11, 133]
+    assert start.tolist() == [7, 0, 10, 3]
+    assert lengths.tolist() == [0, 11, 64, 77, 0, 133]
+    assert rseq.tolist() == [0] * 70 + [1] + [2] + [3] * 130
+    assert rslot.tolist() == [3] * 70 + [-1] + [1] + [5] * 130
+    assert rpos.tolist() == list(range(7, 77)) + [0] + [10] + list(range(3, 133))

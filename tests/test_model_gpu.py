@@ -1,0 +1,386 @@
+"""The engine against the plain implementation, in float32 and in bfloat16: whole requests, the last 32
+tokens one by one, unequal batches whose slots are used again, long decoding, first tokens, generation
+through the entry point, graph replay, and the trace program."""
+
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import (TINY, collect_positions, make_model_dir, max_live_tokens, random_tokens, read_model_dir,
+                     trace_batches, trace_tail, trace_whole)
+from plain import qwen3_plain as plain
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+DTYPES = ["float32", "bfloat16"]
+# Largest allowed |engine - plain| as a fraction of the largest |plain logit| of the request.
+# float32: accumulated float rounding over a few layers (the oracle is float64).
+# bfloat16: activations carry 8 significant bits (2^-9 relative per rounding) through 2-3 layers of
+# about ten rounded tensors each. Models whose weights were sharpened on purpose amplify every rounding;
+# for them the bound is what bfloat16 arithmetic itself does to the plain implementation on the same
+# request (its error against the float64 run, times two), when that is larger.
+TOL = {"float32": 1e-4, "bfloat16": 3e-2}
+LENGTHS = [1, 5, 9, 17, 33, 70, 131, 200]
+
+
+class Case:
+    """A tiny model folder, its plain logits and engines on it."""
+
+    def __init__(self, name, tmp, sharp=False):
+        raw, kw = TINY[name]
+        self.name = name
+        self.dir = make_model_dir(os.path.join(tmp, name + ("_sharp" if sharp else "")), raw, **kw)
+        if sharp:
+            self._sharpen()
+        self.raw, self.weights = read_model_dir(self.dir)
+        self.vocab = raw["vocab_size"]
+        self.requests = {f"r{n}": random_tokens(n, self.vocab, seed=1000 + n) for n in LENGTHS}
+        self._plain = {}
+        self._engines = {}
+
+    def _sharpen(self):
+        """Scale every q_norm weight so that attention is peaked and a lost or misplaced key shows."""
+        from safetensors.torch import load_file, save_file
+        path = os.path.join(self.dir, "model.safetensors")
+        t = load_file(path)
+        for k in t:
+            if k.endswith("q_norm.weight"):
+                t[k] = (t[k].float() * 4.0).to(t[k].dtype)
+        save_file(t, path)
+
+    def plain_logits(self, rid):
+        rid = rid.split("#")[0]          # "r70#2" is request r70 replayed a second time
+        if rid not in self._plain:
+            self._plain[rid] = plain.forward(self.raw, self.weights, self.requests[rid], torch.float64).float()
+        return self._plain[rid]
+
+    def tolerance(self, rid, dtype):
+        """Allowed error as a fraction of the request's largest plain logit."""
+        if dtype == "float32":
+            return TOL[dtype]
+        rid = rid.split("#")[0]
+        key = ("noise", rid)
+        if key not in self._plain:
+            ref = self.plain_logits(rid)
+            low = plain.forward(self.raw, self.weights, self.requests[rid], torch.bfloat16).float()
+            self._plain[key] = float((low - ref).abs().max()) / float(ref.abs().max())
+        return max(TOL[dtype], 2.0 * self._plain[key])
+
+    def engine(self, dtype, **kw):
+        from dryft_amd import Engine
+        key = (dtype, tuple(sorted(kw.items())))
+        if key not in self._engines:
+            args = dict(max_batch=8, max_len=512, use_graph=False)
+            args.update(kw)
+            self._engines[key] = Engine(self.dir, dtype=dtype, **args)
+        return self._engines[key]
+
+
+@pytest.fixture(scope="module")
+def cases(tmp_path_factory):
+    tmp = str(tmp_path_factory.mktemp("models"))
+    out = {n: Case(n, tmp) for n in TINY}
+    out["C_sharp"] = Case("C", tmp, sharp=True)
+    out["A_sharp"] = Case("A", tmp, sharp=True)
+    return out
+
+
+CASE_NAMES = ["A", "B", "C", "C_sharp", "A_sharp"]
+
+
+def replay(engine, records):
+    from dryft_amd.engine.replay import Replayer
+    r = Replayer(engine)
+    outputs = {}
+    for rec in records:
+        logits = r.run_step(rec)
+        if logits is not None and logits.shape[0]:
+            outputs[rec["step"]] = logits.float().cpu()
+    assert not r.slot_of, "every request of the trace must have ended"
+    assert engine.cache.slots.free_count == engine.cache.n_slots, "a slot was lost"
+    for g in engine.cache.kv_groups:
+        assert g.table.pool.free_count == g.table.pool.n_pages, "a page was lost"
+    return outputs
+
+
+def check_against_plain(case, got, dtype, what):
+    assert got, "nothing was compared"
+    worst = 0.0
+    for (rid, pos), row in got.items():
+        ref = case.plain_logits(rid)
+        scale = float(ref.abs().max())
+        err = float((row - ref[pos]).abs().max()) / scale
+        tol = case.tolerance(rid, dtype)
+        assert np.isfinite(err), f"{what}: non-finite logits for {rid} at {pos}"
+        assert err <= tol, f"{what}: {rid} position {pos}: error {err:.3g} of the logit scale > {tol:.3g}"
+        worst = max(worst, err / tol)
+    report = os.environ.get("DRYFT_TEST_REPORT")
+    if report:
+        with open(report, "a") as f:
+            f.write(f"{what} {case.name} {case.dir[-6:]} {dtype}: worst error / tolerance = {worst:.3f}\n")
+    return worst
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", CASE_NAMES)
+def test_whole_requests(cases, name, dtype):
+    case = cases[name]
+    records = list(trace_whole(case.requests))
+    got = collect_positions(records, replay(case.engine(dtype), records))
+    assert len(got) == sum(LENGTHS)
+    check_against_plain(case, got, dtype, "whole")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", CASE_NAMES)
+def test_last_32_tokens_one_by_one(cases, name, dtype):
+    case = cases[name]
+    records = list(trace_tail(case.requests, 32))
+    got = collect_positions(records, replay(case.engine(dtype), records))
+    check_against_plain(case, got, dtype, "tail")
+
+
+def unequal_batches(case):
+    r = case.requests
+    return [
+        {"r5": (r["r5"], 3), "r70": (r["r70"], 40), "r17": (r["r17"], 9), "r1": (r["r1"], 0)},
+        {"r131": (r["r131"], 66), "r9": (r["r9"], 8), "r33": (r["r33"], 2)},
+        {"r200": (r["r200"], 150), "r70#2": (r["r70"], 6), "r5#2": (r["r5"], 4), "r17#2": (r["r17"], 16),
+         "r33#2": (r["r33"], 32)},
+    ]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", CASE_NAMES)
+def test_unequal_batches_reuse_slots(cases, name, dtype):
+    case = cases[name]
+    engine = case.engine(dtype)
+    records = list(trace_batches(unequal_batches(case)))
+    got = collect_positions(records, replay(engine, records))
+    check_against_plain(case, got, dtype, "batches")
+    # the same trace again on the same engine: slots and pages now hold stale bytes of other requests
+    again = collect_positions(records, replay(engine, records))
+    for key in got:
+        assert torch.equal(got[key], again[key]), f"second run differs at {key} (stale state)"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_alone_and_in_a_batch_agree(cases, dtype):
+    """What else is in the batch changes a request's logits by rounding at most."""
+    case = cases["C_sharp"]
+    engine = case.engine(dtype)
+    alone = list(trace_batches([{"r70": (case.requests["r70"], 40)}]))
+    a = collect_positions(alone, replay(engine, alone))
+    batch = list(trace_batches([unequal_batches(case)[0]]))
+    b = collect_positions(batch, replay(engine, batch))
+    tol = 1e-5 if dtype == "float32" else 2e-2
+    for key, row in a.items():
+        scale = float(row.abs().max())
+        assert float((row - b[key]).abs().max()) <= tol * scale, f"{key} depends on the rest of the batch"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["B", "C_sharp"])
+def test_long_decoding_crosses_pages(cases, name, dtype):
+    case = cases[name]
+    toks = case.requests["r200"]
+    records = list(trace_batches([{"r200": (toks, 197)}]))     # 3 tokens start, 197 follow one by one
+    got = collect_positions(records, replay(case.engine(dtype), records))
+    assert len(got) == 198
+    check_against_plain(case, got, dtype, "long decoding")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_first_tokens(cases, name, dtype):
+    """A sequence that starts with a single token, then grows one by one: positions 0, 1, 2, ..."""
+    case = cases[name]
+    toks = case.requests["r9"]
+    records = [{"step": 0, "entries": [{"id": "r9", "tokens": toks[:1], "want": [0]}], "end": []}]
+    for i in range(1, len(toks)):
+        records.append({"step": i, "entries": [{"id": "r9", "tokens": [toks[i]], "want": [0]}],
+                        "end": ["r9"] if i == len(toks) - 1 else []})
+    got = collect_positions(records, replay(case.engine(dtype), records))
+    check_against_plain(case, got, dtype, "first tokens")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_stale_cache_bytes_are_never_read(cases, dtype):
+    """Fill every page with large finite garbage before a run: lengths and tables alone say what is valid."""
+    case = cases["B"]
+    engine = case.engine(dtype, max_batch=4, max_len=256)
+    for g in engine.cache.kv_groups:
+        g.k.fill_(3e4)
+        g.v.fill_(-3e4)
+    records = list(trace_batches([{"r70": (case.requests["r70"], 30), "r9": (case.requests["r9"], 3)}]))
+    got = collect_positions(records, replay(engine, records))
+    check_against_plain(case, got, dtype, "poisoned cache")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_device_lengths_follow_host(cases, dtype):
+    case = cases["A"]
+    engine = case.engine(dtype)
+    from dryft_amd.engine.step import SeqStep
+    slots = engine.acquire(3)
+    engine.step([SeqStep(slots[0], [1, 2, 3], []), SeqStep(slots[1], [4], [0]), SeqStep(slots[2], list(range(70)), [])])
+    engine.step([SeqStep(slots[0], [5], [0]), SeqStep(-1, [0], []), SeqStep(slots[2], [7], [])])
+    host = engine.cache.lengths_host()
+    assert [int(host[s]) for s in slots] == [4, 1, 71]
+    assert engine.cache.lengths_dev.cpu().tolist() == [int(x) for x in host]
+    engine.release(slots)
+    assert not engine.cache.lengths_dev.any()
+
+
+# ------------------------------------------------------------------------------------ generation
+def plain_generation(case, prompt, n, temperature=0.0, uniforms=None):
+    if temperature == 0.0:
+        return plain.generate(case.raw, case.weights, prompt, n, dtype=torch.float64)
+    choose = lambda logits, t: plain.sample_with_temperature(logits, temperature, float(uniforms[t]))
+    return plain.generate(case.raw, case.weights, prompt, n, choose=choose, dtype=torch.float64)
+
+
+def check_generation(case, prompts, ours, n, dtype, temperature=0.0, uniforms=None):
+    """Tokens must equal the plain loop's unless the plain logits leave the choice open within rounding."""
+    for b, prompt in enumerate(prompts):
+        col = [step[b] for step in ours]
+        u = None if uniforms is None else [float(uniforms[t][b]) for t in range(n)]
+        want, logits = plain_generation(case, prompt, n, temperature, u)
+        for t in range(n):
+            if col[t] == want[t]:
+                continue
+            if temperature == 0.0:
+                margin = float(logits[t].max() - logits[t][col[t]])
+                slack = TOL[dtype] * float(logits[t].abs().max()) * 2
+                assert margin <= slack, f"seq {b} step {t}: chose {col[t]}, plain {want[t]}, margin {margin}"
+            else:
+                assert plain.cdf_margin(logits[t], temperature, u[t]) < (1e-5 if dtype == "float32" else 2e-2), \
+                    f"seq {b} step {t}: sampled {col[t]}, plain {want[t]}"
+            break   # after a justified divergence the continuations differ
+
+
+@pytest.mark.parametrize("use_graph", [False, True])
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_greedy_generation_config_a(cases, dtype, use_graph):
+    """Tiny A's workload: prompts of 5, 9 and 17 tokens, 8 greedy steps."""
+    case = cases["A"]
+    prompts = [random_tokens(n, case.vocab, seed=n) for n in (5, 9, 17)]
+    engine = case.engine(dtype, use_graph=use_graph)
+    ours = list(engine.generate(prompts, 8))
+    assert len(ours) == 8 and all(len(s) == 3 and all(isinstance(t, int) for t in s) for s in ours)
+    check_generation(case, prompts, ours, 8, dtype)
+    assert list(engine.generate(prompts, 8)) == ours, "second run differs from the first"
+
+
+@pytest.mark.parametrize("use_graph", [False, True])
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_generation_config_b_greedy_and_temperature(cases, dtype, use_graph):
+    """Tiny B's workload: prompts of 1, 6, 13 and 31 tokens, 12 steps, greedy and temperature 0.8."""
+    case = cases["B"]
+    prompts = [random_tokens(n, case.vocab, seed=50 + n) for n in (1, 6, 13, 31)]
+    engine = case.engine(dtype, use_graph=use_graph)
+    ours = list(engine.generate(prompts, 12))
+    check_generation(case, prompts, ours, 12, dtype)
+    sampled = list(engine.generate(prompts, 12, temperature=0.8, sample_seed=7))
+    gen = torch.Generator().manual_seed(7)
+    uniforms = [torch.rand(4, generator=gen, dtype=torch.float32) for _ in range(12)]
+    check_generation(case, prompts, sampled, 12, dtype, 0.8, uniforms)
+    assert sampled != ours
+    assert list(engine.generate(prompts, 12, temperature=0.8, sample_seed=7)) == sampled
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_small_batch_unchanged_after_a_big_one(cases, dtype):
+    case = cases["B"]
+    engine = case.engine(dtype, use_graph=True)
+    small = [random_tokens(11, case.vocab, seed=3)]
+    big = [random_tokens(n, case.vocab, seed=60 + n) for n in (40, 3, 19, 64, 65, 7, 100, 2)]
+    a = list(engine.generate(small, 6))
+    list(engine.generate(big, 9))
+    assert list(engine.generate(small, 6)) == a, "state leaked from the larger batch"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_stop_tokens_and_more_requests_than_slots(cases, dtype):
+    case = cases["A"]
+    engine = case.engine(dtype, max_batch=3, max_len=128, use_graph=True)
+    prompts = [random_tokens(n, case.vocab, seed=80 + n) for n in (4, 9, 2, 30, 7, 12, 5)]
+    free_run = engine.generate_all(prompts, 10)
+    assert [len(r) for r in free_run] == [10] * 7
+    stop = free_run[1][3]
+    stopped = engine.generate_all(prompts, 10, stop_token_ids=[stop])
+    for full, cut in zip(free_run, stopped):
+        want = full[: full.index(stop) + 1] if stop in full else full
+        assert cut == want
+    steps = list(engine.generate(prompts[:3], 10, stop_token_ids=[stop]))
+    assert all(len(s) == 3 for s in steps)
+    for b in range(3):
+        col = [s[b] for s in steps]
+        cut = stopped[b]
+        assert col[: len(cut)] == cut and all(t == -1 for t in col[len(cut):])
+    assert engine.cache.slots.free_count == 3
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_graph_replay_equals_eager(cases, dtype):
+    """A captured decoding step gives bit-identical logits to the same step run eagerly."""
+    case = cases["B"]
+    from dryft_amd.engine.graph import DecodeGraph
+    from dryft_amd.engine.step import SeqStep
+    engine = case.engine(dtype, max_batch=4, max_len=256)
+    prompts = [random_tokens(n, case.vocab, seed=90 + n) for n in (70, 3, 129)]
+    nxt = [random_tokens(5, case.vocab, seed=95 + i) for i in range(3)]
+    graph = DecodeGraph(engine.stepper, 3)
+    graph.capture()
+    results = []
+    for mode in ("eager", "graph", "graph", "eager"):
+        slots = engine.acquire(3)
+        engine.step([SeqStep(s, p, []) for s, p in zip(slots, prompts)])
+        outs = []
+        for t in range(5):
+            live = [s if not (t >= 3 and i == 1) else -1 for i, s in enumerate(slots)]   # one ends early
+            toks = [nxt[i][t] for i in range(3)]
+            if mode == "eager":
+                lg = engine.step([SeqStep(s, [tk], [0]) for s, tk in zip(live, toks)])
+                keep = [i for i, s in enumerate(live) if s >= 0]
+            else:
+                held = [s for s in live if s >= 0]
+                engine.cache.begin_step(held, [1] * len(held))
+                lg = graph.replay(live, toks)
+                engine.cache.end_step(held, [1] * len(held))
+                keep = [i for i, s in enumerate(live) if s >= 0]
+                lg = lg[keep]
+            outs.append(lg.float().cpu().clone())
+        engine.release(slots)
+        results.append(outs)
+    for other in results[1:]:
+        for a, b in zip(results[0], other):
+            assert torch.equal(a, b), "graph replay differs from eager"
+
+
+# --------------------------------------------------------------------------------- the program
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_trace_run_program(cases, dtype, tmp_path):
+    case = cases["B"]
+    records = list(trace_batches(unequal_batches(case)))
+    out_dir = str(tmp_path / "out")
+    cmd = [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", case.dir, "--dtype", dtype, "--out",
+           out_dir, "--max-tokens", str(max_live_tokens(records))]
+    feed = "".join(json.dumps(r) + "\n" for r in records)
+    proc = subprocess.run(cmd, input=feed, capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert proc.stdout.split("\n")[:-1] == [f"done {r['step']}" for r in records]
+    outputs = {}
+    for r in records:
+        n_want = sum(len(e["want"]) for e in r["entries"])
+        path = os.path.join(out_dir, f"{r['step']}.f32")
+        if n_want:
+            outputs[r["step"]] = torch.from_numpy(np.fromfile(path, dtype="<f4").reshape(n_want, case.vocab))
+        else:
+            assert not os.path.exists(path)
+    check_against_plain(case, collect_positions(records, outputs), dtype, "trace_run")
