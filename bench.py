@@ -1,0 +1,161 @@
+"""Decode and prefill throughput of the Qwen3 engine on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--preset qwen3-4b] [--batch 8] [--layers L]
+
+The workload is the one named for the reference's headline metric: Qwen3-4B layer sizes with
+random weights in bfloat16, prompts of 2,048 uniform random token ids in 4,096-token cache
+slots, greedy decoding. A step is one decode step of the whole batch through the generation
+machinery (graph replay, token choice, token hand-back). One JSON line is printed:
+decoded tokens per second at the main batch size, the prefill rate of one 2,048-token prompt
+with its fraction of the bf16 matrix-core peak, the decode step's fraction of the HBM
+roofline, and decode rates at batch 1 and 64. Timing protocol after the reference's harness
+(agent/bench.py:96-126): untimed warm-up, synchronise on both sides of the timed region.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X: 8 TB/s
+PEAK_FLOPS = {"bf16": 2.5e15, "fp16": 2.5e15, "fp8": 5.0e15, "fp32": 157.3e12}
+PROMPT, SLOT = 2048, 4096
+
+
+def matmul_params(cfg) -> tuple[int, int]:
+    """(weights of one layer's matrix products, weights of the output head)."""
+    per_layer = (cfg.q_dim + 2 * cfg.kv_dim) * cfg.hidden_size + cfg.hidden_size * cfg.q_dim \
+        + 3 * cfg.intermediate_size * cfg.hidden_size
+    return per_layer, cfg.vocab_size * cfg.hidden_size
+
+
+def decode_bytes(cfg, layers: int, batch: int, context: float, elem: int = 2) -> float:
+    """What a decode step has to read: every weight it uses once, and the cache of the live requests."""
+    per_layer, head = matmul_params(cfg)
+    norms = layers * (2 * cfg.hidden_size + 2 * cfg.head_dim) + cfg.hidden_size
+    weights = (layers * per_layer + head + norms) * elem
+    kv = batch * context * layers * 2 * cfg.kv_dim * elem
+    return weights + kv
+
+
+def prefill_flops(cfg, layers: int, tokens: int) -> float:
+    per_layer, head = matmul_params(cfg)
+    linear = 2.0 * tokens * layers * per_layer + 2.0 * head          # the head runs on the last row only
+    attention = layers * 2.0 * tokens * tokens * cfg.q_dim            # QK^T and PV, causal half of each
+    return linear + attention
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--preset", default="qwen3-4b")
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--layers", type=int, default=None, help="run fewer layers than the preset has")
+    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and batch 64 points")
+    ap.add_argument("--no-graph", action="store_true")
+    ap.add_argument("--seed", type=int, default=0)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU only (asked for {args.gpus}); this library has no multi-GPU path")
+        return 2
+
+    import numpy as np
+    import torch
+
+    from dryft_amd import Engine
+    from dryft_amd.models.qwen3 import load_preset
+
+    raw = dict(load_preset(args.preset))
+    full_layers = raw["num_hidden_layers"]
+    if args.layers:
+        raw["num_hidden_layers"] = args.layers
+    layers = raw["num_hidden_layers"]
+    max_batch = args.batch if args.no_points else max(args.batch, 64)
+    engine = Engine(config=raw, seed=args.seed, dtype=args.dtype, max_batch=max_batch, max_len=SLOT,
+                    use_graph=not args.no_graph, verbose=True)
+    cfg = engine.config
+    elem = 2 if args.dtype == "bfloat16" else 4
+    rng = np.random.default_rng(args.seed)
+
+    def prompts(b):
+        return [[int(t) for t in rng.integers(0, cfg.vocab_size, size=PROMPT)] for _ in range(b)]
+
+    def sync():
+        torch.cuda.synchronize()
+
+    def decode_rate(batch: int, steps: int, warmup: int):
+        """(tokens/s, ms per step, mean context) for `steps` decode steps after a 2,048-token prefill."""
+        slots = engine.acquire(batch)
+        try:
+            engine.reserve(slots, [PROMPT + warmup + steps + 1] * batch)
+            tokens = engine.start(slots, prompts(batch), 0)
+            for i in range(warmup):
+                tokens = engine.advance(slots, tokens, 1 + i)
+            sync()
+            t0 = time.perf_counter()
+            for i in range(steps):
+                tokens = engine.advance(slots, tokens, 1 + warmup + i)
+            sync()
+            dt = time.perf_counter() - t0
+        finally:
+            engine.release(slots)
+        context = PROMPT + warmup + (steps + 1) / 2.0
+        return batch * steps / dt, dt / steps * 1e3, context
+
+    def prefill_rate(repeats: int = 3):
+        best = None
+        for _ in range(repeats + 1):                       # the first run warms libraries up
+            slots = engine.acquire(1)
+            p = prompts(1)
+            sync()
+            t0 = time.perf_counter()
+            engine.start(slots, p, 0)
+            sync()
+            dt = time.perf_counter() - t0
+            engine.release(slots)
+            best = dt if best is None else min(best, dt)
+        return PROMPT / best, best * 1e3
+
+    tok_s, ms_step, context = decode_rate(args.batch, args.steps, args.warmup)
+    need = decode_bytes(cfg, layers, args.batch, context, elem)
+    achieved = need / (ms_step * 1e-3) / 1e9
+    pf_tok_s, pf_ms = prefill_rate()
+    peak = PEAK_FLOPS["bf16" if args.dtype == "bfloat16" else "fp32"]
+    pf_frac = prefill_flops(cfg, layers, PROMPT) / (pf_ms * 1e-3) / peak
+    points = {}
+    if not args.no_points:
+        for b in (1, 64):
+            points[f"decode_b{b}"] = round(decode_rate(b, max(16, args.steps // 2), max(4, args.warmup // 2))[0], 1)
+    line = {
+        "metric": "decode tok/s (Qwen3-4B layer sizes, 2,048-token prompts, 4,096-token slots)",
+        "value": round(tok_s, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic (random weights, uniform random token ids)",
+        "config": {
+            "model": args.preset, "global_batch": args.batch, "seq_len": SLOT, "prompt_len": PROMPT,
+            "parallelism": "none", "layers": layers, "layers_of_model": full_layers, "hidden_size": cfg.hidden_size,
+            "num_attention_heads": cfg.num_attention_heads, "num_key_value_heads": cfg.num_key_value_heads,
+            "head_dim": cfg.head_dim, "intermediate_size": cfg.intermediate_size, "vocab_size": cfg.vocab_size,
+            "rope_theta": cfg.rope_theta, "rms_norm_eps": cfg.rms_norm_eps,
+            "tie_word_embeddings": cfg.tie_word_embeddings, "graph": not args.no_graph,
+        },
+        "prefill": {"value": round(pf_tok_s, 1), "tokens": PROMPT, "ms": round(pf_ms, 3), "frac": round(pf_frac, 4)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4)},
+        "points": points,
+    }
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
