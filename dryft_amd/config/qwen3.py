@@ -53,13 +53,16 @@ class Qwen3Config:
         hidden = r.integer("hidden_size")
         heads = r.integer("num_attention_heads")
         kv_heads = r.integer("num_key_value_heads", default=heads if heads else 1)
-        head_dim = raw.get("head_dim") or (hidden // heads if heads else 0)
+        if raw.get("head_dim"):
+            head_dim = r.integer("head_dim")
+        else:                                        # absent, null or 0: config.py:142 of the reference
+            head_dim = hidden // heads if heads else 0
         cfg = cls(
             num_hidden_layers=r.integer("num_hidden_layers"),
             hidden_size=hidden,
             num_attention_heads=heads,
             num_key_value_heads=kv_heads,
-            head_dim=r.integer("head_dim", default=head_dim),
+            head_dim=head_dim,
             intermediate_size=r.integer("intermediate_size"),
             vocab_size=r.integer("vocab_size"),
             rms_norm_eps=r.number("rms_norm_eps"),

@@ -15,7 +15,7 @@ import numpy as np
 import torch
 
 from ..parts.base import StepContext
-from .step import BatchBuffers, Stepper
+from .step import BatchBuffers, Stepper, make_context
 
 
 class DecodeGraph:
@@ -24,8 +24,8 @@ class DecodeGraph:
         dev = stepper.device
         self.buf = BatchBuffers(self.batch, self.batch, dev)
         self.buf.q_len.fill_(1)
-        self.ctx: StepContext = stepper.context(self.buf, self.batch, self.batch, max_q_len=1, max_tiles=self.batch,
-                                                max_kv_len=stepper.cache.max_len, host=None)
+        self.ctx: StepContext = make_context(self.buf, self.batch, self.batch, stepper.model.dtype, max_q_len=1,
+                                             max_tiles=self.batch, max_kv_len=stepper.cache.max_len, host=None)
         self.logits: torch.Tensor | None = None
         self.graph: torch.cuda.CUDAGraph | None = None
         self._stage = torch.zeros(2 * self.batch, dtype=torch.int32).pin_memory()

@@ -49,6 +49,54 @@ class BatchBuffers:
         self.seq_start = torch.zeros(max_seqs, **i32)
 
 
+def stage_batch(cache: CacheStore, buf: BatchBuffers, slots: list[int], q_lens: list[int], tokens,
+                dtype: torch.dtype) -> StepContext:
+    """Host side of a step: room in the cache, the step's facts on the device, rows derived from them.
+
+    ``slots[i] == -1`` marks a sequence that sits out; its ``q_lens[i]`` rows are dead. Advances the
+    device's copy of the lengths; the caller records the same on the host with ``cache.end_step``
+    once the model has run.
+    """
+    device = buf.tokens.device
+    live = [(s, q) for s, q in zip(slots, q_lens) if s >= 0]
+    live_slots, live_q = [s for s, _ in live], [q for _, q in live]
+    if len(set(live_slots)) != len(live_slots):
+        raise ValueError("a slot appears twice in one step")
+    starts_live = cache.begin_step(live_slots, live_q)
+    start_of = dict(zip(live_slots, starts_live))
+    starts = [start_of.get(s, 0) for s in slots]
+    n_rows, n_seqs = int(sum(q_lens)), len(slots)
+    if n_rows > buf.max_rows or n_seqs > buf.max_seqs:
+        raise ValueError(f"step of {n_rows} rows / {n_seqs} sequences exceeds the buffers ({buf.max_rows} / {buf.max_seqs})")
+    # one staging array, one copy: tokens | seq_slot | q_len
+    stage = torch.from_numpy(np.concatenate([np.asarray(tokens, dtype=np.int32), np.asarray(slots, dtype=np.int32),
+                                             np.asarray(q_lens, dtype=np.int32)])).to(device)
+    buf.tokens[:n_rows].copy_(stage[:n_rows])
+    buf.seq_slot[:n_seqs].copy_(stage[n_rows:n_rows + n_seqs])
+    buf.q_len[:n_seqs].copy_(stage[n_rows + n_seqs:])
+    ctx = make_context(buf, n_rows, n_seqs, dtype, max_q_len=max(q_lens),
+                       max_tiles=sum((q + 63) // 64 for q in live_q),
+                       max_kv_len=max([st + q for st, q in zip(starts_live, live_q)], default=0),
+                       host=HostBatch(list(slots), list(q_lens), starts))
+    derive_rows(cache, buf, ctx)
+    return ctx
+
+
+def make_context(buf: BatchBuffers, n_rows: int, n_seqs: int, dtype: torch.dtype, *, max_q_len: int, max_tiles: int,
+                 max_kv_len: int, host: HostBatch | None) -> StepContext:
+    return StepContext(n_rows=n_rows, n_seqs=n_seqs, dtype=dtype, device=buf.tokens.device,
+                       row_seq=buf.row_seq, row_slot=buf.row_slot, row_pos=buf.row_pos, cu_rows=buf.cu_rows,
+                       tile_cu=buf.tile_cu, seq_slot=buf.seq_slot, q_len=buf.q_len, kv_len=buf.kv_len,
+                       seq_start=buf.seq_start, max_q_len=max_q_len, max_tiles=max_tiles, max_kv_len=max_kv_len,
+                       host=host)
+
+
+def derive_rows(cache: CacheStore, buf: BatchBuffers, ctx: StepContext) -> None:
+    """Per-row facts from per-sequence facts, on the device; advances the device's lengths."""
+    ops.prepare_batch(buf.seq_slot, buf.q_len, cache.lengths_dev, ctx.n_seqs, ctx.n_rows, buf.cu_rows,
+                      buf.tile_cu, buf.kv_len, buf.seq_start, buf.row_seq, buf.row_slot, buf.row_pos)
+
+
 class Stepper:
     """Owns a model and its cache and runs steps on them."""
 
@@ -71,14 +119,8 @@ class Stepper:
         """Runs the step and returns float32 logits ``[sum(len(want)), vocab]`` in order."""
         if not seqs:
             return torch.empty((0, self.vocab), dtype=torch.float32, device=self.device)
-        slots = [s.slot for s in seqs]
-        q_lens = [len(s.tokens) for s in seqs]
-        live = [s for s in seqs if s.slot >= 0]
-        if len({s.slot for s in live}) != len(live):
-            raise ValueError("a slot appears twice in one step")
         tokens: list[int] = []
         wanted: list[int] = []
-        base = 0
         for s in seqs:
             if not s.tokens:
                 raise ValueError("a sequence in a step must bring at least one token")
@@ -86,47 +128,23 @@ class Stepper:
                 if not 0 <= w < len(s.tokens):
                     raise ValueError(f"wanted place {w} is outside the {len(s.tokens)} tokens given")
                 if s.slot >= 0:
-                    wanted.append(base + w)
+                    wanted.append(len(tokens) + w)
             tokens.extend(s.tokens)
-            base += len(s.tokens)
         tok = np.asarray(tokens, dtype=np.int64)
-        if tok.size and (tok.min() < 0 or tok.max() >= self.vocab):
+        if tok.min() < 0 or tok.max() >= self.vocab:
             raise ValueError(f"token ids must lie in [0, {self.vocab}); got {int(tok.min())}..{int(tok.max())}")
-        live_slots = [s.slot for s in live]
-        live_q = [len(s.tokens) for s in live]
-        starts_live = self.cache.begin_step(live_slots, live_q)
-        start_of = dict(zip(live_slots, starts_live))
-        starts = [start_of.get(s, 0) for s in slots]
-        n_rows, n_seqs = len(tokens), len(seqs)
-        buf = self._buffers_for(n_rows, n_seqs)
-        # one staging array, one copy: tokens | seq_slot | q_len
-        stage = torch.from_numpy(np.concatenate([tok.astype(np.int32), np.asarray(slots, dtype=np.int32),
-                                                 np.asarray(q_lens, dtype=np.int32)])).to(self.device)
-        buf.tokens[:n_rows].copy_(stage[:n_rows])
-        buf.seq_slot[:n_seqs].copy_(stage[n_rows:n_rows + n_seqs])
-        buf.q_len[:n_seqs].copy_(stage[n_rows + n_seqs:])
-        ctx = self.context(buf, n_rows, n_seqs,
-                           max_q_len=max(q_lens),
-                           max_tiles=sum((q + 63) // 64 for q in live_q),
-                           max_kv_len=max([st + q for st, q in zip(starts_live, live_q)], default=0),
-                           host=HostBatch(slots, q_lens, starts))
-        hidden = self.run(buf, ctx)
-        self.cache.end_step(live_slots, live_q)
+        slots = [s.slot for s in seqs]
+        q_lens = [len(s.tokens) for s in seqs]
+        buf = self._buffers_for(len(tokens), len(seqs))
+        ctx = stage_batch(self.cache, buf, slots, q_lens, tok, self.model.dtype)
+        hidden = self.model.forward(buf.tokens[:ctx.n_rows], ctx, self.cache)
+        self.cache.end_step([s for s in slots if s >= 0], [q for s, q in zip(slots, q_lens) if s >= 0])
         if not wanted:
             return torch.empty((0, self.vocab), dtype=torch.float32, device=self.device)
         rows = torch.tensor(wanted, dtype=torch.int32, device=self.device)
         return self.model.logits(hidden, rows)
 
-    def context(self, buf: BatchBuffers, n_rows: int, n_seqs: int, *, max_q_len: int, max_tiles: int,
-                max_kv_len: int, host: HostBatch | None) -> StepContext:
-        return StepContext(n_rows=n_rows, n_seqs=n_seqs, dtype=self.model.dtype, device=self.device,
-                           row_seq=buf.row_seq, row_slot=buf.row_slot, row_pos=buf.row_pos, cu_rows=buf.cu_rows,
-                           tile_cu=buf.tile_cu, seq_slot=buf.seq_slot, q_len=buf.q_len, kv_len=buf.kv_len,
-                           seq_start=buf.seq_start, max_q_len=max_q_len, max_tiles=max_tiles, max_kv_len=max_kv_len,
-                           host=host)
-
     def run(self, buf: BatchBuffers, ctx: StepContext) -> torch.Tensor:
-        """The device work of a step: row facts from sequence facts, then the model."""
-        ops.prepare_batch(buf.seq_slot, buf.q_len, self.cache.lengths_dev, ctx.n_seqs, ctx.n_rows, buf.cu_rows,
-                          buf.tile_cu, buf.kv_len, buf.seq_start, buf.row_seq, buf.row_slot, buf.row_pos)
+        """The device work of a step whose facts already sit in ``buf`` (what a captured graph holds)."""
+        derive_rows(self.cache, buf, ctx)
         return self.model.forward(buf.tokens[:ctx.n_rows], ctx, self.cache)

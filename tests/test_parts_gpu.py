@@ -1,0 +1,410 @@
+"""Each part alone against the plain implementation, and the generality of their arrangement: a toy mixer
+with state of its own, registered from here; a layer named twice; a run that reads another run's cache."""
+
+import math
+import os
+from dataclasses import dataclass
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import TINY_B, random_tokens
+from plain import qwen3_plain as P
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+def tol(ref, dtype, ulps=4.0):
+    return (ulps * 2.0 ** -8 if dtype == torch.bfloat16 else 2e-5) * float(ref.abs().max()) + 1e-6
+
+
+def close(got, want, dtype, what, ulps=4.0):
+    diff = float((got.float().cpu() - want.float()).abs().max())
+    assert diff <= tol(want, dtype, ulps), f"{what}: {diff} > {tol(want, dtype, ulps)}"
+
+
+def load_part(part, tensors, dtype):
+    from dryft_amd.weights.spec import VECTOR
+    part.load({k: v.to(DEV).to(dtype) for k, v in tensors.items()})
+    return part
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_rmsnorm_part(dtype):
+    from dryft_amd.parts.norm import RMSNorm
+    from dryft_amd.parts.base import Partials
+    torch.manual_seed(0)
+    w = (1 + 0.1 * torch.randn(100)).to(dtype)
+    x, d = torch.randn(9, 100).to(dtype), torch.randn(9, 100).to(dtype)
+    norm = load_part(RMSNorm(100, 1e-5), {"weight": w}, dtype)
+    assert norm.tensor_specs() == {"weight": ((100,), "vector", "ones")}
+    close(norm.forward(x.to(DEV)), P.rms_norm(x.double(), w.double(), 1e-5), dtype, "norm")
+    res, y = norm.add_forward(x.to(DEV).clone(), d.to(DEV))
+    s = (x.float() + d.float()).to(dtype)
+    assert torch.equal(res.cpu(), s)
+    close(y, P.rms_norm(s.double(), w.double(), 1e-5), dtype, "add + norm")
+    parts = torch.randn(2, 9, 100)
+    res, y = norm.add_forward(x.to(DEV).clone(), Partials(parts.to(DEV), 2))
+    s = (x.float() + parts.sum(0)).to(dtype)
+    close(res, s, dtype, "add partials", ulps=1.0)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_rotary_tables(dtype):
+    from dryft_amd.parts.rope import RotaryPositions
+    rot = RotaryPositions(48, 5e6)
+    rot.prepare(300, dtype, DEV)
+    cos, sin = P.rope_tables(48, 5e6, 300)
+    assert torch.equal(rot.cos.cpu(), cos[:, :24].to(dtype)) and torch.equal(rot.sin.cpu(), sin[:, :24].to(dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_swiglu_part(dtype):
+    from dryft_amd.parts.mlp import SwiGLU
+    from dryft_amd.parts.base import Partials
+    torch.manual_seed(1)
+    w = {"gate_proj": torch.randn(136, 80) / 9, "up_proj": torch.randn(136, 80) / 9, "down_proj": torch.randn(80, 136) / 12}
+    w = {k: v.to(dtype) for k, v in w.items()}
+    ffn = load_part(SwiGLU(80, 136), w, dtype)
+    for rows in (1, 7, 100):
+        h = torch.randn(rows, 80).to(dtype)
+        out = ffn.forward(h.to(DEV), None)
+        if isinstance(out, Partials):
+            out = out.data[: out.count].sum(0)
+        want = P.swiglu(h.double(), {"mlp." + k + ".weight": v.double() for k, v in w.items()}, "")
+        close(out, want, dtype, f"swiglu rows={rows}")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_embedding_and_head_parts(dtype):
+    from dryft_amd.parts.embedding import LMHead, TokenEmbedding
+    torch.manual_seed(2)
+    table = torch.randn(331, 80).to(dtype)
+    emb = load_part(TokenEmbedding(331, 80), {"weight": table}, dtype)
+    toks = torch.tensor([0, 330, 7, 7], dtype=torch.int32)
+    assert torch.equal(emb.forward(toks.to(DEV)).cpu(), table[toks.long()])
+    head = LMHead(331, 80, tied=True)
+    assert head.tensor_specs() == {}
+    head.tie(emb.weight)
+    h = torch.randn(5, 80).to(dtype)
+    logits = head.forward(h.to(DEV))
+    assert logits.dtype == torch.float32
+    close(logits, h.double() @ table.double().T, torch.float32 if dtype == torch.float32 else dtype, "tied head", ulps=0.5)
+    own = load_part(LMHead(331, 80, tied=False), {"weight": table * 2}, dtype)
+    close(own.forward(h.to(DEV)), 2 * (h.double() @ table.double().T), torch.float32 if dtype == torch.float32 else dtype,
+          "own head", ulps=0.5)
+
+
+def attention_setup(dtype, n_heads, n_kv, d, hidden, window=None, rotary=True, norm=True):
+    from dryft_amd.cache import CacheStore
+    from dryft_amd.parts.attention import GQAAttention
+    from dryft_amd.parts.rope import RotaryPositions
+    torch.manual_seed(n_heads * d)
+    att = GQAAttention(hidden, n_heads, n_kv, d, qk_norm_eps=1e-6 if norm else None,
+                       positions="rotary" if rotary else None, window=window)
+    w = {"q_proj": torch.randn(n_heads * d, hidden) / 6, "k_proj": torch.randn(n_kv * d, hidden) / 6,
+         "v_proj": torch.randn(n_kv * d, hidden) / 6, "o_proj": torch.randn(hidden, n_heads * d) / 8}
+    if norm:
+        w["q_norm"] = 1 + 0.2 * torch.randn(d)
+        w["k_norm"] = 1 + 0.2 * torch.randn(d)
+    w = {k: v.to(dtype) for k, v in w.items()}
+    load_part(att, w, dtype)
+    cache = CacheStore({0: att.cache_need()}, max_tokens=64 * 12, n_slots=4, max_len=320, dtype=dtype, device=DEV)
+    rot = RotaryPositions(d, 1e4)
+    rot.prepare(320, dtype, DEV)
+    return att, w, cache, {"rotary": rot}
+
+
+def plain_attention(h, w, n_heads, n_kv, d, window=None, rotary=True, norm=True):
+    T = h.shape[0]
+    w = {k: v.double() for k, v in w.items()}
+    q = (h @ w["q_proj"].T).view(T, n_heads, d)
+    k = (h @ w["k_proj"].T).view(T, n_kv, d)
+    v = (h @ w["v_proj"].T).view(T, n_kv, d)
+    if norm:
+        q, k = P.rms_norm(q, w["q_norm"], 1e-6), P.rms_norm(k, w["k_norm"], 1e-6)
+    if rotary:
+        cos, sin = P.rope_tables(d, 1e4, T, torch.float64)
+        q, k = P.apply_rope(q, cos, sin), P.apply_rope(k, cos, sin)
+    return P.causal_gqa_attention(q, k, v, 1 / math.sqrt(d), window).reshape(T, -1) @ w["o_proj"].T
+
+
+def run_mixer(att, cache, positions, dtype, seqs, cuts):
+    """Feed each sequence's rows of hidden states through the mixer in steps cut at ``cuts``."""
+    from dryft_amd.engine.step import BatchBuffers, stage_batch
+    from dryft_amd.parts.base import Partials
+    slots = cache.acquire(len(seqs))
+    buf = BatchBuffers(1024, 8, DEV)
+    outs = [[] for _ in seqs]
+    edges = [0] + list(cuts) + [max(len(s) for s in seqs)]
+    for a, b in zip(edges[:-1], edges[1:]):
+        live = [(i, s[a:b]) for i, s in enumerate(seqs) if len(s[a:b])]
+        if not live:
+            continue
+        q_lens = [len(x) for _, x in live]
+        ctx = stage_batch(cache, buf, [slots[i] for i, _ in live], q_lens, [0] * sum(q_lens), dtype)
+        ctx.positions = positions
+        h = torch.cat([x for _, x in live]).to(DEV)
+        out = att.forward(h, ctx, cache.line(0), True)
+        if isinstance(out, Partials):
+            out = out.data[: out.count].sum(0)
+        cache.end_step([slots[i] for i, _ in live], q_lens)
+        at = 0
+        for (i, x) in live:
+            outs[i].append(out[at: at + len(x)].float().cpu())
+            at += len(x)
+    cache.release(slots)
+    return [torch.cat(o) for o in outs]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape", [(6, 3, 48, 80), (4, 1, 16, 64), (8, 8, 32, 96)])
+@pytest.mark.parametrize("variant", ["qwen3", "window", "bare"])
+def test_attention_part_alone(dtype, shape, variant):
+    n_heads, n_kv, d, hidden = shape
+    kw = {"qwen3": {}, "window": {"window": 70}, "bare": {"rotary": False, "norm": False}}[variant]
+    att, w, cache, positions = attention_setup(dtype, n_heads, n_kv, d, hidden, **kw)
+    torch.manual_seed(7)
+    seqs = [torch.randn(n, hidden).to(dtype) for n in (150, 9, 70)]
+    want = [plain_attention(s.double(), w, n_heads, n_kv, d, **kw) for s in seqs]
+    # whole prompts in one step; then a prompt step plus one row per step; then three uneven cuts
+    for cuts in ([], list(range(100, 150)), [3, 64, 65]):
+        got = run_mixer(att, cache, positions, dtype, seqs, cuts)
+        for g, r in zip(got, want):
+            close(g, r, dtype, f"attention {variant} cuts={cuts[:3]}", ulps=6.0)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_prenorm_block_alone(dtype, tmp_path):
+    """One layer of tiny B, built through the registry from its plan, against the plain layer."""
+    from dryft_amd.cache import CacheStore
+    from dryft_amd.config import Qwen3Config
+    from dryft_amd.engine.step import BatchBuffers, stage_batch
+    from dryft_amd.models.qwen3 import qwen3_plan
+    from dryft_amd.parts import block_class, build_part
+    from dryft_amd.parts.base import Partials
+    from helpers import make_model_dir, read_model_dir
+    raw, weights = read_model_dir(make_model_dir(str(tmp_path / "b"), TINY_B, seed=22, norm_std=0.1))
+    plan = qwen3_plan(Qwen3Config.from_dict(raw))
+    layer = plan.layers[2]
+    parts = {}
+    for role, spec in layer.parts.items():
+        part = build_part(spec)
+        part.load({k: weights[spec.tensors[k]].to(DEV).to(dtype) for k in part.tensor_specs()})
+        parts[role] = part
+    block = block_class(layer.block)(**parts)
+    rot = build_part(plan.positions["rotary"])
+    rot.prepare(128, dtype, DEV)
+    cache = CacheStore({0: parts["mixer"].cache_need()}, max_tokens=256, n_slots=2, max_len=128, dtype=dtype, device=DEV)
+    torch.manual_seed(3)
+    x = torch.randn(37, raw["hidden_size"]).to(dtype)
+    slot = cache.acquire(1)
+    ctx = stage_batch(cache, BatchBuffers(64, 2, DEV), slot, [37], [0] * 37, dtype)
+    ctx.positions = {"rotary": rot}
+    res, pending = block.forward(x.to(DEV).clone(), None, ctx, cache.line(0), True)
+    if isinstance(pending, Partials):
+        pending = pending.data[: pending.count].sum(0)
+    cos, sin = P.rope_tables(raw["head_dim"], raw["rope_theta"], 37, torch.float64)
+    want = P.decoder_layer(x.double(), {k: v.double() for k, v in weights.items()}, 2, raw, cos, sin)
+    close(res.float() + pending.float(), want, dtype, "block", ulps=6.0)
+
+
+# ------------------------------------------------------------------------------------------------
+# A toy architecture defined here: layer 0 mixes with a decaying sum kept as per-sequence state,
+# layer 1 with the library's attention. Nothing in the package knows about it.
+@dataclass(frozen=True)
+class ToyConfig:
+    hidden_size: int
+    vocab_size: int
+    decay: float
+    intermediate_size: int
+
+    @classmethod
+    def from_dict(cls, raw):
+        return cls(raw["hidden_size"], raw["vocab_size"], raw["decay"], raw["intermediate_size"])
+
+
+def toy_plan(cfg):
+    from dryft_amd.config import LayerSpec, ModelPlan, PartSpec, Run
+    H = cfg.hidden_size
+
+    def norm(name):
+        return PartSpec("rmsnorm", dict(size=H, eps=1e-5), {"weight": name})
+
+    def ffn(i):
+        return PartSpec("swiglu", dict(hidden_size=H, intermediate_size=cfg.intermediate_size),
+                        {"gate_proj": f"l{i}.gate", "up_proj": f"l{i}.up", "down_proj": f"l{i}.down"})
+
+    layers = (
+        LayerSpec("prenorm", {"mixer_norm": norm("l0.n1"), "ffn_norm": norm("l0.n2"), "ffn": ffn(0),
+                              "mixer": PartSpec("toy_decay_mixer", dict(hidden_size=H, decay=cfg.decay),
+                                                {"w_in": "l0.w_in", "w_out": "l0.w_out"})}),
+        LayerSpec("prenorm", {"mixer_norm": norm("l1.n1"), "ffn_norm": norm("l1.n2"), "ffn": ffn(1),
+                              "mixer": PartSpec("gqa_attention", dict(hidden_size=H, num_heads=4, num_kv_heads=2,
+                                                                      head_dim=16, positions="rotary"),
+                                                {k: f"l1.{k}" for k in ("q_proj", "k_proj", "v_proj", "o_proj")})}),
+    )
+    return ModelPlan(vocab_size=cfg.vocab_size, hidden_size=H,
+                     embedding=PartSpec("token_embedding", dict(vocab_size=cfg.vocab_size, hidden_size=H), {"weight": "emb"}),
+                     layers=layers, schedule=(Run(0, 0), Run(1, 1)), final_norm=norm("final"),
+                     head=PartSpec("lm_head", dict(vocab_size=cfg.vocab_size, hidden_size=H, tied=True), {}),
+                     positions={"rotary": PartSpec("rotary", dict(dim=16, theta=1e4))})
+
+
+def register_toy():
+    from dryft_amd import register_architecture, register_part
+    from dryft_amd.cache import StateNeed
+    from dryft_amd.models import known_architectures
+    from dryft_amd.parts.base import Mixer, matrix
+
+    class DecayMixer(Mixer):
+        """out_t = s_t @ w_out with s_t = decay * s_{t-1} + h_t @ w_in; s lives in the cache, one per sequence."""
+
+        def __init__(self, hidden_size, decay):
+            self.hidden, self.decay = hidden_size, decay
+
+        def tensor_specs(self):
+            return {"w_in": matrix((self.hidden, self.hidden)), "w_out": matrix((self.hidden, self.hidden))}
+
+        def load(self, tensors):
+            self.w_in, self.w_out = tensors["w_in"].float(), tensors["w_out"].float()
+
+        def cache_need(self):
+            return StateNeed((self.hidden,), "float32")
+
+        def forward(self, h, ctx, line, writes_cache):
+            u = h.float() @ self.w_in.T
+            out = torch.zeros_like(u)
+            row = 0
+            for slot, n in zip(ctx.host.slots, ctx.host.q_lens):       # the step as the host knows it
+                if slot >= 0:
+                    s = line.state[slot]
+                    for t in range(n):
+                        s = self.decay * s + u[row + t]
+                        out[row + t] = s
+                    line.state[slot] = s
+                row += n
+            return (out @ self.w_out.T).to(h.dtype)
+
+    if "ToyDecayLM" not in known_architectures():
+        register_part("toy_decay_mixer", DecayMixer)
+        register_architecture("ToyDecayLM", ToyConfig, toy_plan)
+
+
+def toy_plain(cfg, w, tokens):
+    """The toy model on one whole sequence, written out with the plain part functions."""
+    w = {k: v.double() for k, v in w.items()}
+    x = w["emb"][torch.tensor(tokens)]
+    T = len(tokens)
+    h = P.rms_norm(x, w["l0.n1"], 1e-5)
+    u = h @ w["l0.w_in"].T
+    s = torch.zeros(cfg["hidden_size"], dtype=torch.float64)
+    mixed = []
+    for t in range(T):
+        s = cfg["decay"] * s + u[t]
+        mixed.append(s)
+    x = x + torch.stack(mixed) @ w["l0.w_out"].T
+    x = x + P.swiglu(P.rms_norm(x, w["l0.n2"], 1e-5), {f"mlp.{k}_proj.weight": w[f"l0.{k}"] for k in ("gate", "up", "down")}, "")
+    h = P.rms_norm(x, w["l1.n1"], 1e-5)
+    q = (h @ w["l1.q_proj"].T).view(T, 4, 16)
+    k = (h @ w["l1.k_proj"].T).view(T, 2, 16)
+    v = (h @ w["l1.v_proj"].T).view(T, 2, 16)
+    cos, sin = P.rope_tables(16, 1e4, T, torch.float64)
+    o = P.causal_gqa_attention(P.apply_rope(q, cos, sin), P.apply_rope(k, cos, sin), v, 0.25)
+    x = x + o.reshape(T, 64) @ w["l1.o_proj"].T
+    x = x + P.swiglu(P.rms_norm(x, w["l1.n2"], 1e-5), {f"mlp.{k}_proj.weight": w[f"l1.{k}"] for k in ("gate", "up", "down")}, "")
+    return P.rms_norm(x, w["final"], 1e-5) @ w["emb"].T
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_mixer_with_state_is_registered_built_and_stepped(dtype, tmp_path):
+    from dryft_amd import Engine
+    from dryft_amd.engine.replay import Replayer
+    from helpers import collect_positions, read_model_dir, trace_batches, trace_whole
+    register_toy()
+    raw = {"architectures": ["ToyDecayLM"], "hidden_size": 64, "vocab_size": 97, "decay": 0.8, "intermediate_size": 72}
+    # random weights written to a folder by the library, read back by name
+    from dryft_amd.engine.model import DecoderModel
+    from dryft_amd.weights import random_tensors, write_model_dir
+    model = DecoderModel(toy_plan(ToyConfig.from_dict(raw)), torch.float32, "cpu")
+    assert any(isinstance(n, __import__("dryft_amd").cache.StateNeed) for n in model.cache_needs().values())
+    path = write_model_dir(str(tmp_path / "toy"), raw, random_tensors(model.tensor_specs(), 5, torch.bfloat16, std=0.08))
+    _, weights = read_model_dir(path)
+    engine = Engine(path, dtype=dtype, max_batch=4, max_len=256, use_graph=False)
+    assert len(engine.cache.state_groups) == 1 and len(engine.cache.kv_groups) == 1
+    reqs = {f"t{n}": random_tokens(n, 97, seed=n) for n in (3, 40, 90)}
+    want = {rid: toy_plain(raw, weights, toks).float() for rid, toks in reqs.items()}
+    limit = 1e-4 if dtype == "float32" else 3e-2
+    traces = [list(trace_whole(reqs)),
+              list(trace_batches([{rid: (toks, min(len(toks) - 1, 20)) for rid, toks in reqs.items()}])),
+              list(trace_batches([{"t40": (reqs["t40"], 39)}, {"t90": (reqs["t90"], 5), "t3": (reqs["t3"], 1)}]))]
+    for records in traces:
+        r = Replayer(engine)
+        outputs = {}
+        for rec in records:
+            lg = r.run_step(rec)
+            if lg is not None and lg.shape[0]:
+                outputs[rec["step"]] = lg.float().cpu()
+        for (rid, pos), row in collect_positions(records, outputs).items():
+            ref = want[rid]
+            err = float((row - ref[pos]).abs().max()) / float(ref.abs().max())
+            assert err <= limit, f"{rid}@{pos}: {err}"
+        assert not engine.cache.state_groups[0].data.any(), "state of released slots must be zero again"
+
+
+# ------------------------------------------------------------------------------------------------
+def test_layer_named_twice_and_a_run_that_reads_anothers_cache(tmp_path):
+    """Schedule: layer 0, layer 1, layer 1 again (own cache line), then layer 0 again reading the keys and
+    values its first run wrote."""
+    from dataclasses import replace
+    from dryft_amd import Engine, register_architecture
+    from dryft_amd.config import Qwen3Config, Run
+    from dryft_amd.models import known_architectures
+    from dryft_amd.models.qwen3 import qwen3_plan
+    from helpers import TINY_A, make_model_dir, read_model_dir
+    schedule = (Run(0, 0), Run(1, 1), Run(1, 2), Run(0, 0, writes_cache=False))
+    if "Qwen3Looped" not in known_architectures():
+        register_architecture("Qwen3Looped", Qwen3Config, lambda cfg: replace(qwen3_plan(cfg), schedule=schedule))
+    raw = dict(TINY_A, architectures=["Qwen3ForCausalLM"])
+    path = make_model_dir(str(tmp_path / "m"), raw, seed=4, norm_std=0.1)
+    import json
+    raw_looped = dict(raw, architectures=["Qwen3Looped"])
+    with open(os.path.join(path, "config.json"), "w") as f:
+        json.dump(raw_looped, f)
+    _, weights = read_model_dir(path)
+    w = {k: v.double() for k, v in weights.items()}
+    toks = random_tokens(80, raw["vocab_size"], seed=8)
+    T, d, eps = 80, raw["head_dim"], raw["rms_norm_eps"]
+    cos, sin = P.rope_tables(d, raw["rope_theta"], T, torch.float64)
+
+    def attention(h, i, kv=None):
+        p = f"model.layers.{i}.self_attn."
+        q = P.apply_rope(P.rms_norm((h @ w[p + "q_proj.weight"].T).view(T, 4, d), w[p + "q_norm.weight"], eps), cos, sin)
+        if kv is None:
+            k = P.apply_rope(P.rms_norm((h @ w[p + "k_proj.weight"].T).view(T, 2, d), w[p + "k_norm.weight"], eps), cos, sin)
+            kv = (k, (h @ w[p + "v_proj.weight"].T).view(T, 2, d))
+        return P.causal_gqa_attention(q, kv[0], kv[1], 1 / math.sqrt(d)).reshape(T, -1) @ w[p + "o_proj.weight"].T, kv
+
+    x = w["model.embed_tokens.weight"][torch.tensor(toks)]
+    kept = {}
+    for i, reads in ((0, None), (1, None), (1, None), (0, "first")):
+        p = f"model.layers.{i}."
+        a, kv = attention(P.rms_norm(x, w[p + "input_layernorm.weight"], eps), i, kept.get(0) if reads else None)
+        if i == 0 and not reads:
+            kept[0] = kv
+        x = x + a
+        x = x + P.swiglu(P.rms_norm(x, w[p + "post_attention_layernorm.weight"], eps), w, p)
+    want = (P.rms_norm(x, w["model.norm.weight"], eps) @ w["model.embed_tokens.weight"].T).float()
+    engine = Engine(path, dtype="float32", max_batch=2, max_len=128, use_graph=False)
+    assert len(engine.cache.kv_groups) == 1 and len(engine.cache.kv_groups[0].lines) == 3   # three lines, four runs
+    from dryft_amd.engine.step import SeqStep
+    slot = engine.acquire(1)[0]
+    got = [engine.step([SeqStep(slot, toks[:50], list(range(50)))])]
+    for t in range(50, 80):
+        got.append(engine.step([SeqStep(slot, [toks[t]], [0])]))
+    engine.release([slot])
+    got = torch.cat(got).cpu()
+    assert float((got - want).abs().max()) <= 1e-4 * float(want.abs().max())

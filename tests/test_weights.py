@@ -1,0 +1,150 @@
+"""Weights by name: round trip, the one error that lists everything, dtypes (no GPU)."""
+
+import json
+import os
+
+import pytest
+import torch
+from safetensors.torch import load_file, save_file
+
+from dryft_amd.engine.model import DecoderModel
+from dryft_amd.models import resolve_architecture
+from dryft_amd.weights import (INT_TABLE, MATRIX, VECTOR, TensorSpec, WeightError, load_tensors, random_tensors,
+                               write_model_dir)
+from helpers import TINY_A, TINY_B, make_model_dir
+
+
+def model_for(raw, dtype=torch.float32):
+    arch = resolve_architecture(raw)
+    return DecoderModel(arch.plan(arch.config_class.from_dict(raw)), dtype, "cpu")
+
+
+def test_random_folder_reads_back_equal(tmp_path):
+    path = make_model_dir(str(tmp_path / "m"), TINY_B, seed=3, norm_std=0.1)
+    assert sorted(os.listdir(path)) == ["config.json", "model.safetensors"]
+    model = model_for(TINY_B)
+    specs = model.tensor_specs()
+    again = random_tensors(specs, 3, torch.bfloat16, norm_std=0.1)
+    loaded = load_tensors(path, specs, torch.bfloat16)
+    assert set(loaded) == {s.name for s in specs}
+    for s in specs:
+        assert loaded[s.name].dtype == torch.bfloat16 and tuple(loaded[s.name].shape) == s.shape
+        assert torch.equal(loaded[s.name], again[s.name]), s.name
+    other = random_tensors(specs, 4, torch.bfloat16, norm_std=0.1)
+    assert not torch.equal(other[specs[0].name], again[specs[0].name])
+    norm = loaded["model.layers.0.input_layernorm.weight"].float()
+    assert 0.05 < float(norm.std()) < 0.2 and abs(float(norm.mean()) - 1) < 0.05
+    emb = loaded["model.embed_tokens.weight"].float()
+    assert 0.015 < float(emb.std()) < 0.025
+    # norm weights are exactly one when no spread is asked for
+    ones = random_tensors(specs, 3, torch.bfloat16)["model.norm.weight"]
+    assert torch.equal(ones, torch.ones_like(ones))
+
+
+def test_float32_mode_widens_exactly(tmp_path):
+    path = make_model_dir(str(tmp_path / "m"), TINY_A, seed=1)
+    specs = model_for(TINY_A).tensor_specs()
+    low = load_tensors(path, specs, torch.bfloat16)
+    wide = load_tensors(path, specs, torch.float32)
+    for name, t in wide.items():
+        assert t.dtype == torch.float32 and torch.equal(t, low[name].float())
+
+
+def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
+    path = make_model_dir(str(tmp_path / "m"), TINY_B, seed=3)
+    file = os.path.join(path, "model.safetensors")
+    t = load_file(file)
+    del t["model.layers.1.mlp.up_proj.weight"]
+    del t["model.norm.weight"]
+    t["model.layers.0.self_attn.q_proj.weight"] = t["model.layers.0.self_attn.q_proj.weight"][:, :-1].contiguous()
+    t["model.layers.2.self_attn.k_norm.weight"] = torch.ones(7, dtype=torch.bfloat16)
+    t["model.layers.0.self_attn.rotary_emb.inv_freq"] = torch.ones(4)
+    t["extra.weight"] = torch.ones(2, 2)
+    save_file(t, file)
+    with pytest.raises(WeightError) as e:
+        load_tensors(path, model_for(TINY_B).tensor_specs(), torch.bfloat16)
+    err = e.value
+    assert err.missing == ["model.layers.1.mlp.up_proj.weight", "model.norm.weight"]
+    assert err.unexpected == ["extra.weight", "model.layers.0.self_attn.rotary_emb.inv_freq"]
+    assert [w[0] for w in err.wrong_shape] == ["model.layers.0.self_attn.q_proj.weight",
+                                               "model.layers.2.self_attn.k_norm.weight"]
+    assert err.wrong_shape[0][1:] == ((256, 96), (256, 95))
+    text = str(err)
+    for name in err.missing + err.unexpected + [w[0] for w in err.wrong_shape]:
+        assert name in text
+
+
+def test_untied_model_needs_its_head_and_tied_copy_must_match(tmp_path):
+    path = make_model_dir(str(tmp_path / "b"), TINY_B, seed=3)
+    file = os.path.join(path, "model.safetensors")
+    t = load_file(file)
+    del t["lm_head.weight"]
+    save_file(t, file)
+    with pytest.raises(WeightError) as e:
+        load_tensors(path, model_for(TINY_B).tensor_specs(), torch.bfloat16)
+    assert e.value.missing == ["lm_head.weight"]
+    # tied: a copy of the embedding may be present, and must equal it (reference weights.py:82-88)
+    path = make_model_dir(str(tmp_path / "a"), TINY_A, seed=3)
+    file = os.path.join(path, "model.safetensors")
+    t = load_file(file)
+    t["lm_head.weight"] = t["model.embed_tokens.weight"].clone()
+    save_file(t, file)
+    model = model_for(TINY_A)
+    tensors = load_tensors(path, model.tensor_specs(), torch.float32, ignore=model.optional_names())
+    model.load(tensors)
+    assert model.head.weight is model.embedding.weight
+    t["lm_head.weight"] = t["lm_head.weight"] + 1
+    save_file(t, file)
+    model = model_for(TINY_A)
+    with pytest.raises(ValueError, match="differs from the embedding"):
+        model.load(load_tensors(path, model.tensor_specs(), torch.float32, ignore=model.optional_names()))
+
+
+def test_dtype_rule(tmp_path):
+    """bfloat16 by default; a vector stored in 32-bit stays 32-bit; integer tables become int32."""
+    tensors = {"m": torch.randn(4, 6), "m16": torch.randn(4, 6).to(torch.float16), "v32": torch.randn(6),
+               "vb": torch.randn(6).to(torch.bfloat16), "ids": torch.arange(5, dtype=torch.int64)}
+    write_model_dir(str(tmp_path), {"architectures": ["none"]}, tensors)
+    specs = [TensorSpec("m", (4, 6), MATRIX), TensorSpec("m16", (4, 6), MATRIX), TensorSpec("v32", (6,), VECTOR),
+             TensorSpec("vb", (6,), VECTOR), TensorSpec("ids", (5,), INT_TABLE)]
+    got = load_tensors(str(tmp_path), specs, torch.bfloat16)
+    assert [got[n].dtype for n in ("m", "m16", "v32", "vb", "ids")] == \
+        [torch.bfloat16, torch.bfloat16, torch.float32, torch.bfloat16, torch.int32]
+    assert torch.equal(got["v32"], tensors["v32"]) and got["ids"].tolist() == [0, 1, 2, 3, 4]
+    wide = load_tensors(str(tmp_path), specs, torch.float32)
+    assert [wide[n].dtype for n in ("m", "m16", "v32", "vb", "ids")] == [torch.float32] * 4 + [torch.int32]
+    with pytest.raises(WeightError, match="integer table stored as"):
+        load_tensors(str(tmp_path), [TensorSpec("m", (4, 6), INT_TABLE)] + specs[1:], torch.bfloat16)
+
+
+def test_shards_are_found_through_the_index(tmp_path):
+    path = make_model_dir(str(tmp_path / "m"), TINY_A, seed=9)
+    file = os.path.join(path, "model.safetensors")
+    t = load_file(file)
+    names = sorted(t)
+    half = len(names) // 2
+    save_file({n: t[n] for n in names[:half]}, os.path.join(path, "model-00001-of-00002.safetensors"))
+    save_file({n: t[n] for n in names[half:]}, os.path.join(path, "model-00002-of-00002.safetensors"))
+    os.remove(file)
+    index = {"weight_map": {n: f"model-0000{1 if i < half else 2}-of-00002.safetensors" for i, n in enumerate(names)}}
+    with open(os.path.join(path, "model.safetensors.index.json"), "w") as f:
+        json.dump(index, f)
+    got = load_tensors(path, model_for(TINY_A).tensor_specs(), torch.bfloat16)
+    assert all(torch.equal(got[n], t[n]) for n in names)
+    with pytest.raises(FileNotFoundError):
+        load_tensors(str(tmp_path / "empty"), [], torch.bfloat16)
+
+
+def test_fused_rows_equal_their_parts(tmp_path):
+    """q;k;v and gate;up are stacked by rows (reference weights.py:93-100)."""
+    path = make_model_dir(str(tmp_path / "m"), TINY_B, seed=3)
+    model = model_for(TINY_B)
+    tensors = load_tensors(path, model.tensor_specs(), torch.float32)
+    model.load(tensors)
+    att, ffn = model.blocks[1].mixer, model.blocks[1].ffn
+    p = "model.layers.1."
+    assert torch.equal(att.w_qkv[:256], tensors[p + "self_attn.q_proj.weight"])
+    assert torch.equal(att.w_qkv[256:320], tensors[p + "self_attn.k_proj.weight"])
+    assert torch.equal(att.w_qkv[320:], tensors[p + "self_attn.v_proj.weight"])
+    assert torch.equal(ffn.w_gate_up[:224], tensors[p + "mlp.gate_proj.weight"])
+    assert torch.equal(ffn.w_gate_up[224:], tensors[p + "mlp.up_proj.weight"])
