@@ -1,0 +1,184 @@
+"""Command line: token ids in, token ids out (the library has no tokenizer, like the reference:
+AGENTS.md:120). Option names follow the reference's tools where it has them: ``--model`` with the
+``DRYFT_MODEL_PATH`` environment variable as its default, ``--tiny`` for a random tiny model,
+``--seed``, ``--samples`` and ``--workload name,b,in,out`` (agent/verify.py:181-190,
+agent/bench.py:180-192).
+
+    python -m dryft_amd generate --model DIR --prompt-ids "1,2,3;4,5" --max-new-tokens 8
+    python -m dryft_amd generate --preset tiny-b --weight-seed 0 --random-prompts 3,5,9 --temperature 0.8
+    python -m dryft_amd make-model --preset tiny-a --weight-seed 1 --out DIR
+    python -m dryft_amd bench --preset qwen3-4b --workload b8,8,2048,64
+    python -m dryft_amd replay --model DIR --dtype float32 --out DIR --max-tokens 4096 < steps.jsonl
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import random
+import statistics
+import sys
+import time
+
+
+def _add_model_options(ap: argparse.ArgumentParser) -> None:
+    ap.add_argument("--model", default=os.environ.get("DRYFT_MODEL_PATH"),
+                    help="folder with config.json and safetensors (default: $DRYFT_MODEL_PATH)")
+    ap.add_argument("--preset", help="a named config with random weights instead of --model")
+    ap.add_argument("--tiny", action="store_true", help="same as --preset tiny-a")
+    ap.add_argument("--weight-seed", type=int, default=0, help="seed of the random weights")
+    ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32", "bfloat16", "float32"])
+    ap.add_argument("--max-len", type=int, default=4096, help="longest sequence a cache slot can hold")
+    ap.add_argument("--max-batch", type=int, default=None, help="cache slots (default: the number of prompts)")
+    ap.add_argument("--no-graph", action="store_true", help="run decoding steps without graph capture")
+
+
+def _engine(args, max_batch: int):
+    from . import Engine
+    from .models.qwen3 import load_preset
+
+    kw = dict(dtype=args.dtype, max_batch=args.max_batch or max_batch, max_len=args.max_len,
+              use_graph=not args.no_graph, verbose=True)
+    preset = "tiny-a" if args.tiny else args.preset
+    if preset:
+        return Engine(config=load_preset(preset), seed=args.weight_seed, **kw)
+    if not args.model:
+        raise SystemExit("need --model DIR (or DRYFT_MODEL_PATH), --preset NAME or --tiny")
+    return Engine(args.model, **kw)
+
+
+def _prompts(args, vocab: int) -> list[list[int]]:
+    if args.prompt_ids:
+        return [[int(t) for t in p.split(",") if t.strip()] for p in args.prompt_ids.split(";")]
+    if args.prompt_file:
+        with open(args.prompt_file) as f:
+            return [[int(t) for t in p] for p in json.load(f)]
+    if args.random_prompts:
+        rng = random.Random(args.prompt_seed)
+        return [[rng.randrange(vocab) for _ in range(int(n))] for n in args.random_prompts.split(",")]
+    raise SystemExit("need --prompt-ids, --prompt-file or --random-prompts")
+
+
+def cmd_generate(args) -> int:
+    n = len(args.prompt_ids.split(";")) if args.prompt_ids else (len(args.random_prompts.split(",")) if args.random_prompts else 8)
+    engine = _engine(args, max(1, n))
+    prompts = _prompts(args, engine.config.vocab_size)
+    stops = [int(t) for t in args.stop_ids.split(",")] if args.stop_ids else []
+    columns: list[list[int]] = [[] for _ in prompts]
+    for step in engine.generate(prompts, args.max_new_tokens, temperature=args.temperature,
+                                sample_seed=args.sample_seed, stop_token_ids=stops):
+        for col, t in zip(columns, step):
+            if t >= 0:
+                col.append(t)
+        if args.stream:
+            print(json.dumps(step), flush=True)
+    if not args.stream:
+        for col in columns:
+            print(",".join(map(str, col)))
+    return 0
+
+
+def cmd_make_model(args) -> int:
+    import torch
+
+    from .engine.model import DecoderModel
+    from .models import resolve_architecture
+    from .models.qwen3 import load_preset
+    from .weights import random_tensors, write_model_dir
+
+    if args.config:
+        with open(args.config) as f:
+            raw = json.load(f)
+    else:
+        raw = load_preset("tiny-a" if args.tiny else args.preset)
+    arch = resolve_architecture(raw)
+    model = DecoderModel(arch.plan(arch.config_class.from_dict(raw)), torch.float32, "cpu")
+    dtype = torch.bfloat16 if args.dtype in ("bf16", "bfloat16") else torch.float32
+    tensors = random_tensors(model.tensor_specs(), args.weight_seed, dtype, std=args.std, norm_std=args.norm_std)
+    print(write_model_dir(args.out, raw, tensors))
+    return 0
+
+
+def cmd_bench(args) -> int:
+    """Per workload: one untimed warm-up call, then ``--samples`` timed calls with fresh random prompts
+    (agent/bench.py:96-126); reports median tokens/s, time to first token and time per output token."""
+    import torch
+
+    workloads = [w.split(",") for w in (args.workload or ["b1,1,512,32", "b4,4,2048,32", "b16,16,512,128"])]
+    workloads = [(n, int(b), int(i), int(o)) for n, b, i, o in workloads]
+    args.max_len = max(args.max_len, max(i + o for _, _, i, o in workloads))
+    engine = _engine(args, max(b for _, b, _, _ in workloads))
+    rng = random.Random(args.seed)
+    vocab = engine.config.vocab_size
+    for name, b, inp, out in workloads:
+        totals, firsts = [], []
+        for sample in range(args.samples + 1):
+            ids = [[rng.randrange(vocab) for _ in range(inp)] for _ in range(b)]
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            first = None
+            for _ in engine.generate(ids, out):
+                if first is None:
+                    first = time.perf_counter() - t0
+            torch.cuda.synchronize()
+            if sample:
+                totals.append(time.perf_counter() - t0)
+                firsts.append(first)
+        med, ttft = statistics.median(totals), statistics.median(firsts)
+        tpot = (med - ttft) / (out - 1) if out > 1 else 0.0
+        print(json.dumps({"workload": name, "batch": b, "in": inp, "out": out, "tok_s": round(b * out / med, 1),
+                          "total_ms": round(med * 1e3, 2), "ttft_ms": round(ttft * 1e3, 2),
+                          "tpot_ms": round(tpot * 1e3, 3), "spread": round((max(totals) - min(totals)) / med, 3)}))
+    return 0
+
+
+def main(argv=None) -> int:
+    ap = argparse.ArgumentParser(prog="dryft_amd", description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    sub = ap.add_subparsers(dest="command", required=True)
+
+    g = sub.add_parser("generate", help="generate token ids for given prompts")
+    _add_model_options(g)
+    g.add_argument("--prompt-ids", help='prompts as "1,2,3;4,5"')
+    g.add_argument("--prompt-file", help="JSON file with a list of token-id lists")
+    g.add_argument("--random-prompts", help="lengths of random prompts, e.g. 5,9,17")
+    g.add_argument("--prompt-seed", type=int, default=0)
+    g.add_argument("--max-new-tokens", type=int, default=16)
+    g.add_argument("--temperature", type=float, default=0.0, help="0 = greedy")
+    g.add_argument("--sample-seed", type=int, default=0)
+    g.add_argument("--stop-ids", help="token ids that end a sequence, e.g. 151645,151643")
+    g.add_argument("--stream", action="store_true", help="print one JSON list per step instead of one line per sequence")
+    g.set_defaults(fn=cmd_generate)
+
+    m = sub.add_parser("make-model", help="write a model folder with seeded random weights")
+    m.add_argument("--preset", default="tiny-a")
+    m.add_argument("--tiny", action="store_true")
+    m.add_argument("--config", help="a config.json to use instead of a preset")
+    m.add_argument("--weight-seed", type=int, default=0)
+    m.add_argument("--std", type=float, default=0.02)
+    m.add_argument("--norm-std", type=float, default=0.0)
+    m.add_argument("--dtype", default="bf16", choices=["bf16", "fp32", "bfloat16", "float32"])
+    m.add_argument("--out", required=True)
+    m.set_defaults(fn=cmd_make_model)
+
+    b = sub.add_parser("bench", help="time whole generate calls on given workloads")
+    _add_model_options(b)
+    b.add_argument("--samples", type=int, default=5)
+    b.add_argument("--seed", type=int, default=0)
+    b.add_argument("--workload", action="append", help="name,batch,in,out (may repeat)")
+    b.set_defaults(fn=cmd_bench)
+
+    r = sub.add_parser("replay", help="trace replay (same as bin/trace_run)", add_help=False)
+    r.set_defaults(fn=None)
+
+    if argv is None:
+        argv = sys.argv[1:]
+    if argv and argv[0] == "replay":
+        from .engine.replay import main as replay_main
+        return replay_main(argv[1:])
+    args = ap.parse_args(argv)
+    return args.fn(args)
+
+
+if __name__ == "__main__":
+    sys.exit(main())
