@@ -62,6 +62,8 @@ def main() -> int:
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and batch 64 points")
     ap.add_argument("--no-graph", action="store_true")
+    ap.add_argument("--phase", default="all", choices=["all", "decode", "prefill"],
+                    help="measure only one phase (for profiling); the JSON line then lacks the other")
     ap.add_argument("--seed", type=int, default=0)
     args = ap.parse_args()
     if args.gpus != 1:
@@ -125,14 +127,17 @@ def main() -> int:
             best = dt if best is None else min(best, dt)
         return PROMPT / best, best * 1e3
 
-    tok_s, ms_step, context = decode_rate(args.batch, args.steps, args.warmup)
-    need = decode_bytes(cfg, layers, args.batch, context, elem)
-    achieved = need / (ms_step * 1e-3) / 1e9
-    pf_tok_s, pf_ms = prefill_rate()
-    peak = PEAK_FLOPS["bf16" if args.dtype == "bfloat16" else "fp32"]
-    pf_frac = prefill_flops(cfg, layers, PROMPT) / (pf_ms * 1e-3) / peak
+    tok_s = ms_step = achieved = pf_tok_s = pf_ms = pf_frac = 0.0
+    if args.phase in ("all", "decode"):
+        tok_s, ms_step, context = decode_rate(args.batch, args.steps, args.warmup)
+        need = decode_bytes(cfg, layers, args.batch, context, elem)
+        achieved = need / (ms_step * 1e-3) / 1e9
+    if args.phase in ("all", "prefill"):
+        pf_tok_s, pf_ms = prefill_rate()
+        peak = PEAK_FLOPS["bf16" if args.dtype == "bfloat16" else "fp32"]
+        pf_frac = prefill_flops(cfg, layers, PROMPT) / (pf_ms * 1e-3) / peak
     points = {}
-    if not args.no_points:
+    if not args.no_points and args.phase == "all":
         for b in (1, 64):
             points[f"decode_b{b}"] = round(decode_rate(b, max(16, args.steps // 2), max(4, args.warmup // 2))[0], 1)
     line = {

@@ -44,45 +44,97 @@ struct RowBlock {
   float m, l;            // running maximum and sum of the lane's own row (l % 16)
 };
 
-// One page (64 keys) for one wave. `key0` is the position of the page's first key; the lane's row sees
-// keys j with lo_row <= j <= hi_row. K page: [64][head_dim]; V^T page: [head_dim][64].
 template <int KB>
-__device__ __forceinline__ void attend_page(RowBlock<KB>& st, const bf16_t* __restrict__ k_page,
-                                            const bf16_t* __restrict__ v_page, int head_dim, float scale, int key0,
-                                            int lo_row, int hi_row) {
+__device__ __forceinline__ void init_rows(RowBlock<KB>& st, const bf16_t* q_row, bool row_valid, int head_dim) {
+  const int g = (threadIdx.x % WAVE) / 16;
+#pragma unroll
+  for (int kb = 0; kb < KB; ++kb) {
+    const int d = 32 * kb + 8 * g;
+    st.q[kb] = (row_valid && d < head_dim) ? load8(q_row + d) : zero8();
+  }
+#pragma unroll
+  for (int dt = 0; dt < 2 * KB; ++dt) st.o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  st.m = -INFINITY;
+  st.l = 0.f;
+}
+
+// ---------------------------------------------------------------------------------------------------
+// One page of 64 keys for one wave: loads, scores, online softmax and the second product.
+template <int KB>
+struct PageK {
+  bf16x8 k[4][KB];
+};
+template <int KB>
+struct PageV {
+  bf16x4 v[2 * KB][2][2];
+};
+
+// FULL: head_dim == 32 * KB. Otherwise features at or beyond head_dim are read from a clamped, valid address:
+// the query holds zeros there, so whatever finite value is read adds nothing to a score, and output
+// features beyond head_dim are computed but never stored. This keeps every load unconditional.
+template <int KB, bool FULL>
+__device__ __forceinline__ void load_page_k(PageK<KB>& f, const bf16_t* __restrict__ k_page, int head_dim) {
   const int lane = threadIdx.x % WAVE, c = lane % 16, g = lane / 16;
-  f32x4 s[4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t)
+#pragma unroll
+    for (int kb = 0; kb < KB; ++kb) {
+      const int d = FULL ? 32 * kb + 8 * g : min(32 * kb + 8 * g, head_dim - 8);
+      f.k[t][kb] = load8(k_page + (16 * t + c) * head_dim + d);
+    }
+}
+
+template <int KB, bool FULL>
+__device__ __forceinline__ void load_page_v(PageV<KB>& f, const bf16_t* __restrict__ v_page, int head_dim) {
+  const int lane = threadIdx.x % WAVE, c = lane % 16, g = lane / 16;
+#pragma unroll
+  for (int dt = 0; dt < 2 * KB; ++dt)
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int d = FULL ? 16 * dt + c : min(16 * dt + c, head_dim - 1);
+      const bf16_t* vp = v_page + d * PAGE_TOKENS + 32 * h + 4 * g;
+      f.v[dt][h][0] = *(const bf16x4*)vp;
+      f.v[dt][h][1] = *(const bf16x4*)(vp + 16);
+    }
+}
+
+// scores of one page from its loaded keys: s[t][i] for key 16t + 4g + i, in units of log2(e) so that exp2 serves
+template <int KB>
+__device__ __forceinline__ void page_scores(f32x4 (&s)[4], const PageK<KB>& f, const RowBlock<KB>& st) {
 #pragma unroll
   for (int t = 0; t < 4; ++t) {
     s[t] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int kb = 0; kb < KB; ++kb) {
-      const int d = 32 * kb + 8 * g;
-      const bf16x8 a = d < head_dim ? load8(k_page + (16 * t + c) * head_dim + d) : zero8();
-      s[t] = MFMA16(a, st.q[kb], s[t]);
-    }
+    for (int kb = 0; kb < KB; ++kb) s[t] = MFMA16(f.k[t][kb], st.q[kb], s[t]);
   }
+}
+
+// online softmax over the page's scores, then O^T += V^T P^T
+template <int KB>
+__device__ __forceinline__ void page_update(RowBlock<KB>& st, f32x4 (&s)[4], const PageV<KB>& f, int head_dim,
+                                            float scale_log2, int key0, int lo_row, int hi_row) {
+  const int g = (threadIdx.x % WAVE) / 16;
   float tile_max = -INFINITY;
 #pragma unroll
   for (int t = 0; t < 4; ++t)
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int j = key0 + 16 * t + 4 * g + i;
-      const float v = (j >= lo_row && j <= hi_row) ? s[t][i] * scale : -INFINITY;
+      const float v = (j >= lo_row && j <= hi_row) ? s[t][i] * scale_log2 : -INFINITY;
       s[t][i] = v;
       tile_max = fmaxf(tile_max, v);
     }
   tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, WAVE));
   tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, WAVE));
   const float m_new = fmaxf(st.m, tile_max);
-  const float m_safe = m_new == -INFINITY ? 0.f : m_new;   // a row that has seen no key yet stays empty
-  const float alpha = expf(st.m - m_safe);                  // exp(-inf) = 0 for such a row
+  const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+  const float alpha = exp2f(st.m - m_safe);
   float sum = 0.f;
 #pragma unroll
   for (int t = 0; t < 4; ++t)
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const float p = expf(s[t][i] - m_safe);
+      const float p = exp2f(s[t][i] - m_safe);
       s[t][i] = p;
       sum += p;
     }
@@ -100,41 +152,23 @@ __device__ __forceinline__ void attend_page(RowBlock<KB>& st, const bf16_t* __re
     }
 #pragma unroll
   for (int dt = 0; dt < 2 * KB; ++dt) {
-    if (16 * dt >= head_dim) break;
     st.o[dt] *= alpha;
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
-      const bf16_t* vp = v_page + (16 * dt + c) * PAGE_TOKENS + 32 * h + 4 * g;
-      const bf16x4 v0 = *(const bf16x4*)vp;
-      const bf16x4 v1 = *(const bf16x4*)(vp + 16);
       bf16x8 a;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        a[i] = v0[i];
-        a[4 + i] = v1[i];
+        a[i] = f.v[dt][h][0][i];
+        a[4 + i] = f.v[dt][h][1][i];
       }
       st.o[dt] = MFMA16(a, p[h], st.o[dt]);
     }
   }
 }
 
-template <int KB>
-__device__ __forceinline__ void init_rows(RowBlock<KB>& st, const bf16_t* q_row, bool row_valid, int head_dim) {
-  const int g = (threadIdx.x % WAVE) / 16;
-#pragma unroll
-  for (int kb = 0; kb < KB; ++kb) {
-    const int d = 32 * kb + 8 * g;
-    st.q[kb] = (row_valid && d < head_dim) ? load8(q_row + d) : zero8();
-  }
-#pragma unroll
-  for (int dt = 0; dt < 2 * KB; ++dt) st.o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
-  st.m = -INFINITY;
-  st.l = 0.f;
-}
-
 // ---------------------------------------------------------------------------------------------------
 // Many rows per sequence. Grid: (64-row query tiles, query heads); 4 waves of 16 rows each.
-template <int KB>
+template <int KB, bool FULL>
 __global__ __launch_bounds__(256) void attn_causal_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
     const int* __restrict__ page_table, int max_pages, const int* __restrict__ seq_slot,
@@ -165,43 +199,56 @@ __global__ __launch_bounds__(256) void attn_causal_kernel(
   const int lo_row = window > 0 ? max(0, pos_row - window + 1) : 0;
   const int lo_wave = window > 0 ? max(0, pos0 - window + 1) : 0;
   const int hi_wave = pos0 + rows - 1;
+  const float scale_log2 = scale * 1.44269504088896340736f;
+  const int64_t page_elems = (int64_t)PAGE_TOKENS * head_dim;
   for (int pg = lo_wave / PAGE_TOKENS; pg <= hi_wave / PAGE_TOKENS; ++pg) {
     const int page = page_table[(int64_t)slot * max_pages + pg];
     if (page < 0) continue;
-    const int64_t base = ((int64_t)page * n_kv + kvh) * PAGE_TOKENS * head_dim;
-    attend_page<KB>(st, k_pages + base, v_pages + base, head_dim, scale, pg * PAGE_TOKENS, lo_row, pos_row);
+    PageK<KB> kf;
+    PageV<KB> vf;
+    load_page_k<KB, FULL>(kf, k_pages + ((int64_t)page * n_kv + kvh) * page_elems, head_dim);
+    load_page_v<KB, FULL>(vf, v_pages + ((int64_t)page * n_kv + kvh) * page_elems, head_dim);
+    f32x4 s[4];
+    page_scores<KB>(s, kf, st);
+    page_update<KB>(st, s, vf, head_dim, scale_log2, pg * PAGE_TOKENS, lo_row, pos_row);
   }
   if (!row_valid) return;
   const float inv = 1.f / st.l;
   bf16_t* o = out + (row * n_heads + head) * head_dim;
 #pragma unroll
   for (int dt = 0; dt < 2 * KB; ++dt) {
-    if (16 * dt >= head_dim) break;
+    if (FULL || 16 * dt < head_dim) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) o[16 * dt + 4 * g + i] = float_to_bf16(st.o[dt][i] * inv);
+      for (int i = 0; i < 4; ++i) o[16 * dt + 4 * g + i] = float_to_bf16(st.o[dt][i] * inv);
+    }
   }
 }
 
 // ---------------------------------------------------------------------------------------------------
-// One row per sequence. Grid: (sequences, kv heads * head blocks, splits); one wave each. The wave's 16
-// "rows" are up to 16 query heads that share the kv head. Each split writes an unnormalised partial
-// (o, m, l); the combine kernel merges them in a fixed order, so results do not depend on timing.
-template <int KB>
-__global__ __launch_bounds__(64) void attn_split_kernel(
+// One row per sequence. Grid: (sequences, kv heads * head blocks, splits); four waves per workgroup.
+// The 16 "rows" of a wave are up to 16 query heads that share the kv head. A split covers a run of
+// pages; its waves take them in turn, each page's loads issued before the previous page's second
+// product so that memory stays busy, and merge their results in LDS. Each split writes an
+// unnormalised partial (o, m, l); the combine kernel merges splits in a fixed order, so results do
+// not depend on timing.
+#define SPLIT_WAVES 4
+
+template <int KB, bool FULL>
+__global__ __launch_bounds__(64 * SPLIT_WAVES, 2) void attn_split_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
     const int* __restrict__ page_table, int max_pages, const int* __restrict__ seq_slot,
     const int* __restrict__ cu_rows, const int* __restrict__ kv_len, float* __restrict__ part_o,
     float* __restrict__ part_ml, int n_heads, int n_kv, int head_dim, float scale, int window, int n_splits) {
+  __shared__ float merge_o[SPLIT_WAVES][16][32 * KB + 1];
+  __shared__ float merge_ml[SPLIT_WAVES][16][2];
   const int seq = blockIdx.x, split = blockIdx.z;
   const int group = n_heads / n_kv, blocks = (group + 15) / 16;
   const int kvh = blockIdx.y / blocks, hb = blockIdx.y % blocks;
-  const int lane = threadIdx.x, c = lane % 16, g = lane / 16;
+  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE, c = lane % 16, g = lane / 16;
   const int slot = seq_slot[seq];
   const int head = kvh * group + hb * 16 + c;
   const bool row_valid = hb * 16 + c < group;
   const int64_t row = cu_rows[seq];
-  float* po = part_o + (((int64_t)seq * n_heads + head) * n_splits + split) * head_dim;
-  float* pml = part_ml + (((int64_t)seq * n_heads + head) * n_splits + split) * 2;
   RowBlock<KB> st;
   init_rows<KB>(st, q + (row * n_heads + head) * head_dim, row_valid && slot >= 0, head_dim);
   if (slot >= 0) {
@@ -209,50 +256,101 @@ __global__ __launch_bounds__(64) void attn_split_kernel(
     const int lo = window > 0 ? max(0, pos - window + 1) : 0;
     const int pg_lo = lo / PAGE_TOKENS, pg_hi = pos / PAGE_TOKENS;
     const int per = (pg_hi - pg_lo + n_splits) / n_splits;     // ceil(pages / splits)
-    const int pg0 = pg_lo + split * per, pg1 = min(pg_hi, pg0 + per - 1);
-    for (int pg = pg0; pg <= pg1; ++pg) {
-      const int page = page_table[(int64_t)slot * max_pages + pg];
-      if (page < 0) continue;
-      const int64_t base = ((int64_t)page * n_kv + kvh) * PAGE_TOKENS * head_dim;
-      attend_page<KB>(st, k_pages + base, v_pages + base, head_dim, scale, pg * PAGE_TOKENS, lo, pos);
+    const int pg1 = min(pg_hi, pg_lo + split * per + per - 1);
+    const float scale_log2 = scale * 1.44269504088896340736f;
+    const int* table = page_table + (int64_t)slot * max_pages;
+    const int64_t page_elems = (int64_t)PAGE_TOKENS * head_dim;
+    int pg = pg_lo + split * per + wave;
+    PageK<KB> kf;
+    PageV<KB> vf;
+    int page = pg <= pg1 ? table[pg] : -1;
+    if (page >= 0) load_page_k<KB, FULL>(kf, k_pages + ((int64_t)page * n_kv + kvh) * page_elems, head_dim);
+    while (pg <= pg1) {
+      const int pg_next = pg + SPLIT_WAVES;
+      const int page_next = pg_next <= pg1 ? table[pg_next] : -1;
+      if (page >= 0) {
+        load_page_v<KB, FULL>(vf, v_pages + ((int64_t)page * n_kv + kvh) * page_elems, head_dim);
+        f32x4 s[4];
+        page_scores<KB>(s, kf, st);
+        if (page_next >= 0)
+          load_page_k<KB, FULL>(kf, k_pages + ((int64_t)page_next * n_kv + kvh) * page_elems, head_dim);
+        page_update<KB>(st, s, vf, head_dim, scale_log2, pg * PAGE_TOKENS, lo, pos);
+      } else if (page_next >= 0) {
+        load_page_k<KB, FULL>(kf, k_pages + ((int64_t)page_next * n_kv + kvh) * page_elems, head_dim);
+      }
+      pg = pg_next;
+      page = page_next;
     }
   }
-  if (!row_valid) return;
+  // merge the four waves' results: o = sum_w 2^(m_w - m) o_w, l likewise
 #pragma unroll
-  for (int dt = 0; dt < 2 * KB; ++dt) {
-    if (16 * dt >= head_dim) break;
-    *(f32x4*)(po + 16 * dt + 4 * g) = st.o[dt];
-  }
+  for (int dt = 0; dt < 2 * KB; ++dt)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) merge_o[wave][c][16 * dt + 4 * g + i] = st.o[dt][i];
   if (g == 0) {
-    pml[0] = st.m;
-    pml[1] = st.l;
+    merge_ml[wave][c][0] = st.m;
+    merge_ml[wave][c][1] = st.l;
+  }
+  __syncthreads();
+  const int tid = threadIdx.x;
+  for (int r = 0; r < 16; ++r) {
+    if (hb * 16 + r >= group) break;
+    float m = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < SPLIT_WAVES; ++w) m = fmaxf(m, merge_ml[w][r][0]);
+    float wgt[SPLIT_WAVES], l = 0.f;
+#pragma unroll
+    for (int w = 0; w < SPLIT_WAVES; ++w) {
+      const float mw = merge_ml[w][r][0];
+      wgt[w] = mw == -INFINITY ? 0.f : exp2f(mw - m);
+      l += wgt[w] * merge_ml[w][r][1];
+    }
+    const int h = kvh * group + hb * 16 + r;
+    float* po = part_o + (((int64_t)seq * n_heads + h) * n_splits + split) * head_dim;
+    for (int d = tid; d < head_dim; d += blockDim.x) {
+      float o = 0.f;
+#pragma unroll
+      for (int w = 0; w < SPLIT_WAVES; ++w) o += wgt[w] * merge_o[w][r][d];
+      po[d] = o;
+    }
+    if (tid == 0) {
+      float* pml = part_ml + (((int64_t)seq * n_heads + h) * n_splits + split) * 2;
+      pml[0] = m;       // in units of log2(e)
+      pml[1] = l;
+    }
   }
 }
 
-// out[seq_row, head, :] = sum_s w_s o_s / sum_s w_s l_s,  w_s = exp(m_s - max m)  (attn_decode.py:102-118)
-__global__ void attn_combine_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
-                                    const int* __restrict__ seq_slot, const int* __restrict__ cu_rows,
-                                    bf16_t* __restrict__ out, int n_heads, int head_dim, int n_splits) {
-  const int seq = blockIdx.x, head = blockIdx.y;
+// out[seq_row, head, :] = sum_s w_s o_s / sum_s w_s l_s,  w_s = 2^(m_s - max m)  (attn_decode.py:102-118)
+#define COMBINE_MAX_SPLITS 64
+__global__ __launch_bounds__(128) void attn_combine_kernel(const float* __restrict__ part_o,
+                                                           const float* __restrict__ part_ml,
+                                                           const int* __restrict__ seq_slot,
+                                                           const int* __restrict__ cu_rows, bf16_t* __restrict__ out,
+                                                           int n_heads, int head_dim, int n_splits) {
+  __shared__ float wgt[COMBINE_MAX_SPLITS];
+  __shared__ float inv_l;
+  const int seq = blockIdx.x, head = blockIdx.y, tid = threadIdx.x;
   const int64_t row = cu_rows[seq];
   bf16_t* o = out + (row * n_heads + head) * head_dim;
   const float* ml = part_ml + ((int64_t)seq * n_heads + head) * n_splits * 2;
   const float* po = part_o + ((int64_t)seq * n_heads + head) * n_splits * head_dim;
   const bool live = seq_slot[seq] >= 0;
-  float m = -INFINITY;
-  if (live)
-    for (int s = 0; s < n_splits; ++s) m = fmaxf(m, ml[2 * s]);
-  for (int d = threadIdx.x; d < head_dim; d += blockDim.x) {
-    float num = 0.f, den = 0.f;
-    if (live && m != -INFINITY)
-      for (int s = 0; s < n_splits; ++s) {
-        const float ms = ml[2 * s];
-        if (ms == -INFINITY) continue;   // a split that saw no key
-        const float w = expf(ms - m);
-        num += w * po[s * head_dim + d];
-        den += w * ml[2 * s + 1];
-      }
-    o[d] = float_to_bf16(den > 0.f ? num / den : 0.f);
+  if (tid < WAVE) {                       // the first wave turns (m_s, l_s) into weights
+    const float ms = (live && tid < n_splits) ? ml[2 * tid] : -INFINITY;
+    const float ls = (live && tid < n_splits) ? ml[2 * tid + 1] : 0.f;
+    const float m = wave_max(ms);
+    const float w = (ms == -INFINITY) ? 0.f : exp2f(ms - m);
+    const float l = wave_sum(w * ls);
+    if (tid < n_splits) wgt[tid] = w;
+    if (tid == 0) inv_l = l > 0.f ? 1.f / l : 0.f;
+  }
+  __syncthreads();
+  for (int d = tid; d < head_dim; d += blockDim.x) {
+    float num = 0.f;
+#pragma unroll 8
+    for (int s = 0; s < n_splits; ++s) num += wgt[s] * po[s * head_dim + d];
+    o[d] = float_to_bf16(num * inv_l);
   }
 }
 
@@ -280,11 +378,19 @@ DRYFT_API int dryft_attn_causal_bf16(const void* q, const void* k_pages, const v
   if (n_seqs <= 0 || max_tiles <= 0) return 0;
   if (!head_shape_ok(n_heads, n_kv, head_dim)) return -1;
   dim3 grid(max_tiles, n_heads), block(256);
-  DISPATCH_KB((head_dim + 31) / 32,
-              hipLaunchKernelGGL(attn_causal_kernel<KB>, grid, block, 0, stream, (const bf16_t*)q,
-                                 (const bf16_t*)k_pages, (const bf16_t*)v_pages, page_table, max_pages, seq_slot,
-                                 cu_rows, tile_cu, seq_start, n_seqs, (bf16_t*)out, n_heads, n_kv, head_dim, scale,
-                                 window));
+  if (head_dim % 32 == 0) {
+    DISPATCH_KB(head_dim / 32,
+                hipLaunchKernelGGL((attn_causal_kernel<KB, true>), grid, block, 0, stream, (const bf16_t*)q,
+                                   (const bf16_t*)k_pages, (const bf16_t*)v_pages, page_table, max_pages, seq_slot,
+                                   cu_rows, tile_cu, seq_start, n_seqs, (bf16_t*)out, n_heads, n_kv, head_dim, scale,
+                                   window));
+  } else {
+    DISPATCH_KB((head_dim + 31) / 32,
+                hipLaunchKernelGGL((attn_causal_kernel<KB, false>), grid, block, 0, stream, (const bf16_t*)q,
+                                   (const bf16_t*)k_pages, (const bf16_t*)v_pages, page_table, max_pages, seq_slot,
+                                   cu_rows, tile_cu, seq_start, n_seqs, (bf16_t*)out, n_heads, n_kv, head_dim, scale,
+                                   window));
+  }
   return DRYFT_LAUNCH_CHECK();
 }
 
@@ -293,16 +399,23 @@ DRYFT_API int dryft_attn_split_bf16(const void* q, const void* k_pages, const vo
                                     int n_seqs, float* part_o, float* part_ml, int n_splits, void* out, int n_heads,
                                     int n_kv, int head_dim, float scale, int window, hipStream_t stream) {
   if (n_seqs <= 0) return 0;
-  if (!head_shape_ok(n_heads, n_kv, head_dim) || n_splits < 1) return -1;
+  if (!head_shape_ok(n_heads, n_kv, head_dim) || n_splits < 1 || n_splits > COMBINE_MAX_SPLITS) return -1;
   const int group = n_heads / n_kv, blocks = (group + 15) / 16;
-  dim3 grid(n_seqs, n_kv * blocks, n_splits), block(64);
-  DISPATCH_KB((head_dim + 31) / 32,
-              hipLaunchKernelGGL(attn_split_kernel<KB>, grid, block, 0, stream, (const bf16_t*)q,
-                                 (const bf16_t*)k_pages, (const bf16_t*)v_pages, page_table, max_pages, seq_slot,
-                                 cu_rows, kv_len, part_o, part_ml, n_heads, n_kv, head_dim, scale, window, n_splits));
+  dim3 grid(n_seqs, n_kv * blocks, n_splits), block(64 * SPLIT_WAVES);
+  if (head_dim % 32 == 0) {
+    DISPATCH_KB(head_dim / 32,
+                hipLaunchKernelGGL((attn_split_kernel<KB, true>), grid, block, 0, stream, (const bf16_t*)q,
+                                   (const bf16_t*)k_pages, (const bf16_t*)v_pages, page_table, max_pages, seq_slot,
+                                   cu_rows, kv_len, part_o, part_ml, n_heads, n_kv, head_dim, scale, window, n_splits));
+  } else {
+    DISPATCH_KB((head_dim + 31) / 32,
+                hipLaunchKernelGGL((attn_split_kernel<KB, false>), grid, block, 0, stream, (const bf16_t*)q,
+                                   (const bf16_t*)k_pages, (const bf16_t*)v_pages, page_table, max_pages, seq_slot,
+                                   cu_rows, kv_len, part_o, part_ml, n_heads, n_kv, head_dim, scale, window, n_splits));
+  }
   int rc = DRYFT_LAUNCH_CHECK();
   if (rc) return rc;
-  hipLaunchKernelGGL(attn_combine_kernel, dim3(n_seqs, n_heads), dim3(64), 0, stream, part_o, part_ml, seq_slot,
+  hipLaunchKernelGGL(attn_combine_kernel, dim3(n_seqs, n_heads), dim3(128), 0, stream, part_o, part_ml, seq_slot,
                      cu_rows, (bf16_t*)out, n_heads, head_dim, n_splits);
   return DRYFT_LAUNCH_CHECK();
 }

@@ -94,61 +94,90 @@ __device__ __forceinline__ bf16x8 zero8g() {
 }
 
 // A wave computes C^T[n, m] = W[n, :] . x[m, :] for NTW tiles of 16 weight rows and MT tiles of 16
-// activation rows, over its share of K. Per 64 values of K a lane reads 32 contiguous bytes of its
-// weight row (4 lanes cover one 128-byte line) and the same 32 bytes' worth of its activation row; the
-// two halves feed two 32-deep products. Both operands use the same order of K, so the order itself
-// does not matter.
-template <int MT, int NTW, typename O>
+// activation rows, over its share of K, 64 values of K per step: a lane reads two 16-byte pieces of its
+// weight row (the four lanes of a row cover 64 contiguous bytes per piece) and the same of its activation
+// row. Rows beyond N or M are read from a clamped, valid row and their results are never stored, so the
+// main loop has no guards and is unrolled to keep many loads in flight. With SWIGLU the two weight tiles
+// of a wave are rows [n0, n0+16) of the first half (gate) and of the second half (up) of W, and the
+// epilogue stores T(T(silu(gate)) * up) for the N = rows/2 outputs (reference: kernels/silu_mul.py:29-32).
+#define SKINNY_UNROLL 4
+template <int MT, int NTW, bool SWIGLU, typename O>
 __global__ __launch_bounds__(256) void gemm_skinny_kernel(const bf16_t* __restrict__ x, int64_t x_stride,
                                                           const bf16_t* __restrict__ w, O* __restrict__ y,
                                                           float* __restrict__ partials, int M, int N, int K) {
   __shared__ f32x4 red[4][MT * NTW][WAVE];
   const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE, c = lane % 16, g = lane / 16;
-  const int n0 = blockIdx.x * 16 * NTW;
+  const int n0 = blockIdx.x * 16 * (SWIGLU ? 1 : NTW);
   const int splits = gridDim.y, units = splits * 4, unit = blockIdx.y * 4 + wave;
   const int kblocks = (K + 63) / 64, per = (kblocks + units - 1) / units;
-  const int kb0 = unit * per, kb1 = min(kblocks, kb0 + per);
+  const int kb0 = min(kblocks, unit * per), kb1 = min(kblocks, kb0 + per);
+  const int kb1_full = min(kb1, K / 64);              // blocks that lie wholly inside K
   f32x4 acc[NTW][MT];
 #pragma unroll
   for (int nt = 0; nt < NTW; ++nt)
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) acc[nt][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
   const bf16_t* wp[NTW];
-  bool w_ok[NTW];
 #pragma unroll
   for (int nt = 0; nt < NTW; ++nt) {
-    const int n = n0 + 16 * nt + c;
-    w_ok[nt] = n < N;
-    wp[nt] = w + (int64_t)(w_ok[nt] ? n : 0) * K;
+    const int n = SWIGLU ? nt * N + min(n0 + c, N - 1) : min(n0 + 16 * nt + c, N - 1);
+    wp[nt] = w + (int64_t)n * K + 8 * g;
   }
   const bf16_t* xp[MT];
-  bool x_ok[MT];
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt) {
-    const int m = 16 * mt + c;
-    x_ok[mt] = m < M;
-    xp[mt] = x + (int64_t)(x_ok[mt] ? m : 0) * x_stride;
+  for (int mt = 0; mt < MT; ++mt) xp[mt] = x + (int64_t)min(16 * mt + c, M - 1) * x_stride + 8 * g;
+  int kb = kb0;
+  for (; kb + SKINNY_UNROLL <= kb1_full; kb += SKINNY_UNROLL) {   // all loads of several blocks first, then the products
+    bf16x8 a[SKINNY_UNROLL][NTW][2], b[SKINNY_UNROLL][MT][2];
+#pragma unroll
+    for (int u = 0; u < SKINNY_UNROLL; ++u) {
+      const int k = (kb + u) * 64;
+#pragma unroll
+      for (int nt = 0; nt < NTW; ++nt) {
+        a[u][nt][0] = *(const bf16x8*)(wp[nt] + k);
+        a[u][nt][1] = *(const bf16x8*)(wp[nt] + k + 32);
+      }
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        b[u][mt][0] = *(const bf16x8*)(xp[mt] + k);
+        b[u][mt][1] = *(const bf16x8*)(xp[mt] + k + 32);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < SKINNY_UNROLL; ++u)
+#pragma unroll
+      for (int nt = 0; nt < NTW; ++nt)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][nt][0], b[u][mt][0], acc[nt][mt], 0, 0, 0);
+          acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][nt][1], b[u][mt][1], acc[nt][mt], 0, 0, 0);
+        }
   }
-  for (int kb = kb0; kb < kb1; ++kb) {
-    const int k = kb * 64 + 16 * g;
-    const bool k0_ok = k < K, k1_ok = k + 8 < K;
-    bf16x8 a[NTW][2], b[MT][2];
-#pragma unroll
-    for (int nt = 0; nt < NTW; ++nt) {
-      a[nt][0] = (w_ok[nt] && k0_ok) ? *(const bf16x8*)(wp[nt] + k) : zero8g();
-      a[nt][1] = (w_ok[nt] && k1_ok) ? *(const bf16x8*)(wp[nt] + k + 8) : zero8g();
-    }
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      b[mt][0] = (x_ok[mt] && k0_ok) ? *(const bf16x8*)(xp[mt] + k) : zero8g();
-      b[mt][1] = (x_ok[mt] && k1_ok) ? *(const bf16x8*)(xp[mt] + k + 8) : zero8g();
-    }
+  for (; kb < kb1_full; ++kb) {
+    const int k = kb * 64;
 #pragma unroll
     for (int nt = 0; nt < NTW; ++nt)
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) {
-        acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[nt][0], b[mt][0], acc[nt][mt], 0, 0, 0);
-        acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[nt][1], b[mt][1], acc[nt][mt], 0, 0, 0);
+        const bf16x8 a0 = *(const bf16x8*)(wp[nt] + k), a1 = *(const bf16x8*)(wp[nt] + k + 32);
+        const bf16x8 b0 = *(const bf16x8*)(xp[mt] + k), b1 = *(const bf16x8*)(xp[mt] + k + 32);
+        acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, b0, acc[nt][mt], 0, 0, 0);
+        acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, b1, acc[nt][mt], 0, 0, 0);
+      }
+  }
+  if (kb0 <= K / 64 && K / 64 < kb1) {                // the last, partial block of K (K is a multiple of 8)
+    const int k = (K / 64) * 64;
+    const bool ok0 = k + 8 * g < K, ok1 = k + 32 + 8 * g < K;
+#pragma unroll
+    for (int nt = 0; nt < NTW; ++nt)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        const bf16x8 a0 = ok0 ? *(const bf16x8*)(wp[nt] + k) : zero8g();
+        const bf16x8 b0 = ok0 ? *(const bf16x8*)(xp[mt] + k) : zero8g();
+        const bf16x8 a1 = ok1 ? *(const bf16x8*)(wp[nt] + k + 32) : zero8g();
+        const bf16x8 b1 = ok1 ? *(const bf16x8*)(xp[mt] + k + 32) : zero8g();
+        acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, b0, acc[nt][mt], 0, 0, 0);
+        acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, b1, acc[nt][mt], 0, 0, 0);
       }
   }
 #pragma unroll
@@ -156,6 +185,30 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const bf16_t* __restri
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) red[wave][nt * MT + mt][lane] = acc[nt][mt];
   __syncthreads();
+  if (SWIGLU) {
+    // activation-row tile mt is finished by wave mt % 4: gate and up of the same (n, m) sit in the same lane
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      if (mt % 4 != wave) continue;
+      f32x4 gate = red[0][mt][lane], up = red[0][MT + mt][lane];
+#pragma unroll
+      for (int wv = 1; wv < 4; ++wv) {
+        gate += red[wv][mt][lane];
+        up += red[wv][MT + mt][lane];
+      }
+      const int m = 16 * mt + c;
+      if (m >= M) continue;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int n = n0 + 4 * g + i;
+        if (n >= N) continue;
+        const float gv = rounded_as<bf16_t>(gate[i]), uv = rounded_as<bf16_t>(up[i]);
+        const float sv = rounded_as<bf16_t>(gv / (1.f + expf(-gv)));
+        store_from_float(y + (int64_t)m * N + n, sv * uv);
+      }
+    }
+    return;
+  }
   // tile t is summed (waves in order 0..3) and stored by wave t % 4
 #pragma unroll
   for (int t = 0; t < MT * NTW; ++t) {
@@ -184,11 +237,11 @@ static int launch_skinny(const void* x, int64_t x_stride, const void* w, void* y
                          int splits, int out_f32, hipStream_t stream) {
   dim3 grid((N + 16 * NTW - 1) / (16 * NTW), splits), block(256);
   if (out_f32)
-    hipLaunchKernelGGL((gemm_skinny_kernel<MT, NTW, float>), grid, block, 0, stream, (const bf16_t*)x, x_stride,
+    hipLaunchKernelGGL((gemm_skinny_kernel<MT, NTW, false, float>), grid, block, 0, stream, (const bf16_t*)x, x_stride,
                        (const bf16_t*)w, (float*)y, partials, M, N, K);
   else
-    hipLaunchKernelGGL((gemm_skinny_kernel<MT, NTW, bf16_t>), grid, block, 0, stream, (const bf16_t*)x, x_stride,
-                       (const bf16_t*)w, (bf16_t*)y, partials, M, N, K);
+    hipLaunchKernelGGL((gemm_skinny_kernel<MT, NTW, false, bf16_t>), grid, block, 0, stream, (const bf16_t*)x,
+                       x_stride, (const bf16_t*)w, (bf16_t*)y, partials, M, N, K);
   return DRYFT_LAUNCH_CHECK();
 }
 
@@ -216,6 +269,25 @@ DRYFT_API int dryft_gemm_skinny_bf16(const void* x, int64_t x_stride, const void
     default: return -1;
   }
 #undef SK
+}
+
+// y[M, N] = T(T(silu(x . Wg^T)) * (x . Wu^T)) with W = [Wg; Wu] of 2N rows
+DRYFT_API int dryft_gemm_skinny_swiglu_bf16(const void* x, int64_t x_stride, const void* w, void* y, int M, int N,
+                                            int K, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (M > 64 || K <= 0 || K % 8 || x_stride % 8) return -1;
+  dim3 grid((N + 15) / 16, 1), block(256);
+#define SW(MTV)                                                                                                    \
+  hipLaunchKernelGGL((gemm_skinny_kernel<MTV, 2, true, bf16_t>), grid, block, 0, stream, (const bf16_t*)x, x_stride, \
+                     (const bf16_t*)w, (bf16_t*)y, (float*)nullptr, M, N, K)
+  switch ((M + 15) / 16) {
+    case 1: SW(1); break;
+    case 2: SW(2); break;
+    case 3: SW(3); break;
+    default: SW(4); break;
+  }
+#undef SW
+  return DRYFT_LAUNCH_CHECK();
 }
 
 // y = T(sum_s partials[s]) in the order s = 0, 1, ...

@@ -41,6 +41,99 @@ __global__ void add_rmsnorm_kernel(const T* __restrict__ res, const D* __restric
   }
 }
 
+// The same for rows whose width is a multiple of 8 and at most 8 * 8 * blockDim: a thread owns runs of 8
+// contiguous values, reads them with 16-byte loads issued together, and keeps them in registers between the
+// two passes. This is the kernel that decoding steps use: few rows, so latency rather than bandwidth counts.
+typedef __attribute__((ext_vector_type(4))) float vf4;
+typedef __attribute__((ext_vector_type(4))) uint32_t vu4;
+
+__device__ __forceinline__ void load8_as_float(const float* p, float (&v)[8]) {
+  const vf4 a = *(const vf4*)p, b = *(const vf4*)(p + 4);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) { v[i] = a[i]; v[4 + i] = b[i]; }
+}
+__device__ __forceinline__ void load8_as_float(const bf16_t* p, float (&v)[8]) {
+  const vu4 a = *(const vu4*)p;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) { v[2 * i] = __uint_as_float(a[i] << 16); v[2 * i + 1] = __uint_as_float(a[i] & 0xffff0000u); }
+}
+__device__ __forceinline__ void store8_from_float(float* p, const float (&v)[8]) {
+  *(vf4*)p = vf4{v[0], v[1], v[2], v[3]};
+  *(vf4*)(p + 4) = vf4{v[4], v[5], v[6], v[7]};
+}
+__device__ __forceinline__ void store8_from_float(bf16_t* p, const float (&v)[8]) {
+  vu4 a;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) a[i] = (uint32_t)float_to_bf16(v[2 * i]).bits | ((uint32_t)float_to_bf16(v[2 * i + 1]).bits << 16);
+  *(vu4*)p = a;
+}
+
+#define NORM_VEC_RUNS 8   // runs of 8 values a thread may hold
+
+template <typename T, typename D, int RUNS>
+__global__ __launch_bounds__(512) void add_rmsnorm_vec_kernel(const T* __restrict__ res, const D* __restrict__ delta,
+                                                              int n_partials, int64_t partial_stride,
+                                                              const void* __restrict__ w, int w_f32,
+                                                              T* __restrict__ res_out, T* __restrict__ y, int width,
+                                                              float eps) {
+  __shared__ float scratch[16];
+  const int64_t row = blockIdx.x;
+  const int64_t base = row * width;
+  float v[RUNS][8];
+  float ss = 0.f;
+#pragma unroll
+  for (int r = 0; r < RUNS; ++r) {
+    const int i = (r * blockDim.x + threadIdx.x) * 8;
+    if (i < width) {
+      load8_as_float(res + base + i, v[r]);
+      if (n_partials > 0) {
+        float d[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        for (int p = 0; p < n_partials; ++p) {
+          float t[8];
+          load8_as_float(delta + p * partial_stride + base + i, t);
+#pragma unroll
+          for (int j = 0; j < 8; ++j) d[j] += t[j];
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[r][j] = rounded_as<T>(v[r][j] + d[j]);
+        store8_from_float(res_out + base + i, v[r]);
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) ss += v[r][j] * v[r][j];
+    }
+  }
+  ss = block_sum(ss, scratch);
+  const float inv = rsqrtf(ss / (float)width + eps);
+#pragma unroll
+  for (int r = 0; r < RUNS; ++r) {
+    const int i = (r * blockDim.x + threadIdx.x) * 8;
+    if (i < width) {
+      float o[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) o[j] = rounded_as<T>(v[r][j] * inv) * load_vector(w, i + j, w_f32);
+      store8_from_float(y + base + i, o);
+    }
+  }
+}
+
+template <typename T, typename D>
+static void launch_norm_vec(const void* res, const void* delta, int n_partials, int64_t partial_stride, const void* w,
+                            int w_f32, void* res_out, void* y, int n_rows, int width, float eps, hipStream_t stream) {
+  const int runs_total = width / 8;
+  int threads = 64;
+  while (threads < 512 && threads < runs_total) threads *= 2;
+  const int runs = (runs_total + threads - 1) / threads;
+  dim3 grid(n_rows), block(threads);
+#define NV(R)                                                                                                        \
+  hipLaunchKernelGGL((add_rmsnorm_vec_kernel<T, D, R>), grid, block, 0, stream, (const T*)res, (const D*)delta,      \
+                     n_partials, partial_stride, w, w_f32, (T*)res_out, (T*)y, width, eps)
+  if (runs <= 1) NV(1);
+  else if (runs <= 2) NV(2);
+  else if (runs <= 4) NV(4);
+  else NV(8);
+#undef NV
+}
+
 // delta_kind: 0 = none (plain norm), 1 = same dtype as the activations, 2 = float partial sums
 DRYFT_API int dryft_add_rmsnorm(const void* res, const void* delta, int delta_kind, int n_partials,
                                 int64_t partial_stride, const void* w, int w_f32, void* res_out, void* y,
@@ -49,6 +142,17 @@ DRYFT_API int dryft_add_rmsnorm(const void* res, const void* delta, int delta_ki
   const int threads = width >= 2048 ? 512 : 256;
   dim3 grid(n_rows), block(threads);
   if (delta_kind == 0) n_partials = 0;
+  const bool aligned = (((uintptr_t)res | (uintptr_t)delta | (uintptr_t)res_out | (uintptr_t)y) & 15) == 0 &&
+                       (partial_stride % 4) == 0;
+  if (width % 8 == 0 && width <= 8 * NORM_VEC_RUNS * 512 && aligned && n_rows <= 4096) {
+    if (is_f32)
+      launch_norm_vec<float, float>(res, delta, n_partials, partial_stride, w, w_f32, res_out, y, n_rows, width, eps, stream);
+    else if (delta_kind == 2)
+      launch_norm_vec<bf16_t, float>(res, delta, n_partials, partial_stride, w, w_f32, res_out, y, n_rows, width, eps, stream);
+    else
+      launch_norm_vec<bf16_t, bf16_t>(res, delta, n_partials, partial_stride, w, w_f32, res_out, y, n_rows, width, eps, stream);
+    return DRYFT_LAUNCH_CHECK();
+  }
   if (is_f32) {
     hipLaunchKernelGGL((add_rmsnorm_kernel<float, float>), grid, block, 0, stream, (const float*)res,
                        (const float*)delta, n_partials, partial_stride, w, w_f32, (float*)res_out, (float*)y, width,

@@ -31,8 +31,9 @@ _SIGNATURES = {
                                             _P]},
     "gemm": {"dryft_gemm_tiled": [_P, _L, _P, _P, _I, _I, _I, _I, _I, _P],
              "dryft_gemm_skinny_bf16": [_P, _L, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
+             "dryft_gemm_skinny_swiglu_bf16": [_P, _L, _P, _P, _I, _I, _I, _P],
              "dryft_sum_partials": [_P, _P, _L, _I, _I, _P]},
-    "sampling": {"dryft_argmax_rows": [_P, _I, _I, _L, _P, _P],
+    "sampling": {"dryft_argmax_rows": [_P, _I, _I, _L, _P, _I, _P, _P, _P],
                  "dryft_sample_rows": [_P, _I, _I, _L, _F, _P, _P, _P]},
 }
 _functions: dict[str, object] = {}
@@ -320,6 +321,23 @@ def gemm_skinny_bf16(x, w, out, partials=None, ntw: int = 1, splits: int = 1) ->
                                                  int(ntw), int(splits), out_f32, _stream()), "gemm_skinny_bf16")
 
 
+def gemm_skinny_swiglu_bf16(x, w_gate_up, out) -> torch.Tensor:
+    """``silu(x @ Wg.T) * (x @ Wu.T)`` for ``w_gate_up = [Wg; Wu]``, at most 64 rows, in one kernel."""
+    _gpu(x, "x", torch.bfloat16)
+    _gpu(w_gate_up, "w_gate_up", torch.bfloat16)
+    _gpu(out, "out", torch.bfloat16)
+    m, k = x.shape
+    two_n = w_gate_up.shape[0]
+    _require(two_n % 2 == 0 and w_gate_up.shape == (two_n, k) and w_gate_up.is_contiguous() and x.stride(1) == 1,
+             "gemm_skinny_swiglu: x [M,K] row-major, w [2N,K] contiguous")
+    _require(m <= 64 and k % 8 == 0 and x.stride(0) % 8 == 0, f"gemm_skinny_swiglu: needs M <= 64 and K % 8 == 0, got M={m} K={k}")
+    _require(x.data_ptr() % 16 == 0 and w_gate_up.data_ptr() % 16 == 0, "gemm_skinny_swiglu: operands must be 16-byte aligned")
+    _require(out.shape == (m, two_n // 2) and out.is_contiguous(), f"gemm_skinny_swiglu: out must be [{m},{two_n // 2}]")
+    _check(_fn("gemm", "dryft_gemm_skinny_swiglu_bf16")(_ptr(x), x.stride(0), _ptr(w_gate_up), _ptr(out), m, two_n // 2, k,
+                                                        _stream()), "gemm_skinny_swiglu_bf16")
+    return out
+
+
 def sum_partials(partials: torch.Tensor, out: torch.Tensor, splits: int) -> torch.Tensor:
     _gpu(partials, "partials", torch.float32)
     _gpu(out, "out")
@@ -337,8 +355,13 @@ def argmax_rows(logits: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     _gpu(out, "out", torch.int32)
     rows, vocab = logits.shape
     _require(logits.stride(1) == 1 and out.numel() >= rows and out.is_contiguous(), "argmax_rows: bad operands")
-    _check(_fn("sampling", "dryft_argmax_rows")(_ptr(logits), rows, vocab, logits.stride(0), _ptr(out), _stream()),
-           "argmax_rows")
+    chunks = 1 if vocab < 8192 else min(64, vocab // 2048)
+    scratch_v = scratch_i = None
+    if chunks > 1:
+        scratch_v = torch.empty(rows * chunks, dtype=torch.float32, device=logits.device)
+        scratch_i = torch.empty(rows * chunks, dtype=torch.int32, device=logits.device)
+    _check(_fn("sampling", "dryft_argmax_rows")(_ptr(logits), rows, vocab, logits.stride(0), _ptr(out), chunks,
+                                                _ptr(scratch_v), _ptr(scratch_i), _stream()), "argmax_rows")
     return out
 
 

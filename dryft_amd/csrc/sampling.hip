@@ -85,10 +85,73 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(const float
   if (tid == 0) out[blockIdx.x] = chosen;
 }
 
-DRYFT_API int dryft_argmax_rows(const float* logits, int n_rows, int vocab, int64_t row_stride, int* out,
-                                hipStream_t stream) {
+// Greedy choice in two stages for wide rows: `chunks` workgroups per row each find the best of their
+// stretch, then one wave per row picks among them (lower index wins on equal values in both stages).
+__global__ __launch_bounds__(256) void argmax_chunks_kernel(const float* __restrict__ logits, int vocab,
+                                                            int64_t row_stride, int chunks, float* __restrict__ best_v,
+                                                            int* __restrict__ best_i) {
+  __shared__ float sv[4];
+  __shared__ int si[4];
+  const int row = blockIdx.x, chunk = blockIdx.y;
+  const int per = (vocab + chunks - 1) / chunks;
+  const int i0 = chunk * per, i1 = min(vocab, i0 + per);
+  const float* r = logits + row * row_stride;
+  float v = -INFINITY;
+  int idx = 0x7fffffff;
+  for (int i = i0 + threadIdx.x; i < i1; i += blockDim.x) {
+    const float x = r[i];
+    if (x > v || (x == v && i < idx)) { v = x; idx = i; }
+  }
+#pragma unroll
+  for (int o = WAVE / 2; o > 0; o >>= 1) {
+    const float ov = __shfl_xor(v, o, WAVE);
+    const int oi = __shfl_xor(idx, o, WAVE);
+    if (ov > v || (ov == v && oi < idx)) { v = ov; idx = oi; }
+  }
+  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+  if (lane == 0) { sv[wave] = v; si[wave] = idx; }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < 4; ++w)
+      if (sv[w] > v || (sv[w] == v && si[w] < idx)) { v = sv[w]; idx = si[w]; }
+    best_v[row * chunks + chunk] = v;
+    best_i[row * chunks + chunk] = idx;
+  }
+}
+
+__global__ __launch_bounds__(64) void argmax_pick_kernel(const float* __restrict__ best_v, const int* __restrict__ best_i,
+                                                         int chunks, int vocab, int* __restrict__ out) {
+  const int row = blockIdx.x;
+  float v = -INFINITY;
+  int idx = 0x7fffffff;
+  for (int c = threadIdx.x; c < chunks; c += WAVE) {
+    const float x = best_v[row * chunks + c];
+    const int i = best_i[row * chunks + c];
+    if (x > v || (x == v && i < idx)) { v = x; idx = i; }
+  }
+#pragma unroll
+  for (int o = WAVE / 2; o > 0; o >>= 1) {
+    const float ov = __shfl_xor(v, o, WAVE);
+    const int oi = __shfl_xor(idx, o, WAVE);
+    if (ov > v || (ov == v && oi < idx)) { v = ov; idx = oi; }
+  }
+  if (threadIdx.x == 0) out[row] = idx < vocab ? idx : 0;
+}
+
+// scratch_v / scratch_i: room for n_rows * chunks entries each when chunks > 1
+DRYFT_API int dryft_argmax_rows(const float* logits, int n_rows, int vocab, int64_t row_stride, int* out, int chunks,
+                                float* scratch_v, int* scratch_i, hipStream_t stream) {
   if (n_rows <= 0) return 0;
-  hipLaunchKernelGGL(argmax_rows_kernel, dim3(n_rows), dim3(SAMPLE_THREADS), 0, stream, logits, vocab, row_stride, out);
+  if (chunks <= 1) {
+    hipLaunchKernelGGL(argmax_rows_kernel, dim3(n_rows), dim3(SAMPLE_THREADS), 0, stream, logits, vocab, row_stride, out);
+    return DRYFT_LAUNCH_CHECK();
+  }
+  if (chunks > 65535 || scratch_v == nullptr || scratch_i == nullptr) return -1;
+  hipLaunchKernelGGL(argmax_chunks_kernel, dim3(n_rows, chunks), dim3(256), 0, stream, logits, vocab, row_stride, chunks,
+                     scratch_v, scratch_i);
+  int rc = DRYFT_LAUNCH_CHECK();
+  if (rc) return rc;
+  hipLaunchKernelGGL(argmax_pick_kernel, dim3(n_rows), dim3(64), 0, stream, scratch_v, scratch_i, chunks, vocab, out);
   return DRYFT_LAUNCH_CHECK();
 }
 

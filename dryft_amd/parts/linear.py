@@ -20,7 +20,8 @@ from ..csrc import ops
 from .base import Partials
 
 SKINNY_ROWS = 64
-_TARGET_WORKGROUPS = 512   # about two per compute unit
+_TARGET_WORKGROUPS = 320   # a little more than one per compute unit
+_BLOCKS_PER_WAVE = 10      # 64-value blocks of K a wave should walk at most
 
 
 def skinny_plan(m: int, n: int, k: int) -> tuple[int, int]:
@@ -34,11 +35,13 @@ def skinny_plan(m: int, n: int, k: int) -> tuple[int, int]:
         ntw = 4
     workgroups = (tiles + ntw - 1) // ntw
     k_blocks = (k + 63) // 64
-    splits = max(1, min((_TARGET_WORKGROUPS + workgroups - 1) // workgroups, k_blocks // 8, 16))
+    want = max((_TARGET_WORKGROUPS + workgroups - 1) // workgroups,        # enough workgroups to fill the chip
+               (k_blocks + 4 * _BLOCKS_PER_WAVE - 1) // (4 * _BLOCKS_PER_WAVE))  # and no wave with a long walk over K
+    splits = max(1, min(want, k_blocks // 8, 16))
     return ntw, splits
 
 
-def _skinny_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
+def skinny_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
     return x.shape[1] % 8 == 0 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0
 
 
@@ -49,7 +52,7 @@ def linear(x: torch.Tensor, w: torch.Tensor, *, out_dtype: torch.dtype | None = 
     out_dtype = out_dtype or x.dtype
     if x.dtype == torch.float32:
         return ops.gemm_tiled(x, w, torch.empty((m, n), dtype=torch.float32, device=x.device))
-    if m <= SKINNY_ROWS and _skinny_ok(x, w):
+    if m <= SKINNY_ROWS and skinny_ok(x, w):
         ntw, splits = skinny_plan(m, n, k)
         if splits > 1:
             partials = torch.empty((splits, m, n), dtype=torch.float32, device=x.device)
@@ -62,7 +65,7 @@ def linear(x: torch.Tensor, w: torch.Tensor, *, out_dtype: torch.dtype | None = 
         return out
     if out_dtype == torch.float32:
         out = torch.empty((m, n), dtype=torch.float32, device=x.device)
-        if _skinny_ok(x, w):
+        if skinny_ok(x, w):
             ntw, _ = skinny_plan(SKINNY_ROWS, n, k)
             for m0 in range(0, m, SKINNY_ROWS):
                 ops.gemm_skinny_bf16(x[m0:m0 + SKINNY_ROWS], w, out[m0:m0 + SKINNY_ROWS], None, ntw, 1)

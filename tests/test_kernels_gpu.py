@@ -322,6 +322,19 @@ def test_gemm_skinny(m, n, k, ntw, splits):
         close(out, want, torch.float32, what="skinny split-K")
 
 
+@pytest.mark.parametrize("m", [1, 8, 16, 40, 64])
+@pytest.mark.parametrize("inter,k", [(9728, 2560), (224, 96), (136, 80), (37 * 8, 72)])
+def test_gemm_skinny_swiglu(m, inter, k):
+    torch.manual_seed(m + inter)
+    x = torch.randn(m, k).to(torch.bfloat16)
+    w = (torch.randn(2 * inter, k) * 2 / math.sqrt(k)).to(torch.bfloat16)
+    gu = (x.double() @ w.double().T).to(torch.bfloat16).float()            # the unfused path rounds the product first
+    want = (torch.nn.functional.silu(gu[:, :inter]).to(torch.bfloat16).float() * gu[:, inter:]).to(torch.bfloat16)
+    out = torch.empty(m, inter, dtype=torch.bfloat16, device=DEV)
+    ops().gemm_skinny_swiglu_bf16(x.to(DEV), w.to(DEV), out)
+    close(out, want, torch.bfloat16, what="fused swiglu")
+
+
 def test_linear_dispatch_matches_everywhere():
     """The same product through every route the linear helper can take."""
     from dryft_amd.parts.linear import linear
