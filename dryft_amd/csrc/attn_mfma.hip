@@ -167,15 +167,19 @@ __device__ __forceinline__ void page_update(RowBlock<KB>& st, f32x4 (&s)[4], con
 }
 
 // ---------------------------------------------------------------------------------------------------
-// Many rows per sequence. Grid: (64-row query tiles, query heads); 4 waves of 16 rows each.
-template <int KB, bool FULL>
-__global__ __launch_bounds__(256) void attn_causal_kernel(
+// Many rows per sequence. Grid: (64-position query tiles, query heads / GP); 4 waves of 16 positions each.
+// A wave serves GP query heads that share one kv head: it loads a page of keys and values once and
+// uses it for each of them, which divides the cache traffic by GP.
+template <int KB, bool FULL, int GP>
+__global__ __launch_bounds__(256, 1) void attn_causal_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
     const int* __restrict__ page_table, int max_pages, const int* __restrict__ seq_slot,
     const int* __restrict__ cu_rows, const int* __restrict__ tile_cu, const int* __restrict__ seq_start, int n_seqs,
     bf16_t* __restrict__ out, int n_heads, int n_kv, int head_dim, float scale, int window) {
-  const int tile = blockIdx.x, head = blockIdx.y;
-  if (tile >= tile_cu[n_seqs]) return;
+  const int n_tiles = tile_cu[n_seqs];
+  if ((int)blockIdx.x >= n_tiles) return;
+  const int tile = n_tiles - 1 - blockIdx.x;                  // late tiles see the most keys: start them first
+  const int head0 = blockIdx.y * GP;
   int lo = 0, hi = n_seqs;  // the sequence whose tiles include `tile`
   while (hi - lo > 1) {
     const int mid = (lo + hi) >> 1;
@@ -191,9 +195,11 @@ __global__ __launch_bounds__(256) void attn_causal_kernel(
   const int rows = min(16, q_len - first);
   const bool row_valid = c < rows;
   const int64_t row = (int64_t)cu_rows[seq] + first + c;
-  const int kvh = head / (n_heads / n_kv);
-  RowBlock<KB> st;
-  init_rows<KB>(st, q + (row * n_heads + head) * head_dim, row_valid, head_dim);
+  const int kvh = head0 / (n_heads / n_kv);
+  RowBlock<KB> st[GP];
+#pragma unroll
+  for (int hh = 0; hh < GP; ++hh)
+    init_rows<KB>(st[hh], q + (row * n_heads + head0 + hh) * head_dim, row_valid, head_dim);
   const int pos0 = seq_start[seq] + first;                    // position of the wave's first row
   const int pos_row = row_valid ? pos0 + c : -1;              // an absent row sees nothing
   const int lo_row = window > 0 ? max(0, pos_row - window + 1) : 0;
@@ -201,25 +207,41 @@ __global__ __launch_bounds__(256) void attn_causal_kernel(
   const int hi_wave = pos0 + rows - 1;
   const float scale_log2 = scale * 1.44269504088896340736f;
   const int64_t page_elems = (int64_t)PAGE_TOKENS * head_dim;
-  for (int pg = lo_wave / PAGE_TOKENS; pg <= hi_wave / PAGE_TOKENS; ++pg) {
-    const int page = page_table[(int64_t)slot * max_pages + pg];
-    if (page < 0) continue;
-    PageK<KB> kf;
-    PageV<KB> vf;
-    load_page_k<KB, FULL>(kf, k_pages + ((int64_t)page * n_kv + kvh) * page_elems, head_dim);
-    load_page_v<KB, FULL>(vf, v_pages + ((int64_t)page * n_kv + kvh) * page_elems, head_dim);
-    f32x4 s[4];
-    page_scores<KB>(s, kf, st);
-    page_update<KB>(st, s, vf, head_dim, scale_log2, pg * PAGE_TOKENS, lo_row, pos_row);
+  const int* table = page_table + (int64_t)slot * max_pages;
+  const int pg_last = hi_wave / PAGE_TOKENS;
+  int pg = lo_wave / PAGE_TOKENS;
+  int page = table[pg];
+  PageK<KB> kf;
+  PageV<KB> vf;
+  if (page >= 0) load_page_k<KB, FULL>(kf, k_pages + ((int64_t)page * n_kv + kvh) * page_elems, head_dim);
+  for (; pg <= pg_last; ++pg) {
+    const int page_next = pg < pg_last ? table[pg + 1] : -1;
+    if (page >= 0) {
+      load_page_v<KB, FULL>(vf, v_pages + ((int64_t)page * n_kv + kvh) * page_elems, head_dim);
+      f32x4 s[GP][4];
+#pragma unroll
+      for (int hh = 0; hh < GP; ++hh) page_scores<KB>(s[hh], kf, st[hh]);
+      if (page_next >= 0)
+        load_page_k<KB, FULL>(kf, k_pages + ((int64_t)page_next * n_kv + kvh) * page_elems, head_dim);
+#pragma unroll
+      for (int hh = 0; hh < GP; ++hh)
+        page_update<KB>(st[hh], s[hh], vf, head_dim, scale_log2, pg * PAGE_TOKENS, lo_row, pos_row);
+    } else if (page_next >= 0) {
+      load_page_k<KB, FULL>(kf, k_pages + ((int64_t)page_next * n_kv + kvh) * page_elems, head_dim);
+    }
+    page = page_next;
   }
   if (!row_valid) return;
-  const float inv = 1.f / st.l;
-  bf16_t* o = out + (row * n_heads + head) * head_dim;
 #pragma unroll
-  for (int dt = 0; dt < 2 * KB; ++dt) {
-    if (FULL || 16 * dt < head_dim) {
+  for (int hh = 0; hh < GP; ++hh) {
+    const float inv = 1.f / st[hh].l;
+    bf16_t* o = out + (row * n_heads + head0 + hh) * head_dim;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) o[16 * dt + 4 * g + i] = float_to_bf16(st.o[dt][i] * inv);
+    for (int dt = 0; dt < 2 * KB; ++dt) {
+      if (FULL || 16 * dt < head_dim) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[16 * dt + 4 * g + i] = float_to_bf16(st[hh].o[dt][i] * inv);
+      }
     }
   }
 }
@@ -371,27 +393,44 @@ static int head_shape_ok(int n_heads, int n_kv, int head_dim) {
   return head_dim > 0 && head_dim % 16 == 0 && head_dim <= 256 && n_kv > 0 && n_heads % n_kv == 0;
 }
 
+template <int GP>
+static int launch_causal(const void* q, const void* k_pages, const void* v_pages, const int* page_table, int max_pages,
+                         const int* seq_slot, const int* cu_rows, const int* tile_cu, const int* seq_start, int n_seqs,
+                         int max_tiles, void* out, int n_heads, int n_kv, int head_dim, float scale, int window,
+                         hipStream_t stream) {
+  dim3 grid(max_tiles, n_heads / GP), block(256);
+  if (head_dim % 32 == 0) {
+    DISPATCH_KB(head_dim / 32,
+                hipLaunchKernelGGL((attn_causal_kernel<KB, true, GP>), grid, block, 0, stream, (const bf16_t*)q,
+                                   (const bf16_t*)k_pages, (const bf16_t*)v_pages, page_table, max_pages, seq_slot,
+                                   cu_rows, tile_cu, seq_start, n_seqs, (bf16_t*)out, n_heads, n_kv, head_dim, scale,
+                                   window));
+  } else {
+    DISPATCH_KB((head_dim + 31) / 32,
+                hipLaunchKernelGGL((attn_causal_kernel<KB, false, GP>), grid, block, 0, stream, (const bf16_t*)q,
+                                   (const bf16_t*)k_pages, (const bf16_t*)v_pages, page_table, max_pages, seq_slot,
+                                   cu_rows, tile_cu, seq_start, n_seqs, (bf16_t*)out, n_heads, n_kv, head_dim, scale,
+                                   window));
+  }
+  return DRYFT_LAUNCH_CHECK();
+}
+
 DRYFT_API int dryft_attn_causal_bf16(const void* q, const void* k_pages, const void* v_pages, const int* page_table,
                                      int max_pages, const int* seq_slot, const int* cu_rows, const int* tile_cu,
                                      const int* seq_start, int n_seqs, int max_tiles, void* out, int n_heads,
                                      int n_kv, int head_dim, float scale, int window, hipStream_t stream) {
   if (n_seqs <= 0 || max_tiles <= 0) return 0;
   if (!head_shape_ok(n_heads, n_kv, head_dim)) return -1;
-  dim3 grid(max_tiles, n_heads), block(256);
-  if (head_dim % 32 == 0) {
-    DISPATCH_KB(head_dim / 32,
-                hipLaunchKernelGGL((attn_causal_kernel<KB, true>), grid, block, 0, stream, (const bf16_t*)q,
-                                   (const bf16_t*)k_pages, (const bf16_t*)v_pages, page_table, max_pages, seq_slot,
-                                   cu_rows, tile_cu, seq_start, n_seqs, (bf16_t*)out, n_heads, n_kv, head_dim, scale,
-                                   window));
-  } else {
-    DISPATCH_KB((head_dim + 31) / 32,
-                hipLaunchKernelGGL((attn_causal_kernel<KB, false>), grid, block, 0, stream, (const bf16_t*)q,
-                                   (const bf16_t*)k_pages, (const bf16_t*)v_pages, page_table, max_pages, seq_slot,
-                                   cu_rows, tile_cu, seq_start, n_seqs, (bf16_t*)out, n_heads, n_kv, head_dim, scale,
-                                   window));
-  }
-  return DRYFT_LAUNCH_CHECK();
+  const int group = n_heads / n_kv;
+  // heads of one group served together: the largest of 4, 2, 1 that divides the group (and fits the registers)
+  if (group % 4 == 0 && head_dim <= 128)
+    return launch_causal<4>(q, k_pages, v_pages, page_table, max_pages, seq_slot, cu_rows, tile_cu, seq_start, n_seqs,
+                            max_tiles, out, n_heads, n_kv, head_dim, scale, window, stream);
+  if (group % 2 == 0 && head_dim <= 128)
+    return launch_causal<2>(q, k_pages, v_pages, page_table, max_pages, seq_slot, cu_rows, tile_cu, seq_start, n_seqs,
+                            max_tiles, out, n_heads, n_kv, head_dim, scale, window, stream);
+  return launch_causal<1>(q, k_pages, v_pages, page_table, max_pages, seq_slot, cu_rows, tile_cu, seq_start, n_seqs,
+                          max_tiles, out, n_heads, n_kv, head_dim, scale, window, stream);
 }
 
 DRYFT_API int dryft_attn_split_bf16(const void* q, const void* k_pages, const void* v_pages, const int* page_table,
