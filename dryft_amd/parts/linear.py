@@ -5,11 +5,12 @@ engine/dryft_qwen3/model.py:153, 179-180, 237, 258-261). Here:
 
 * float32: this library's own kernel, plain multiply-adds, so the 32-bit path has no
   reduced-precision matrix mode anywhere;
-* bfloat16, at most 64 rows (decoding and the output head): this library's
-  weight-streaming matrix-core kernel, which can leave its result as float32 partial
-  sums over K for the consumer to add;
-* bfloat16, many rows (prompts): the vendor library through ``torch.mm``, as in the
-  reference; sizes it or the skinny kernel cannot take go to the plain kernel.
+* bfloat16, at most 16 rows (decoding at small batch) and the output head up to 64 rows:
+  this library's weight-streaming matrix-core kernel, which can leave its result as
+  float32 partial sums over K for the consumer to add;
+* bfloat16, more rows (prompts, decoding at large batch): the vendor library through
+  ``torch.mm``, as in the reference; sizes it or the skinny kernel cannot take go to the
+  plain kernel.
 """
 
 from __future__ import annotations
@@ -19,7 +20,8 @@ import torch
 from ..csrc import ops
 from .base import Partials
 
-SKINNY_ROWS = 64
+SKINNY_ROWS = 64          # the most rows the skinny kernel takes
+SKINNY_BEST = 16          # up to here it beats the vendor library on every projection shape measured
 _TARGET_WORKGROUPS = 320   # a little more than one per compute unit
 _BLOCKS_PER_WAVE = 10      # 64-value blocks of K a wave should walk at most
 
@@ -52,7 +54,8 @@ def linear(x: torch.Tensor, w: torch.Tensor, *, out_dtype: torch.dtype | None = 
     out_dtype = out_dtype or x.dtype
     if x.dtype == torch.float32:
         return ops.gemm_tiled(x, w, torch.empty((m, n), dtype=torch.float32, device=x.device))
-    if m <= SKINNY_ROWS and skinny_ok(x, w):
+    library_ok = k % 8 == 0 and n % 8 == 0 and x.is_contiguous()
+    if m <= SKINNY_ROWS and skinny_ok(x, w) and (m <= SKINNY_BEST or out_dtype == torch.float32 or not library_ok):
         ntw, splits = skinny_plan(m, n, k)
         if splits > 1:
             partials = torch.empty((splits, m, n), dtype=torch.float32, device=x.device)
@@ -71,7 +74,7 @@ def linear(x: torch.Tensor, w: torch.Tensor, *, out_dtype: torch.dtype | None = 
                 ops.gemm_skinny_bf16(x[m0:m0 + SKINNY_ROWS], w, out[m0:m0 + SKINNY_ROWS], None, ntw, 1)
             return out
         return ops.gemm_tiled(x, w, out)
-    if k % 8 == 0 and n % 8 == 0 and x.is_contiguous():
+    if library_ok:
         return torch.mm(x, w.t())
     return ops.gemm_tiled(x, w, torch.empty((m, n), dtype=x.dtype, device=x.device))
 
