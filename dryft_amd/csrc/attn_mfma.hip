@@ -31,10 +31,10 @@ __device__ __forceinline__ bf16x8 zero8() {
 
 __device__ __forceinline__ bf16x8 load8(const bf16_t* p) { return *(const bf16x8*)p; }
 
-__device__ __forceinline__ __bf16 to_bf16(float f) {
-  bf16_t b = float_to_bf16(f);
-  return __builtin_bit_cast(__bf16, b.bits);
-}
+__device__ __forceinline__ __bf16 to_bf16(float f) { return (__bf16)f; }
+
+// 2^x by the hardware instruction alone: arguments here are <= 0 or -inf, results below the normal range may flush to 0
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 // State of one wave's 16 rows while it walks over pages of keys.
 template <int KB>  // KB = ceil(head_dim / 32)
@@ -109,40 +109,43 @@ __device__ __forceinline__ void page_scores(f32x4 (&s)[4], const PageK<KB>& f, c
   }
 }
 
-// online softmax over the page's scores, then O^T += V^T P^T
-template <int KB>
-__device__ __forceinline__ void page_update(RowBlock<KB>& st, f32x4 (&s)[4], const PageV<KB>& f, int head_dim,
-                                            float scale_log2, int key0, int lo_row, int hi_row) {
+// Online softmax over the page's scores: updates the row's running maximum and sum, returns the factor by
+// which the row's accumulator must shrink and leaves the probabilities in `p` as the second product's B operand.
+// `scale_log2` turns a raw score into units of log2(e); st.m is kept in those units. MASKED: some key of the
+// page may be hidden from some row (the page of the diagonal, a window's edge, the end of the sequence).
+template <int KB, bool MASKED>
+__device__ __forceinline__ float page_softmax(RowBlock<KB>& st, f32x4 (&s)[4], bf16x8 (&p)[2], float scale_log2,
+                                              int key0, int lo_row, int hi_row) {
   const int g = (threadIdx.x % WAVE) / 16;
   float tile_max = -INFINITY;
 #pragma unroll
   for (int t = 0; t < 4; ++t)
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int j = key0 + 16 * t + 4 * g + i;
-      const float v = (j >= lo_row && j <= hi_row) ? s[t][i] * scale_log2 : -INFINITY;
-      s[t][i] = v;
-      tile_max = fmaxf(tile_max, v);
+      if (MASKED) {
+        const int j = key0 + 16 * t + 4 * g + i;
+        if (!(j >= lo_row && j <= hi_row)) s[t][i] = -INFINITY;
+      }
+      tile_max = fmaxf(tile_max, s[t][i]);
     }
   tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, WAVE));
   tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, WAVE));
-  const float m_new = fmaxf(st.m, tile_max);
-  const float m_safe = m_new == -INFINITY ? 0.f : m_new;
-  const float alpha = exp2f(st.m - m_safe);
+  const float m_new = fmaxf(st.m, tile_max * scale_log2);   // scale > 0, so the maximum commutes with it
+  const float m_safe = m_new == -INFINITY ? 0.f : m_new;    // a row that has seen no key yet stays empty
+  const float alpha = fast_exp2(st.m - m_safe);              // exp2(-inf) = 0 for such a row
   float sum = 0.f;
 #pragma unroll
   for (int t = 0; t < 4; ++t)
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const float p = exp2f(s[t][i] - m_safe);
-      s[t][i] = p;
-      sum += p;
+      const float e = fast_exp2(fmaf(s[t][i], scale_log2, -m_safe));   // -inf stays -inf: e = 0
+      s[t][i] = e;
+      sum += e;
     }
   sum += __shfl_xor(sum, 16, WAVE);
   sum += __shfl_xor(sum, 32, WAVE);
   st.l = st.l * alpha + sum;
   st.m = m_new;
-  bf16x8 p[2];
 #pragma unroll
   for (int h = 0; h < 2; ++h)
 #pragma unroll
@@ -150,9 +153,16 @@ __device__ __forceinline__ void page_update(RowBlock<KB>& st, f32x4 (&s)[4], con
       p[h][i] = to_bf16(s[2 * h][i]);
       p[h][4 + i] = to_bf16(s[2 * h + 1][i]);
     }
+  return alpha;
+}
+
+// O^T = alpha * O^T + V^T P^T
+template <int KB>
+__device__ __forceinline__ void page_values(RowBlock<KB>& st, const bf16x8 (&p)[2], float alpha, const PageV<KB>& f) {
+  const bool rescale = __any(alpha != 1.f);                   // once the maxima have settled nothing changes
 #pragma unroll
   for (int dt = 0; dt < 2 * KB; ++dt) {
-    st.o[dt] *= alpha;
+    if (rescale) st.o[dt] *= alpha;
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
       bf16x8 a;
@@ -166,20 +176,107 @@ __device__ __forceinline__ void page_update(RowBlock<KB>& st, f32x4 (&s)[4], con
   }
 }
 
+template <int KB, bool MASKED>
+__device__ __forceinline__ void page_update_impl(RowBlock<KB>& st, f32x4 (&s)[4], const PageV<KB>& f, float scale_log2,
+                                                 int key0, int lo_row, int hi_row) {
+  bf16x8 p[2];
+  const float alpha = page_softmax<KB, MASKED>(st, s, p, scale_log2, key0, lo_row, hi_row);
+  page_values<KB>(st, p, alpha, f);
+}
+
+// `masked` must be the same for all lanes of the wave.
+template <int KB>
+__device__ __forceinline__ void page_update(RowBlock<KB>& st, f32x4 (&s)[4], const PageV<KB>& f, int head_dim,
+                                            float scale_log2, int key0, int lo_row, int hi_row, bool masked = true) {
+  if (masked)
+    page_update_impl<KB, true>(st, s, f, scale_log2, key0, lo_row, hi_row);
+  else
+    page_update_impl<KB, false>(st, s, f, scale_log2, key0, lo_row, hi_row);
+}
+
 // ---------------------------------------------------------------------------------------------------
-// Many rows per sequence. Grid: (64-position query tiles, query heads / GP); 4 waves of 16 positions each.
-// A wave serves GP query heads that share one kv head: it loads a page of keys and values once and
-// uses it for each of them, which divides the cache traffic by GP.
+// Many rows per sequence. Grid: (pairs of 64-position query tiles, query heads / GP); 4 waves of 16 positions each.
+// A wave serves GP query heads that share one kv head. The workgroup copies each page of keys and values
+// from the cache into LDS once (the next page's loads are in flight while the current one is used), every
+// wave reads its operands from there into registers once per page and uses them for each of its heads.
+// LDS rows are padded by 16 bytes so that the 16 lanes that read 16 different rows hit different banks.
+#define K_PAD 8
+#define V_PAD 8
+
+template <int KB, bool FULL>
+__device__ __forceinline__ void lds_page_k(PageK<KB>& f, const bf16_t* k_lds, int head_dim) {
+  const int lane = threadIdx.x % WAVE, c = lane % 16, g = lane / 16;
+#pragma unroll
+  for (int t = 0; t < 4; ++t)
+#pragma unroll
+    for (int kb = 0; kb < KB; ++kb) {
+      const int d = FULL ? 32 * kb + 8 * g : min(32 * kb + 8 * g, head_dim - 8);
+      f.k[t][kb] = load8(k_lds + (16 * t + c) * (head_dim + K_PAD) + d);
+    }
+}
+
+template <int KB, bool FULL>
+__device__ __forceinline__ void lds_page_v(PageV<KB>& f, const bf16_t* v_lds, int head_dim) {
+  const int lane = threadIdx.x % WAVE, c = lane % 16, g = lane / 16;
+#pragma unroll
+  for (int dt = 0; dt < 2 * KB; ++dt)
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int d = FULL ? 16 * dt + c : min(16 * dt + c, head_dim - 1);
+      const bf16_t* vp = v_lds + d * (PAGE_TOKENS + V_PAD) + 32 * h + 4 * g;
+      f.v[dt][h][0] = *(const bf16x4*)vp;
+      f.v[dt][h][1] = *(const bf16x4*)(vp + 16);
+    }
+}
+
+// a page is 8 * head_dim pieces of 16 bytes for the keys and as many for the values; thread t moves pieces t, t+256, ...
+template <int KB>
+struct PageStage {
+  bf16x8 k[KB], v[KB];
+};
+
+template <int KB>
+__device__ __forceinline__ void stage_load(PageStage<KB>& st, const bf16_t* __restrict__ k_page,
+                                           const bf16_t* __restrict__ v_page, int head_dim) {
+  const int pieces = 8 * head_dim;
+#pragma unroll
+  for (int i = 0; i < KB; ++i) {
+    const int j = threadIdx.x + 256 * i;
+    if (j < pieces) {
+      st.k[i] = load8(k_page + 8 * j);
+      st.v[i] = load8(v_page + 8 * j);
+    }
+  }
+}
+
+template <int KB>
+__device__ __forceinline__ void stage_store(const PageStage<KB>& st, bf16_t* k_lds, bf16_t* v_lds, int head_dim) {
+  const int pieces = 8 * head_dim;
+#pragma unroll
+  for (int i = 0; i < KB; ++i) {
+    const int j = threadIdx.x + 256 * i;
+    if (j < pieces) {
+      const int e = 8 * j;                                   // element index within the page
+      *(bf16x8*)(k_lds + (e / head_dim) * (head_dim + K_PAD) + e % head_dim) = st.k[i];
+      *(bf16x8*)(v_lds + (e / PAGE_TOKENS) * (PAGE_TOKENS + V_PAD) + e % PAGE_TOKENS) = st.v[i];
+    }
+  }
+}
+
 template <int KB, bool FULL, int GP>
-__global__ __launch_bounds__(256, 1) void attn_causal_kernel(
+__global__ __launch_bounds__(256, (GP * KB <= 8 && KB <= 4) ? 2 : 1) void attn_causal_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
     const int* __restrict__ page_table, int max_pages, const int* __restrict__ seq_slot,
     const int* __restrict__ cu_rows, const int* __restrict__ tile_cu, const int* __restrict__ seq_start, int n_seqs,
     bf16_t* __restrict__ out, int n_heads, int n_kv, int head_dim, float scale, int window) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   const int n_tiles = tile_cu[n_seqs];
-  if ((int)blockIdx.x >= n_tiles) return;
-  const int tile = n_tiles - 1 - blockIdx.x;                  // late tiles see the most keys: start them first
   const int head0 = blockIdx.y * GP;
+  // A tile late in a sequence sees many keys, an early one few. Every workgroup takes one tile from each end
+  // of the list, so all of them have about the same work.
+  for (int half = 0; half < 2; ++half) {
+  const int tile = half == 0 ? n_tiles - 1 - (int)blockIdx.x : (int)blockIdx.x;
+  if (tile < 0 || tile >= n_tiles || (half == 1 && tile >= n_tiles - 1 - (int)blockIdx.x)) continue;
   int lo = 0, hi = n_seqs;  // the sequence whose tiles include `tile`
   while (hi - lo > 1) {
     const int mid = (lo + hi) >> 1;
@@ -187,12 +284,15 @@ __global__ __launch_bounds__(256, 1) void attn_causal_kernel(
   }
   while (lo + 1 < n_seqs && tile_cu[lo + 1] <= tile) ++lo;
   const int seq = lo, slot = seq_slot[seq];
-  if (slot < 0) return;
+  if (slot < 0) continue;                                     // the whole workgroup skips the tile together
+  __syncthreads();                                            // the previous tile's pages are no longer read
+  const int k_elems = PAGE_TOKENS * (head_dim + K_PAD), v_elems = head_dim * (PAGE_TOKENS + V_PAD);
+  bf16_t* const smem = (bf16_t*)lds_raw;    // [2][64][D+8] keys, then [2][D][64+8] values
   const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE, c = lane % 16, g = lane / 16;
   const int q_len = cu_rows[seq + 1] - cu_rows[seq];
-  const int first = (tile - tile_cu[seq]) * 64 + 16 * wave;   // first of the wave's rows within the sequence
-  if (first >= q_len) return;
-  const int rows = min(16, q_len - first);
+  const int tile_first = (tile - tile_cu[seq]) * 64;          // first row of the tile within the sequence
+  const int first = tile_first + 16 * wave;                   // first of the wave's rows
+  const int rows = max(0, min(16, q_len - first));            // a wave past the sequence's end has none
   const bool row_valid = c < rows;
   const int64_t row = (int64_t)cu_rows[seq] + first + c;
   const int kvh = head0 / (n_heads / n_kv);
@@ -200,50 +300,74 @@ __global__ __launch_bounds__(256, 1) void attn_causal_kernel(
 #pragma unroll
   for (int hh = 0; hh < GP; ++hh)
     init_rows<KB>(st[hh], q + (row * n_heads + head0 + hh) * head_dim, row_valid, head_dim);
-  const int pos0 = seq_start[seq] + first;                    // position of the wave's first row
+  const int pos_tile = seq_start[seq] + tile_first;           // position of the tile's first row
+  const int pos0 = pos_tile + 16 * wave;
   const int pos_row = row_valid ? pos0 + c : -1;              // an absent row sees nothing
   const int lo_row = window > 0 ? max(0, pos_row - window + 1) : 0;
   const int lo_wave = window > 0 ? max(0, pos0 - window + 1) : 0;
-  const int hi_wave = pos0 + rows - 1;
+  const int hi_wave = pos0 + rows - 1;                        // below lo_wave for a wave without rows
+  const int lo_tile = window > 0 ? max(0, pos_tile - window + 1) : 0;
+  const int hi_tile = pos_tile + min(64, q_len - tile_first) - 1;
   const float scale_log2 = scale * 1.44269504088896340736f;
   const int64_t page_elems = (int64_t)PAGE_TOKENS * head_dim;
   const int* table = page_table + (int64_t)slot * max_pages;
-  const int pg_last = hi_wave / PAGE_TOKENS;
-  int pg = lo_wave / PAGE_TOKENS;
-  int page = table[pg];
-  PageK<KB> kf;
-  PageV<KB> vf;
-  if (page >= 0) load_page_k<KB, FULL>(kf, k_pages + ((int64_t)page * n_kv + kvh) * page_elems, head_dim);
-  for (; pg <= pg_last; ++pg) {
-    const int page_next = pg < pg_last ? table[pg + 1] : -1;
-    if (page >= 0) {
-      load_page_v<KB, FULL>(vf, v_pages + ((int64_t)page * n_kv + kvh) * page_elems, head_dim);
-      f32x4 s[GP][4];
+  const int pg_first = lo_tile / PAGE_TOKENS, pg_last = hi_tile / PAGE_TOKENS;
+  PageStage<KB> stage;
+  int page = table[pg_first];
+  if (page >= 0)
+    stage_load<KB>(stage, k_pages + ((int64_t)page * n_kv + kvh) * page_elems,
+                   v_pages + ((int64_t)page * n_kv + kvh) * page_elems, head_dim);
+  for (int pg = pg_first; pg <= pg_last; ++pg) {
+    const int buf = (pg - pg_first) & 1;
+    bf16_t* const k_lds = smem + buf * k_elems;
+    bf16_t* const v_lds = smem + 2 * k_elems + buf * v_elems;
+    if (page >= 0) stage_store<KB>(stage, k_lds, v_lds, head_dim);
+    __syncthreads();   // the page is in LDS; and every wave is done with the buffer the next page will overwrite
+    const int page_now = page;
+    page = pg < pg_last ? table[pg + 1] : -1;
+    if (page >= 0)
+      stage_load<KB>(stage, k_pages + ((int64_t)page * n_kv + kvh) * page_elems,
+                     v_pages + ((int64_t)page * n_kv + kvh) * page_elems, head_dim);
+    const int key0 = pg * PAGE_TOKENS;
+    if (page_now >= 0 && key0 <= hi_wave && key0 + PAGE_TOKENS > lo_wave) {   // some row of the wave sees some key
+      // every key of the page is seen by every row of the wave unless the page reaches past the wave's first row,
+      // starts before a window's edge, or the wave has fewer than 16 rows
+      const bool masked = key0 + PAGE_TOKENS - 1 > pos0 || rows < 16 ||
+                          (window > 0 && key0 < pos0 + 15 - window + 1);
+      bf16x8 p[GP][2];
+      float alpha[GP];
+      {
+        PageK<KB> kf;                      // the keys are dead once every head has its probabilities,
+        lds_page_k<KB, FULL>(kf, k_lds, head_dim);
 #pragma unroll
-      for (int hh = 0; hh < GP; ++hh) page_scores<KB>(s[hh], kf, st[hh]);
-      if (page_next >= 0)
-        load_page_k<KB, FULL>(kf, k_pages + ((int64_t)page_next * n_kv + kvh) * page_elems, head_dim);
+        for (int hh = 0; hh < GP; ++hh) {
+          f32x4 s[4];
+          page_scores<KB>(s, kf, st[hh]);
+          alpha[hh] = masked ? page_softmax<KB, true>(st[hh], s, p[hh], scale_log2, key0, lo_row, pos_row)
+                             : page_softmax<KB, false>(st[hh], s, p[hh], scale_log2, key0, lo_row, pos_row);
+        }
+      }
+      PageV<KB> vf;                        // so the values can take their registers
+      lds_page_v<KB, FULL>(vf, v_lds, head_dim);
 #pragma unroll
-      for (int hh = 0; hh < GP; ++hh)
-        page_update<KB>(st[hh], s[hh], vf, head_dim, scale_log2, pg * PAGE_TOKENS, lo_row, pos_row);
-    } else if (page_next >= 0) {
-      load_page_k<KB, FULL>(kf, k_pages + ((int64_t)page_next * n_kv + kvh) * page_elems, head_dim);
+      for (int hh = 0; hh < GP; ++hh) page_values<KB>(st[hh], p[hh], alpha[hh], vf);
     }
-    page = page_next;
   }
-  if (!row_valid) return;
+  if (row_valid) {
 #pragma unroll
-  for (int hh = 0; hh < GP; ++hh) {
-    const float inv = 1.f / st[hh].l;
-    bf16_t* o = out + (row * n_heads + head0 + hh) * head_dim;
+    for (int hh = 0; hh < GP; ++hh) {
+      const float inv = 1.f / st[hh].l;
+      bf16_t* o = out + (row * n_heads + head0 + hh) * head_dim;
 #pragma unroll
-    for (int dt = 0; dt < 2 * KB; ++dt) {
-      if (FULL || 16 * dt < head_dim) {
+      for (int dt = 0; dt < 2 * KB; ++dt) {
+        if (FULL || 16 * dt < head_dim) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) o[16 * dt + 4 * g + i] = float_to_bf16(st[hh].o[dt][i] * inv);
+          for (int i = 0; i < 4; ++i) o[16 * dt + 4 * g + i] = float_to_bf16(st[hh].o[dt][i] * inv);
+        }
       }
     }
   }
+  }  // the two tiles of the workgroup
 }
 
 // ---------------------------------------------------------------------------------------------------
@@ -398,20 +522,25 @@ static int launch_causal(const void* q, const void* k_pages, const void* v_pages
                          const int* seq_slot, const int* cu_rows, const int* tile_cu, const int* seq_start, int n_seqs,
                          int max_tiles, void* out, int n_heads, int n_kv, int head_dim, float scale, int window,
                          hipStream_t stream) {
-  dim3 grid(max_tiles, n_heads / GP), block(256);
-  if (head_dim % 32 == 0) {
-    DISPATCH_KB(head_dim / 32,
-                hipLaunchKernelGGL((attn_causal_kernel<KB, true, GP>), grid, block, 0, stream, (const bf16_t*)q,
-                                   (const bf16_t*)k_pages, (const bf16_t*)v_pages, page_table, max_pages, seq_slot,
-                                   cu_rows, tile_cu, seq_start, n_seqs, (bf16_t*)out, n_heads, n_kv, head_dim, scale,
-                                   window));
-  } else {
-    DISPATCH_KB((head_dim + 31) / 32,
-                hipLaunchKernelGGL((attn_causal_kernel<KB, false, GP>), grid, block, 0, stream, (const bf16_t*)q,
-                                   (const bf16_t*)k_pages, (const bf16_t*)v_pages, page_table, max_pages, seq_slot,
-                                   cu_rows, tile_cu, seq_start, n_seqs, (bf16_t*)out, n_heads, n_kv, head_dim, scale,
-                                   window));
+  dim3 grid((max_tiles + 1) / 2, n_heads / GP), block(256);
+  // two pages of keys [64][D+8] and two of values [D][64+8]
+  const size_t lds = 2 * ((size_t)PAGE_TOKENS * (head_dim + K_PAD) + (size_t)head_dim * (PAGE_TOKENS + V_PAD)) * 2;
+#define LAUNCH_CAUSAL(FULLV)                                                                                       \
+  {                                                                                                                \
+    auto kernel = attn_causal_kernel<KB, FULLV, GP>;                                                               \
+    if (lds > 64 * 1024 &&                                                                                          \
+        hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) \
+      return -1;                                                                                                   \
+    hipLaunchKernelGGL(kernel, grid, block, lds, stream, (const bf16_t*)q, (const bf16_t*)k_pages,                 \
+                       (const bf16_t*)v_pages, page_table, max_pages, seq_slot, cu_rows, tile_cu, seq_start, n_seqs, \
+                       (bf16_t*)out, n_heads, n_kv, head_dim, scale, window);                                      \
   }
+  if (head_dim % 32 == 0) {
+    DISPATCH_KB(head_dim / 32, LAUNCH_CAUSAL(true));
+  } else {
+    DISPATCH_KB((head_dim + 31) / 32, LAUNCH_CAUSAL(false));
+  }
+#undef LAUNCH_CAUSAL
   return DRYFT_LAUNCH_CHECK();
 }
 
@@ -422,11 +551,11 @@ DRYFT_API int dryft_attn_causal_bf16(const void* q, const void* k_pages, const v
   if (n_seqs <= 0 || max_tiles <= 0) return 0;
   if (!head_shape_ok(n_heads, n_kv, head_dim)) return -1;
   const int group = n_heads / n_kv;
-  // heads of one group served together: the largest of 4, 2, 1 that divides the group (and fits the registers)
-  if (group % 4 == 0 && head_dim <= 128)
-    return launch_causal<4>(q, k_pages, v_pages, page_table, max_pages, seq_slot, cu_rows, tile_cu, seq_start, n_seqs,
-                            max_tiles, out, n_heads, n_kv, head_dim, scale, window, stream);
-  if (group % 2 == 0 && head_dim <= 128)
+  // Heads of one kv group can be served together (one load of each page for several heads), at the price of
+  // registers, so of fewer workgroups per compute unit. It pays once there are workgroups enough to fill the
+  // chip twice over even so.
+  const int pairs = (max_tiles + 1) / 2;
+  if (group % 2 == 0 && head_dim <= 128 && (int64_t)pairs * (n_heads / 2) >= 1024)
     return launch_causal<2>(q, k_pages, v_pages, page_table, max_pages, seq_slot, cu_rows, tile_cu, seq_start, n_seqs,
                             max_tiles, out, n_heads, n_kv, head_dim, scale, window, stream);
   return launch_causal<1>(q, k_pages, v_pages, page_table, max_pages, seq_slot, cu_rows, tile_cu, seq_start, n_seqs,

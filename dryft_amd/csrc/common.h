@@ -15,16 +15,11 @@ struct bf16_t {
 
 __device__ __forceinline__ float bf16_to_float(bf16_t v) { return __uint_as_float(((uint32_t)v.bits) << 16); }
 
-// round to nearest, ties to even; NaN stays NaN
+// round to nearest, ties to even (v_cvt_pk_bf16_f32 on gfx950)
 __device__ __forceinline__ bf16_t float_to_bf16(float f) {
-  uint32_t u = __float_as_uint(f);
+  const __bf16 h = (__bf16)f;
   bf16_t r;
-  if ((u & 0x7fffffffu) > 0x7f800000u) {
-    r.bits = (uint16_t)((u >> 16) | 0x0040u);
-  } else {
-    u += 0x7fffu + ((u >> 16) & 1u);
-    r.bits = (uint16_t)(u >> 16);
-  }
+  r.bits = __builtin_bit_cast(uint16_t, h);
   return r;
 }
 
