@@ -37,6 +37,31 @@ template <typename T> __device__ __forceinline__ float rounded_as(float v);
 template <> __device__ __forceinline__ float rounded_as<float>(float v) { return v; }
 template <> __device__ __forceinline__ float rounded_as<bf16_t>(float v) { return bf16_to_float(float_to_bf16(v)); }
 
+// Eight contiguous values at a 16-byte aligned address, as floats.
+typedef __attribute__((ext_vector_type(4))) float vf4;
+typedef __attribute__((ext_vector_type(4))) uint32_t vu4;
+
+__device__ __forceinline__ void load8_as_float(const float* p, float (&v)[8]) {
+  const vf4 a = *(const vf4*)p, b = *(const vf4*)(p + 4);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) { v[i] = a[i]; v[4 + i] = b[i]; }
+}
+__device__ __forceinline__ void load8_as_float(const bf16_t* p, float (&v)[8]) {
+  const vu4 a = *(const vu4*)p;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) { v[2 * i] = __uint_as_float(a[i] << 16); v[2 * i + 1] = __uint_as_float(a[i] & 0xffff0000u); }
+}
+__device__ __forceinline__ void store8_from_float(float* p, const float (&v)[8]) {
+  *(vf4*)p = vf4{v[0], v[1], v[2], v[3]};
+  *(vf4*)(p + 4) = vf4{v[4], v[5], v[6], v[7]};
+}
+__device__ __forceinline__ void store8_from_float(bf16_t* p, const float (&v)[8]) {
+  vu4 a;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) a[i] = (uint32_t)float_to_bf16(v[2 * i]).bits | ((uint32_t)float_to_bf16(v[2 * i + 1]).bits << 16);
+  *(vu4*)p = a;
+}
+
 // A vector whose dtype is only known at run time (norm weights: bfloat16, or float32 if stored so).
 __device__ __forceinline__ float load_vector(const void* p, int i, int is_f32) {
   return is_f32 ? ((const float*)p)[i] : bf16_to_float(((const bf16_t*)p)[i]);

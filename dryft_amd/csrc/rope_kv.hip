@@ -21,12 +21,12 @@ __global__ void qk_norm_rope_kv_kernel(const T* __restrict__ qkv, int64_t qkv_st
                                        const int* __restrict__ row_slot, const int* __restrict__ row_pos,
                                        T* __restrict__ q_out, T* __restrict__ k_pages, T* __restrict__ v_pages,
                                        const int* __restrict__ page_table, int max_pages, int write_kv, int n_heads,
-                                       int n_kv, int head_dim) {
+                                       int n_kv, int head_dim, int skip_v, int first_job) {
   __shared__ float normed[4][MAX_HEAD_DIM];
   const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
   const int64_t row = blockIdx.x;
-  const int job = blockIdx.y * 4 + wave;  // [0,nH): q heads; [nH,nH+nKV): k heads; then v heads
-  if (job >= n_heads + 2 * n_kv) return;
+  const int job = first_job + blockIdx.y * 4 + wave;  // [0,nH): q heads; [nH,nH+nKV): k heads; then v heads
+  if (job >= n_heads + (skip_v ? 1 : 2) * n_kv) return;
   const int slot = row_slot[row];
   const int pos = row_pos[row];
   const bool is_q = job < n_heads, is_k = !is_q && job < n_heads + n_kv;
@@ -88,6 +88,142 @@ __global__ void qk_norm_rope_kv_kernel(const T* __restrict__ qkv, int64_t qkv_st
   }
 }
 
+// The same for head widths of 32, 64, 128 or 256 rotated over their full width: a head is spread over
+// head_dim / 8 lanes that hold 8 contiguous values each, moved with 16-byte loads and stores; the sum of squares
+// and the exchange with the rotation partner (the lane head_dim / 16 away) go through lane shuffles. Value
+// heads are not handled here.
+template <typename T>
+__global__ __launch_bounds__(256) void qk_norm_rope_vec_kernel(const T* __restrict__ qkv, int64_t qkv_stride,
+                                                               const void* __restrict__ q_w, const void* __restrict__ k_w,
+                                                               int w_f32, int has_norm, float eps,
+                                                               const T* __restrict__ cos_t, const T* __restrict__ sin_t,
+                                                               const int* __restrict__ row_slot,
+                                                               const int* __restrict__ row_pos, T* __restrict__ q_out,
+                                                               T* __restrict__ k_pages, T* __restrict__ v_pages,
+                                                               const int* __restrict__ page_table, int max_pages,
+                                                               int write_kv, int with_v, int n_heads, int n_kv,
+                                                               int head_dim) {
+  const int lph = head_dim / 8;                        // lanes per head: 4, 8, 16 or 32
+  const int64_t row = blockIdx.x;
+  const int job = blockIdx.y * (256 / lph) + threadIdx.x / lph;
+  const int part = threadIdx.x % lph;
+  const int jobs = n_heads + (write_kv ? (with_v ? 2 : 1) * n_kv : 0);   // q heads, k heads, then v heads
+  const bool live_job = job < jobs;                    // lanes of a dead job still take part in the shuffles
+  const bool is_v = job >= n_heads + n_kv;
+  const int slot = row_slot[row], pos = row_pos[row];
+  const bool is_q = job < n_heads;
+  float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  if (live_job && slot >= 0) load8_as_float(qkv + row * qkv_stride + (int64_t)job * head_dim + 8 * part, v);
+  if (has_norm) {                                      // (value heads run through it too; their result is not used)
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) ss += v[j] * v[j];
+    for (int o = lph / 2; o > 0; o >>= 1) ss += __shfl_xor(ss, o, WAVE);
+    const float inv = rsqrtf(ss / (float)head_dim + eps);
+    const void* w = is_q ? q_w : k_w;
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      v[j] = rounded_as<T>(rounded_as<T>(v[j] * inv) * (live_job ? load_vector(w, 8 * part + j, w_f32) : 0.f));
+  }
+  float other[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) other[j] = __shfl_xor(v[j], lph / 2, WAVE);
+  if (!live_job) return;
+  if (is_v) {                                          // copied as it is, transposed into its page
+    if (slot < 0) return;
+    const int page = page_of(page_table, max_pages, slot, pos);
+    if (page < 0) return;
+    T* vd = v_pages + (((int64_t)page * n_kv + (job - n_heads - n_kv)) * head_dim + 8 * part) * PAGE_TOKENS +
+            pos % PAGE_TOKENS;
+    const T* vs = qkv + row * qkv_stride + (int64_t)job * head_dim + 8 * part;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) vd[(int64_t)j * PAGE_TOKENS] = vs[j];
+    return;
+  }
+  T* dst;
+  if (is_q) {
+    dst = q_out + (row * n_heads + job) * head_dim + 8 * part;
+    if (slot < 0) {
+      const float z[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      store8_from_float(dst, z);
+      return;
+    }
+  } else {
+    if (slot < 0) return;
+    const int page = page_of(page_table, max_pages, slot, pos);
+    if (page < 0) return;
+    dst = k_pages + (((int64_t)page * n_kv + (job - n_heads)) * PAGE_TOKENS + pos % PAGE_TOKENS) * head_dim + 8 * part;
+  }
+  const int half_lanes = lph / 2;
+  const bool first = part < half_lanes;
+  float c[8], sn[8];
+  const int64_t at = (int64_t)pos * (head_dim / 2) + 8 * (first ? part : part - half_lanes);
+  load8_as_float(cos_t + at, c);
+  load8_as_float(sin_t + at, sn);
+  float o[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const float a = rounded_as<T>(v[j] * c[j]), b = rounded_as<T>(other[j] * sn[j]);
+    o[j] = first ? a - b : a + b;                       // x1*c - x2*s ; x2*c + x1*s
+  }
+  store8_from_float(dst, o);
+}
+
+// Values of a step with many rows: a workgroup takes 64 consecutive rows of one kv head, turns the tile in LDS
+// and writes runs of 8 consecutive positions with one 16-byte store where they lie together in a page. (The
+// per-row kernel above writes a row's values 128 bytes apart.) head_dim must be a multiple of 8.
+#define V_TILE_ROWS 64
+#define V_TILE_LD (V_TILE_ROWS + 8)
+template <typename T>
+__global__ __launch_bounds__(256) void v_tile_write_kernel(const T* __restrict__ qkv, int64_t qkv_stride, int v_col0,
+                                                           const int* __restrict__ row_slot,
+                                                           const int* __restrict__ row_pos, T* __restrict__ v_pages,
+                                                           const int* __restrict__ page_table, int max_pages,
+                                                           int n_rows, int n_kv, int head_dim) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char v_tile_raw[];
+  __shared__ int64_t dest[V_TILE_ROWS];
+  T* tile = (T*)v_tile_raw;                                 // [head_dim][V_TILE_LD]: already transposed
+  const int r0 = blockIdx.x * V_TILE_ROWS, kvh = blockIdx.y;
+  const int rows = min(V_TILE_ROWS, n_rows - r0);
+  const int chunks = head_dim / 8;
+  for (int e = threadIdx.x; e < V_TILE_ROWS * chunks; e += blockDim.x) {
+    const int t = e / chunks, ch = e % chunks;
+    float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    if (t < rows) load8_as_float(qkv + (int64_t)(r0 + t) * qkv_stride + v_col0 + kvh * head_dim + 8 * ch, v);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) store_from_float(tile + (8 * ch + j) * V_TILE_LD + t, v[j]);
+  }
+  if (threadIdx.x < V_TILE_ROWS) {
+    int64_t where = -1;
+    if ((int)threadIdx.x < rows) {
+      const int slot = row_slot[r0 + threadIdx.x], pos = row_pos[r0 + threadIdx.x];
+      if (slot >= 0) {
+        const int page = page_of(page_table, max_pages, slot, pos);
+        if (page >= 0) where = ((int64_t)page * n_kv + kvh) * head_dim * PAGE_TOKENS + pos % PAGE_TOKENS;
+      }
+    }
+    dest[threadIdx.x] = where;
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < head_dim * (V_TILE_ROWS / 8); e += blockDim.x) {
+    const int d = e / (V_TILE_ROWS / 8), t0 = (e % (V_TILE_ROWS / 8)) * 8;
+    const int64_t w0 = dest[t0];
+    bool together = w0 >= 0 && (w0 % 8) == 0;
+#pragma unroll
+    for (int j = 1; j < 8; ++j) together = together && dest[t0 + j] == w0 + j;
+    const T* src = tile + d * V_TILE_LD + t0;
+    if (together) {
+      float v[8];
+      load8_as_float(src, v);
+      store8_from_float(v_pages + w0 + (int64_t)d * PAGE_TOKENS, v);
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        if (dest[t0 + j] >= 0) v_pages[dest[t0 + j] + (int64_t)d * PAGE_TOKENS] = src[j];
+    }
+  }
+}
+
 DRYFT_API int dryft_qk_norm_rope_kv(const void* qkv, int64_t qkv_stride, const void* q_w, const void* k_w, int w_f32,
                                     int has_norm, float eps, const void* cos_t, const void* sin_t, int rot,
                                     const int* row_slot, const int* row_pos, void* q_out, void* k_pages,
@@ -95,17 +231,56 @@ DRYFT_API int dryft_qk_norm_rope_kv(const void* qkv, int64_t qkv_stride, const v
                                     int n_heads, int n_kv, int head_dim, int is_f32, hipStream_t stream) {
   if (n_rows <= 0) return 0;
   if (head_dim > MAX_HEAD_DIM || rot > head_dim || (rot & 1)) return -1;
-  const int jobs = n_heads + 2 * n_kv;
-  dim3 grid(n_rows, (jobs + 3) / 4), block(256);
+  const bool aligned = (((uintptr_t)qkv | (uintptr_t)q_out | (uintptr_t)k_pages | (uintptr_t)v_pages |
+                         (uintptr_t)cos_t | (uintptr_t)sin_t) & 15) == 0 && qkv_stride % 8 == 0;
+  // many rows: the values go through the tile kernel
+  const int skip_v = (write_kv && n_rows >= 32 && head_dim % 8 == 0 && aligned) ? 1 : 0;
+  const bool vec = aligned && rot == head_dim && (head_dim == 32 || head_dim == 64 || head_dim == 128 || head_dim == 256);
+  if (vec) {
+    const int lph = head_dim / 8, per_block = 256 / lph;
+    const int with_v = (write_kv && !skip_v) ? 1 : 0;
+    const int qk_jobs = n_heads + (write_kv ? (with_v ? 2 : 1) * n_kv : 0);
+    dim3 qgrid(n_rows, (qk_jobs + per_block - 1) / per_block);
+    if (is_f32)
+      hipLaunchKernelGGL(qk_norm_rope_vec_kernel<float>, qgrid, dim3(256), 0, stream, (const float*)qkv, qkv_stride, q_w,
+                         k_w, w_f32, has_norm, eps, (const float*)cos_t, (const float*)sin_t, row_slot, row_pos,
+                         (float*)q_out, (float*)k_pages, (float*)v_pages, page_table, max_pages, write_kv, with_v, n_heads, n_kv,
+                         head_dim);
+    else
+      hipLaunchKernelGGL(qk_norm_rope_vec_kernel<bf16_t>, qgrid, dim3(256), 0, stream, (const bf16_t*)qkv, qkv_stride,
+                         q_w, k_w, w_f32, has_norm, eps, (const bf16_t*)cos_t, (const bf16_t*)sin_t, row_slot, row_pos,
+                         (bf16_t*)q_out, (bf16_t*)k_pages, (bf16_t*)v_pages, page_table, max_pages, write_kv, with_v, n_heads,
+                         n_kv, head_dim);
+    int rc = DRYFT_LAUNCH_CHECK();
+    if (rc) return rc;
+  }
+  // the per-row kernel takes everything when the vector kernel does not apply
+  const int first_job = 0;
+  const int jobs = n_heads + (skip_v ? 1 : 2) * n_kv;
+  if (!vec) {
+  dim3 grid(n_rows, (jobs - first_job + 3) / 4), block(256);
   if (is_f32)
     hipLaunchKernelGGL(qk_norm_rope_kv_kernel<float>, grid, block, 0, stream, (const float*)qkv, qkv_stride, q_w, k_w,
                        w_f32, has_norm, eps, (const float*)cos_t, (const float*)sin_t, rot, row_slot, row_pos,
                        (float*)q_out, (float*)k_pages, (float*)v_pages, page_table, max_pages, write_kv, n_heads, n_kv,
-                       head_dim);
+                       head_dim, skip_v, first_job);
   else
     hipLaunchKernelGGL(qk_norm_rope_kv_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)qkv, qkv_stride, q_w,
                        k_w, w_f32, has_norm, eps, (const bf16_t*)cos_t, (const bf16_t*)sin_t, rot, row_slot, row_pos,
                        (bf16_t*)q_out, (bf16_t*)k_pages, (bf16_t*)v_pages, page_table, max_pages, write_kv, n_heads,
-                       n_kv, head_dim);
+                       n_kv, head_dim, skip_v, first_job);
+  }
+  int rc = DRYFT_LAUNCH_CHECK();
+  if (rc || !skip_v) return rc;
+  dim3 vgrid((n_rows + V_TILE_ROWS - 1) / V_TILE_ROWS, n_kv);
+  const int v_col0 = (n_heads + n_kv) * head_dim;
+  if (is_f32)
+    hipLaunchKernelGGL(v_tile_write_kernel<float>, vgrid, dim3(256), head_dim * V_TILE_LD * 4, stream,
+                       (const float*)qkv, qkv_stride, v_col0, row_slot, row_pos, (float*)v_pages, page_table, max_pages,
+                       n_rows, n_kv, head_dim);
+  else
+    hipLaunchKernelGGL(v_tile_write_kernel<bf16_t>, vgrid, dim3(256), head_dim * V_TILE_LD * 2, stream,
+                       (const bf16_t*)qkv, qkv_stride, v_col0, row_slot, row_pos, (bf16_t*)v_pages, page_table,
+                       max_pages, n_rows, n_kv, head_dim);
   return DRYFT_LAUNCH_CHECK();
 }
