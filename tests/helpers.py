@@ -29,7 +29,15 @@ TINY_C = {
     "rope_theta": 50000.0, "rms_norm_eps": 3e-6, "tie_word_embeddings": False, "max_position_embeddings": 2048,
     "hidden_act": "silu", "attention_bias": False,
 }
-TINY = {"A": (TINY_A, dict(seed=11, norm_std=0.0, std=0.02)), "B": (TINY_B, dict(seed=22, norm_std=0.1, std=0.02)),
+# a fourth one whose widths are not multiples of 8 (no 16-byte rows) and whose vocabulary is a prime: it takes
+# the plain kernels where the vector and matrix-core kernels refuse the sizes; one kv head per query head
+TINY_D = {
+    "architectures": ["Qwen3ForCausalLM"], "model_type": "qwen3", "num_hidden_layers": 2, "hidden_size": 100,
+    "num_attention_heads": 5, "num_key_value_heads": 5, "head_dim": 16, "intermediate_size": 108, "vocab_size": 257,
+    "rope_theta": 20000.0, "rms_norm_eps": 2e-6, "tie_word_embeddings": True, "max_position_embeddings": 1024,
+    "hidden_act": "silu", "attention_bias": False,
+}
+TINY = {"D": (TINY_D, dict(seed=44, norm_std=0.1, std=0.04)), "A": (TINY_A, dict(seed=11, norm_std=0.0, std=0.02)), "B": (TINY_B, dict(seed=22, norm_std=0.1, std=0.02)),
         "C": (TINY_C, dict(seed=33, norm_std=0.1, std=0.05))}
 
 

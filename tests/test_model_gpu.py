@@ -90,7 +90,7 @@ def cases(tmp_path_factory):
     return out
 
 
-CASE_NAMES = ["A", "B", "C", "C_sharp", "A_sharp"]
+CASE_NAMES = ["A", "B", "C", "D", "C_sharp", "A_sharp"]
 
 
 def replay(engine, records):
