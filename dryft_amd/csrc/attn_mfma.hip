@@ -377,16 +377,85 @@ __global__ __launch_bounds__(256, (GP * KB <= 8 && KB <= 4) ? 2 : 1) void attn_c
 // product so that memory stays busy, and merge their results in LDS. Each split writes an
 // unnormalised partial (o, m, l); the combine kernel merges splits in a fixed order, so results do
 // not depend on timing.
+// One q or k head of one row, as the fused projection left it: RMSNorm over the head (optional), then the
+// rotation of pairs (j, j + rot/2), with the same roundings as the stand-alone kernel (rope_kv.hip). One wave;
+// `tmp` is the wave's own LDS scratch of head_dim floats (head_dim <= 256). The result is written as bfloat16 to
+// `dst` (in LDS) and, if given, to `dst2` (in global memory). All loads are issued before anything waits on them.
+__device__ __forceinline__ void wave_norm_rope(const bf16_t* __restrict__ src, const void* __restrict__ w, int w_f32,
+                                               int has_norm, float eps, const bf16_t* __restrict__ cos_t,
+                                               const bf16_t* __restrict__ sin_t, int rot, int pos, int head_dim,
+                                               float* tmp, bf16_t* dst, bf16_t* dst2) {
+  const int lane = threadIdx.x % WAVE;
+  const int half = rot / 2;
+  float x[4], cs[4], sn[4], wt[4];
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const int i = lane + WAVE * u;
+    const bool in = i < head_dim;
+    x[u] = in ? bf16_to_float(src[i]) : 0.f;
+    wt[u] = (in && has_norm) ? load_vector(w, i, w_f32) : 1.f;
+    const int j = i < half ? i : i - half;
+    cs[u] = (in && i < rot) ? bf16_to_float(cos_t[(int64_t)pos * half + j]) : 1.f;
+    sn[u] = (in && i < rot) ? bf16_to_float(sin_t[(int64_t)pos * half + j]) : 0.f;
+  }
+  if (has_norm) {
+    float ss = 0.f;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) ss += x[u] * x[u];
+    ss = wave_sum(ss);
+    const float inv = rsqrtf(ss / (float)head_dim + eps);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) x[u] = rounded_as<bf16_t>(rounded_as<bf16_t>(x[u] * inv) * wt[u]);
+  }
+#pragma unroll
+  for (int u = 0; u < 4; ++u)
+    if (lane + WAVE * u < head_dim) tmp[lane + WAVE * u] = x[u];
+  __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "workgroup");
+  __builtin_amdgcn_wave_barrier();
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const int i = lane + WAVE * u;
+    if (i >= head_dim) continue;
+    float o = x[u];
+    if (i < rot) {
+      const float other = tmp[i < half ? i + half : i - half];
+      const float a = rounded_as<bf16_t>(o * cs[u]), b = rounded_as<bf16_t>(other * sn[u]);
+      o = i < half ? a - b : a + b;
+    }
+    const bf16_t r = float_to_bf16(o);
+    dst[i] = r;
+    if (dst2 != nullptr) dst2[i] = r;
+  }
+}
+
+// What the fused form of the split kernel needs to do the work of the norm/rotation/append kernel itself.
+struct FusedQKV {
+  const bf16_t* qkv;       // [rows, stride]: q heads, k heads, v heads of each row; null: q is given ready
+  int64_t stride;
+  const void* q_w;
+  const void* k_w;
+  int w_f32, has_norm;
+  float eps;
+  const bf16_t* cos_t;
+  const bf16_t* sin_t;
+  int rot;
+  int write_kv;
+};
+
 #define SPLIT_WAVES 4
+#define SPLIT_MAX_D 256
 
 template <int KB, bool FULL>
 __global__ __launch_bounds__(64 * SPLIT_WAVES, 2) void attn_split_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
     const int* __restrict__ page_table, int max_pages, const int* __restrict__ seq_slot,
     const int* __restrict__ cu_rows, const int* __restrict__ kv_len, float* __restrict__ part_o,
-    float* __restrict__ part_ml, int n_heads, int n_kv, int head_dim, float scale, int window, int n_splits) {
+    float* __restrict__ part_ml, int n_heads, int n_kv, int head_dim, float scale, int window, int n_splits,
+    FusedQKV fused, bf16_t* __restrict__ k_pages_w, bf16_t* __restrict__ v_pages_w) {
   __shared__ float merge_o[SPLIT_WAVES][16][32 * KB + 1];
   __shared__ float merge_ml[SPLIT_WAVES][16][2];
+  __shared__ __attribute__((aligned(16))) bf16_t q_lds[16][32 * KB];
+  __shared__ __attribute__((aligned(16))) bf16_t kv_new[2][32 * KB];   // the row's own key (normed, rotated) and value
   const int seq = blockIdx.x, split = blockIdx.z;
   const int group = n_heads / n_kv, blocks = (group + 15) / 16;
   const int kvh = blockIdx.y / blocks, hb = blockIdx.y % blocks;
@@ -395,38 +464,110 @@ __global__ __launch_bounds__(64 * SPLIT_WAVES, 2) void attn_split_kernel(
   const int head = kvh * group + hb * 16 + c;
   const bool row_valid = hb * 16 + c < group;
   const int64_t row = cu_rows[seq];
-  RowBlock<KB> st;
-  init_rows<KB>(st, q + (row * n_heads + head) * head_dim, row_valid && slot >= 0, head_dim);
+  // pages of this split, taken by its waves in turn
+  int pos = 0, lo = 0, pg = 0, pg1 = -1, pg_hi = 0, pg_first = 0;
+  const int* table = page_table + (int64_t)max(slot, 0) * max_pages;
   if (slot >= 0) {
-    const int pos = kv_len[seq] - 1;                           // the row's own position; its key is cached
-    const int lo = window > 0 ? max(0, pos - window + 1) : 0;
-    const int pg_lo = lo / PAGE_TOKENS, pg_hi = pos / PAGE_TOKENS;
+    pos = kv_len[seq] - 1;                                     // the row's own position
+    lo = window > 0 ? max(0, pos - window + 1) : 0;
+    const int pg_lo = lo / PAGE_TOKENS;
+    pg_hi = pos / PAGE_TOKENS;
     const int per = (pg_hi - pg_lo + n_splits) / n_splits;     // ceil(pages / splits)
-    const int pg1 = min(pg_hi, pg_lo + split * per + per - 1);
-    const float scale_log2 = scale * 1.44269504088896340736f;
-    const int* table = page_table + (int64_t)slot * max_pages;
-    const int64_t page_elems = (int64_t)PAGE_TOKENS * head_dim;
-    int pg = pg_lo + split * per + wave;
-    PageK<KB> kf;
-    PageV<KB> vf;
-    int page = pg <= pg1 ? table[pg] : -1;
-    if (page >= 0) load_page_k<KB, FULL>(kf, k_pages + ((int64_t)page * n_kv + kvh) * page_elems, head_dim);
-    while (pg <= pg1) {
-      const int pg_next = pg + SPLIT_WAVES;
-      const int page_next = pg_next <= pg1 ? table[pg_next] : -1;
-      if (page >= 0) {
-        load_page_v<KB, FULL>(vf, v_pages + ((int64_t)page * n_kv + kvh) * page_elems, head_dim);
-        f32x4 s[4];
-        page_scores<KB>(s, kf, st);
-        if (page_next >= 0)
-          load_page_k<KB, FULL>(kf, k_pages + ((int64_t)page_next * n_kv + kvh) * page_elems, head_dim);
-        page_update<KB>(st, s, vf, head_dim, scale_log2, pg * PAGE_TOKENS, lo, pos);
-      } else if (page_next >= 0) {
-        load_page_k<KB, FULL>(kf, k_pages + ((int64_t)page_next * n_kv + kvh) * page_elems, head_dim);
+    pg1 = min(pg_hi, pg_lo + split * per + per - 1);
+    pg_first = pg_lo + split * per;
+    pg = pg_first + wave;
+  }
+  const float scale_log2 = scale * 1.44269504088896340736f;
+  const int64_t page_elems = (int64_t)PAGE_TOKENS * head_dim;
+  PageK<KB> kf;
+  PageV<KB> vf;
+  int page = pg <= pg1 ? table[pg] : -1;
+  if (page >= 0) load_page_k<KB, FULL>(kf, k_pages + ((int64_t)page * n_kv + kvh) * page_elems, head_dim);
+  RowBlock<KB> st;
+  const bool fused_on = fused.qkv != nullptr;
+  // exactly one split has the row's own page among its pages (splits past the sequence's end have none)
+  const bool owns_last = fused_on && slot >= 0 && pg_first <= pg_hi && pg1 == pg_hi;
+  if (fused_on) {
+    // The row's q, k and v come straight from the projection (the first page of keys is already on its way). The
+    // waves norm and rotate the query heads this workgroup serves into LDS. The workgroup whose pages include the
+    // row's own position also norms and rotates the new key, appends key and value to the cache, and keeps both in
+    // LDS: the wave that reads that page puts them into its operands itself, so nothing has to wait for memory.
+    float* tmp = &merge_o[wave][0][0];                          // free until the merge
+    if (slot >= 0) {
+      const bf16_t* src_row = fused.qkv + row * fused.stride;
+      for (int r = wave; r < group; r += SPLIT_WAVES)
+        wave_norm_rope(src_row + (int64_t)(kvh * group + r) * head_dim, fused.q_w, fused.w_f32, fused.has_norm,
+                       fused.eps, fused.cos_t, fused.sin_t, fused.rot, pos, head_dim, tmp, &q_lds[r][0], nullptr);
+      if (owns_last) {
+        const int page_last = table[pg_hi];
+        const int64_t base = ((int64_t)max(page_last, 0) * n_kv + kvh) * page_elems;
+        const int at = pos % PAGE_TOKENS;
+        const bool store = fused.write_kv && page_last >= 0;
+        if (wave == SPLIT_WAVES - 1)
+          wave_norm_rope(src_row + (int64_t)(n_heads + kvh) * head_dim, fused.k_w, fused.w_f32, fused.has_norm,
+                         fused.eps, fused.cos_t, fused.sin_t, fused.rot, pos, head_dim, tmp, &kv_new[0][0],
+                         store ? k_pages_w + base + (int64_t)at * head_dim : nullptr);
+        if (wave == SPLIT_WAVES - 2) {
+          const bf16_t* vs = src_row + (int64_t)(n_heads + n_kv + kvh) * head_dim;
+          for (int i = lane; i < head_dim; i += WAVE) {
+            const bf16_t v = vs[i];
+            kv_new[1][i] = v;
+            if (store) v_pages_w[base + (int64_t)i * PAGE_TOKENS + at] = v;
+          }
+        }
       }
-      pg = pg_next;
-      page = page_next;
     }
+    __syncthreads();
+    init_rows<KB>(st, &q_lds[c][0], row_valid && slot >= 0, head_dim);
+  } else {
+    init_rows<KB>(st, q + (row * n_heads + head) * head_dim, row_valid && slot >= 0, head_dim);
+  }
+  while (pg <= pg1) {
+    const int pg_next = pg + SPLIT_WAVES;
+    const int page_next = pg_next <= pg1 ? table[pg_next] : -1;
+    if (page >= 0) {
+      load_page_v<KB, FULL>(vf, v_pages + ((int64_t)page * n_kv + kvh) * page_elems, head_dim);
+      if (fused_on && fused.write_kv && pg == pg_hi) {
+        // this page holds the row's own position, whose key and value may not have reached memory yet: take them
+        // from LDS. Key `at` is row at%16 of key tile at/16; as a value it is one element of one lane group.
+        const int at = pos % PAGE_TOKENS;
+        if (c == at % 16) {
+#pragma unroll
+          for (int t = 0; t < 4; ++t)
+            if (t == at / 16) {
+#pragma unroll
+              for (int kb = 0; kb < KB; ++kb) {
+                const int d = FULL ? 32 * kb + 8 * g : min(32 * kb + 8 * g, head_dim - 8);
+                kf.k[t][kb] = load8(&kv_new[0][d]);
+              }
+            }
+        }
+        const int rem = at % 32, hsel = at / 32, half_sel = rem / 16, gsel = (rem % 16) / 4, isel = rem % 4;
+        if (g == gsel) {
+#pragma unroll
+          for (int dt = 0; dt < 2 * KB; ++dt) {
+            const int d = FULL ? 16 * dt + c : min(16 * dt + c, head_dim - 1);
+            const __bf16 nv = __builtin_bit_cast(__bf16, kv_new[1][d].bits);
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+              for (int hf = 0; hf < 2; ++hf)
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                  if (h == hsel && hf == half_sel && i == isel) vf.v[dt][h][hf][i] = nv;
+          }
+        }
+      }
+      f32x4 s[4];
+      page_scores<KB>(s, kf, st);
+      if (page_next >= 0)
+        load_page_k<KB, FULL>(kf, k_pages + ((int64_t)page_next * n_kv + kvh) * page_elems, head_dim);
+      page_update<KB>(st, s, vf, head_dim, scale_log2, pg * PAGE_TOKENS, lo, pos);
+    } else if (page_next >= 0) {
+      load_page_k<KB, FULL>(kf, k_pages + ((int64_t)page_next * n_kv + kvh) * page_elems, head_dim);
+    }
+    pg = pg_next;
+    page = page_next;
   }
   // merge the four waves' results: o = sum_w 2^(m_w - m) o_w, l likewise
 #pragma unroll
@@ -562,28 +703,53 @@ DRYFT_API int dryft_attn_causal_bf16(const void* q, const void* k_pages, const v
                           max_tiles, out, n_heads, n_kv, head_dim, scale, window, stream);
 }
 
-DRYFT_API int dryft_attn_split_bf16(const void* q, const void* k_pages, const void* v_pages, const int* page_table,
-                                    int max_pages, const int* seq_slot, const int* cu_rows, const int* kv_len,
-                                    int n_seqs, float* part_o, float* part_ml, int n_splits, void* out, int n_heads,
-                                    int n_kv, int head_dim, float scale, int window, hipStream_t stream) {
+static int launch_split(const void* q, const void* k_pages, const void* v_pages, const int* page_table, int max_pages,
+                        const int* seq_slot, const int* cu_rows, const int* kv_len, int n_seqs, float* part_o,
+                        float* part_ml, int n_splits, void* out, int n_heads, int n_kv, int head_dim, float scale,
+                        int window, FusedQKV fused, hipStream_t stream) {
   if (n_seqs <= 0) return 0;
   if (!head_shape_ok(n_heads, n_kv, head_dim) || n_splits < 1 || n_splits > COMBINE_MAX_SPLITS) return -1;
   const int group = n_heads / n_kv, blocks = (group + 15) / 16;
+  if (fused.qkv != nullptr && (blocks != 1 || fused.rot > head_dim || (fused.rot & 1))) return -1;
   dim3 grid(n_seqs, n_kv * blocks, n_splits), block(64 * SPLIT_WAVES);
+#define LAUNCH_SPLIT(FULLV)                                                                                        \
+  hipLaunchKernelGGL((attn_split_kernel<KB, FULLV>), grid, block, 0, stream, (const bf16_t*)q, (const bf16_t*)k_pages, \
+                     (const bf16_t*)v_pages, page_table, max_pages, seq_slot, cu_rows, kv_len, part_o, part_ml,    \
+                     n_heads, n_kv, head_dim, scale, window, n_splits, fused, (bf16_t*)k_pages, (bf16_t*)v_pages)
   if (head_dim % 32 == 0) {
-    DISPATCH_KB(head_dim / 32,
-                hipLaunchKernelGGL((attn_split_kernel<KB, true>), grid, block, 0, stream, (const bf16_t*)q,
-                                   (const bf16_t*)k_pages, (const bf16_t*)v_pages, page_table, max_pages, seq_slot,
-                                   cu_rows, kv_len, part_o, part_ml, n_heads, n_kv, head_dim, scale, window, n_splits));
+    DISPATCH_KB(head_dim / 32, LAUNCH_SPLIT(true));
   } else {
-    DISPATCH_KB((head_dim + 31) / 32,
-                hipLaunchKernelGGL((attn_split_kernel<KB, false>), grid, block, 0, stream, (const bf16_t*)q,
-                                   (const bf16_t*)k_pages, (const bf16_t*)v_pages, page_table, max_pages, seq_slot,
-                                   cu_rows, kv_len, part_o, part_ml, n_heads, n_kv, head_dim, scale, window, n_splits));
+    DISPATCH_KB((head_dim + 31) / 32, LAUNCH_SPLIT(false));
   }
+#undef LAUNCH_SPLIT
   int rc = DRYFT_LAUNCH_CHECK();
   if (rc) return rc;
   hipLaunchKernelGGL(attn_combine_kernel, dim3(n_seqs, n_heads), dim3(128), 0, stream, part_o, part_ml, seq_slot,
                      cu_rows, (bf16_t*)out, n_heads, head_dim, n_splits);
   return DRYFT_LAUNCH_CHECK();
+}
+
+DRYFT_API int dryft_attn_split_bf16(const void* q, const void* k_pages, const void* v_pages, const int* page_table,
+                                    int max_pages, const int* seq_slot, const int* cu_rows, const int* kv_len,
+                                    int n_seqs, float* part_o, float* part_ml, int n_splits, void* out, int n_heads,
+                                    int n_kv, int head_dim, float scale, int window, hipStream_t stream) {
+  FusedQKV none = {};
+  return launch_split(q, k_pages, v_pages, page_table, max_pages, seq_slot, cu_rows, kv_len, n_seqs, part_o, part_ml,
+                      n_splits, out, n_heads, n_kv, head_dim, scale, window, none, stream);
+}
+
+// The same with the work of the norm/rotation/append kernel folded in: `qkv` is the fused projection's output
+// for one row per sequence. Takes kv groups of at most 16 query heads.
+DRYFT_API int dryft_attn_decode_fused_bf16(const void* qkv, int64_t qkv_stride, const void* q_w, const void* k_w,
+                                           int w_f32, int has_norm, float eps, const void* cos_t, const void* sin_t,
+                                           int rot, int write_kv, void* k_pages, void* v_pages, const int* page_table,
+                                           int max_pages, const int* seq_slot, const int* cu_rows, const int* kv_len,
+                                           int n_seqs, float* part_o, float* part_ml, int n_splits, void* out,
+                                           int n_heads, int n_kv, int head_dim, float scale, int window,
+                                           hipStream_t stream) {
+  if (qkv == nullptr) return -1;
+  FusedQKV fused = {(const bf16_t*)qkv, qkv_stride, q_w, k_w, w_f32, has_norm, eps, (const bf16_t*)cos_t,
+                    (const bf16_t*)sin_t, rot, write_kv};
+  return launch_split(nullptr, k_pages, v_pages, page_table, max_pages, seq_slot, cu_rows, kv_len, n_seqs, part_o,
+                      part_ml, n_splits, out, n_heads, n_kv, head_dim, scale, window, fused, stream);
 }

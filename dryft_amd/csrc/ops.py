@@ -28,7 +28,9 @@ _SIGNATURES = {
     "attn_rows": {"dryft_attn_rows": [_P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _F, _I, _I, _P]},
     "attn_mfma": {"dryft_attn_causal_bf16": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _P, _I, _I, _I, _F, _I, _P],
                   "dryft_attn_split_bf16": [_P, _P, _P, _P, _I, _P, _P, _P, _I, _P, _P, _I, _P, _I, _I, _I, _F, _I,
-                                            _P]},
+                                            _P],
+                  "dryft_attn_decode_fused_bf16": [_P, _L, _P, _P, _I, _I, _F, _P, _P, _I, _I, _P, _P, _P, _I, _P, _P,
+                                                   _P, _I, _P, _P, _I, _P, _I, _I, _I, _F, _I, _P]},
     "gemm": {"dryft_gemm_tiled": [_P, _L, _P, _P, _I, _I, _I, _I, _I, _P],
              "dryft_gemm_skinny_bf16": [_P, _L, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
              "dryft_gemm_skinny_swiglu_bf16": [_P, _L, _P, _P, _I, _I, _I, _P],
@@ -277,6 +279,49 @@ def attn_split_bf16(q, k_pages, v_pages, page_table, seq_slot, cu_rows, kv_len, 
         _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(page_table), page_table.shape[1], _ptr(seq_slot), _ptr(cu_rows),
         _ptr(kv_len), n_seqs, _ptr(part_o), _ptr(part_ml), n_splits, _ptr(out), n_heads, n_kv, head_dim, float(scale),
         int(window), _stream()), "attn_split_bf16")
+
+
+def attn_decode_fused_bf16(qkv, q_weight, k_weight, eps: float, cos, sin, rot: int, write_kv: bool, k_pages, v_pages,
+                           page_table, seq_slot, cu_rows, kv_len, n_seqs: int, part_o, part_ml, n_splits: int, out,
+                           n_heads: int, n_kv: int, head_dim: int, scale: float, window: int) -> None:
+    """One row per sequence: q/k norm, rotation, append to the cache and attention in one kernel (plus the combine).
+
+    ``qkv`` is the fused projection's output ``[n_seqs rows, (heads + 2 kv heads) * head_dim]``; row ``i`` belongs to
+    sequence ``i`` (``cu_rows[i] == i``).
+    """
+    _gpu(qkv, "qkv", torch.bfloat16)
+    _gpu(out, "out", torch.bfloat16)
+    need_cols = (n_heads + 2 * n_kv) * head_dim
+    _require(qkv.dim() == 2 and qkv.stride(1) == 1 and qkv.shape[1] >= need_cols and qkv.shape[0] >= n_seqs,
+             f"attn_decode_fused: qkv must be [rows >= {n_seqs}, >= {need_cols}]")
+    _require(out.is_contiguous() and out.numel() >= n_seqs * n_heads * head_dim, "attn_decode_fused: out too small")
+    _require(n_heads // n_kv <= 16, "attn_decode_fused: at most 16 query heads per kv head")
+    _check_pages(k_pages, v_pages, page_table, n_kv, head_dim, torch.bfloat16)
+    has_norm = q_weight is not None
+    w_f32 = 0
+    if has_norm:
+        for name, w in (("q_weight", q_weight), ("k_weight", k_weight)):
+            _gpu(w, name)
+            _require(w.shape == (head_dim,) and w.is_contiguous(), f"{name}: must be [{head_dim}]")
+        _require(q_weight.dtype == k_weight.dtype, "q_weight and k_weight must share a dtype")
+        w_f32 = _float_flag(q_weight, "q_weight")
+    if rot:
+        _require(rot % 2 == 0 and rot <= head_dim, f"rotary width {rot} must be even and at most {head_dim}")
+        for name, t in (("cos", cos), ("sin", sin)):
+            _gpu(t, name, torch.bfloat16)
+            _require(t.dim() == 2 and t.shape[1] == rot // 2 and t.is_contiguous(), f"{name}: must be [positions, {rot // 2}]")
+    for name, t, n in (("seq_slot", seq_slot, n_seqs), ("cu_rows", cu_rows, n_seqs + 1), ("kv_len", kv_len, n_seqs)):
+        _gpu(t, name, torch.int32)
+        _require(t.numel() >= n, f"{name}: needs {n} entries")
+    _gpu(part_o, "part_o", torch.float32)
+    _gpu(part_ml, "part_ml", torch.float32)
+    _require(part_o.numel() >= n_seqs * n_heads * n_splits * head_dim and part_ml.numel() >= n_seqs * n_heads * n_splits * 2,
+             "attn_decode_fused: partial buffers too small")
+    _check(_fn("attn_mfma", "dryft_attn_decode_fused_bf16")(
+        _ptr(qkv), qkv.stride(0), _ptr(q_weight), _ptr(k_weight), w_f32, int(has_norm), float(eps), _ptr(cos), _ptr(sin),
+        int(rot), int(write_kv), _ptr(k_pages), _ptr(v_pages), _ptr(page_table), page_table.shape[1], _ptr(seq_slot),
+        _ptr(cu_rows), _ptr(kv_len), n_seqs, _ptr(part_o), _ptr(part_ml), n_splits, _ptr(out), n_heads, n_kv, head_dim,
+        float(scale), int(window), _stream()), "attn_decode_fused_bf16")
 
 
 # -------------------------------------------------------------------------------------------- gemm

@@ -78,24 +78,32 @@ class GQAAttention(Mixer):
             cos, sin = table.cos, table.sin
             if ctx.max_kv_len > table.n_positions:
                 raise ValueError(f"position tables cover {table.n_positions} positions, the step reaches {ctx.max_kv_len}")
+        window = self.window or 0
+        out = torch.empty((rows, self.n_heads, self.head_dim), dtype=h.dtype, device=h.device)
+        decoding = h.dtype == torch.bfloat16 and ctx.max_q_len == 1
+        if decoding:
+            splits = self.decode_splits(ctx.n_seqs, ctx.max_kv_len)
+            part_o = torch.empty((ctx.n_seqs, self.n_heads, splits, self.head_dim), dtype=torch.float32, device=h.device)
+            part_ml = torch.empty((ctx.n_seqs, self.n_heads, splits, 2), dtype=torch.float32, device=h.device)
+        if decoding and self.n_heads // self.n_kv <= 16:
+            # one token per sequence: norm, rotation, append and attention in one kernel
+            ops.attn_decode_fused_bf16(qkv, self.q_norm, self.k_norm, self.qk_norm_eps or 0.0, cos, sin, self.rotary_dim,
+                                       writes_cache, line.k, line.v, line.page_table, ctx.seq_slot, ctx.cu_rows,
+                                       ctx.kv_len, ctx.n_seqs, part_o, part_ml, splits, out, self.n_heads, self.n_kv,
+                                       self.head_dim, self.scale, window)
+            return linear(out.view(rows, self.q_dim), self.w_o, allow_partials=True)
         q = torch.empty((rows, self.n_heads, self.head_dim), dtype=h.dtype, device=h.device)
         ops.qk_norm_rope_kv(qkv, self.q_norm, self.k_norm, self.qk_norm_eps or 0.0, cos, sin, self.rotary_dim,
                             ctx.row_slot, ctx.row_pos, q, line.k, line.v, line.page_table, writes_cache,
                             self.n_heads, self.n_kv, self.head_dim)
-        out = torch.empty_like(q)
-        window = self.window or 0
-        if h.dtype == torch.bfloat16:
-            if ctx.max_q_len == 1:
-                splits = self.decode_splits(ctx.n_seqs, ctx.max_kv_len)
-                part_o = torch.empty((ctx.n_seqs, self.n_heads, splits, self.head_dim), dtype=torch.float32, device=h.device)
-                part_ml = torch.empty((ctx.n_seqs, self.n_heads, splits, 2), dtype=torch.float32, device=h.device)
-                ops.attn_split_bf16(q, line.k, line.v, line.page_table, ctx.seq_slot, ctx.cu_rows, ctx.kv_len,
-                                    ctx.n_seqs, part_o, part_ml, splits, out, self.n_heads, self.n_kv, self.head_dim,
-                                    self.scale, window)
-            else:
-                ops.attn_causal_bf16(q, line.k, line.v, line.page_table, ctx.seq_slot, ctx.cu_rows, ctx.tile_cu,
-                                     ctx.seq_start, ctx.n_seqs, ctx.max_tiles, out, self.n_heads, self.n_kv,
-                                     self.head_dim, self.scale, window)
+        if decoding:
+            ops.attn_split_bf16(q, line.k, line.v, line.page_table, ctx.seq_slot, ctx.cu_rows, ctx.kv_len,
+                                ctx.n_seqs, part_o, part_ml, splits, out, self.n_heads, self.n_kv, self.head_dim,
+                                self.scale, window)
+        elif h.dtype == torch.bfloat16:
+            ops.attn_causal_bf16(q, line.k, line.v, line.page_table, ctx.seq_slot, ctx.cu_rows, ctx.tile_cu,
+                                 ctx.seq_start, ctx.n_seqs, ctx.max_tiles, out, self.n_heads, self.n_kv,
+                                 self.head_dim, self.scale, window)
         else:
             ops.attn_rows(q, line.k, line.v, line.page_table, ctx.row_slot, ctx.row_pos, out, self.n_heads, self.n_kv,
                           self.head_dim, self.scale, window)

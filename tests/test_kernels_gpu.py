@@ -276,6 +276,56 @@ def test_attn_split_bf16(case, splits):
     run_attention_case(splits, torch.bfloat16, *case)
 
 
+@pytest.mark.parametrize("n_heads,n_kv,D,splits,window", [(32, 8, 128, 3, 0), (6, 3, 48, 1, 0), (4, 2, 16, 2, 0),
+                                                          (16, 1, 64, 4, 0), (8, 2, 32, 2, 50)])
+def test_attn_decode_fused_equals_the_two_kernels(n_heads, n_kv, D, splits, window):
+    """Norm + rotation + append + attention in one kernel gives what the separate kernels give, bit for bit,
+    in the output and in the cache."""
+    torch.manual_seed(n_heads + D)
+    o = ops()
+    lengths = [1, 64, 65, 200, 130]                  # cached tokens after the step (the new one included)
+    B, n_slots, max_pages = len(lengths), 7, 4
+    n_pages = n_slots * max_pages
+    rng = np.random.default_rng(D)
+    table = torch.tensor(rng.permutation(n_pages).reshape(n_slots, max_pages), dtype=torch.int32, device=DEV)
+    slots = [int(x) for x in rng.permutation(n_slots)[:B]]
+    slots[2] = -1                                    # one sequence sits out
+    seq_slot = torch.tensor(slots, dtype=torch.int32, device=DEV)
+    cu = torch.arange(B + 1, dtype=torch.int32, device=DEV)
+    kv_len = torch.tensor(lengths, dtype=torch.int32, device=DEV)
+    row_pos = torch.tensor([n - 1 for n in lengths], dtype=torch.int32, device=DEV)
+    qkv = (2 * torch.randn(B, (n_heads + 2 * n_kv) * D)).to(torch.bfloat16).to(DEV)
+    wq = (1 + 0.1 * torch.randn(D)).to(torch.bfloat16).to(DEV)
+    wk = (1 + 0.1 * torch.randn(D)).to(torch.bfloat16).to(DEV)
+    ang = torch.arange(256).float()[:, None] * (1.0 / (1e4 ** (torch.arange(0, D, 2).float() / D)))[None]
+    cos, sin = ang.cos().to(torch.bfloat16).to(DEV), ang.sin().to(torch.bfloat16).to(DEV)
+    k0 = torch.randn(n_pages, n_kv, 64, D).to(torch.bfloat16).to(DEV)
+    v0 = torch.randn(n_pages, n_kv, D, 64).to(torch.bfloat16).to(DEV)
+    scale = D ** -0.5
+    po = torch.empty(B * n_heads * splits * D, dtype=torch.float32, device=DEV)
+    pml = torch.empty(B * n_heads * splits * 2, dtype=torch.float32, device=DEV)
+    # the two kernels
+    k1, v1 = k0.clone(), v0.clone()
+    q = torch.empty(B, n_heads, D, dtype=torch.bfloat16, device=DEV)
+    out1 = torch.zeros(B, n_heads, D, dtype=torch.bfloat16, device=DEV)
+    o.qk_norm_rope_kv(qkv, wq, wk, 1e-6, cos, sin, D, seq_slot, row_pos, q, k1, v1, table, True, n_heads, n_kv, D)
+    o.attn_split_bf16(q, k1, v1, table, seq_slot, cu, kv_len, B, po, pml, splits, out1, n_heads, n_kv, D, scale, window)
+    # the one kernel
+    k2, v2 = k0.clone(), v0.clone()
+    out2 = torch.zeros(B, n_heads, D, dtype=torch.bfloat16, device=DEV)
+    o.attn_decode_fused_bf16(qkv, wq, wk, 1e-6, cos, sin, D, True, k2, v2, table, seq_slot, cu, kv_len, B, po, pml,
+                             splits, out2, n_heads, n_kv, D, scale, window)
+    assert torch.equal(k1, k2) and torch.equal(v1, v2), "the cache differs"
+    assert not torch.equal(k1, k0), "nothing was appended"
+    assert torch.equal(out1, out2), "the output differs"
+    # a run that only reads the cache leaves it alone
+    k3, v3 = k1.clone(), v1.clone()
+    out3 = torch.zeros_like(out2)
+    o.attn_decode_fused_bf16(qkv, wq, wk, 1e-6, cos, sin, D, False, k3, v3, table, seq_slot, cu, kv_len, B, po, pml,
+                             splits, out3, n_heads, n_kv, D, scale, window)
+    assert torch.equal(k3, k1) and torch.equal(v3, v1) and torch.equal(out3, out2)
+
+
 @pytest.mark.parametrize("kind", ["rows", "causal", 3])
 def test_attention_window(kind):
     tq = 1 if kind == 3 else 90
