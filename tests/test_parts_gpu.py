@@ -408,3 +408,76 @@ def test_layer_named_twice_and_a_run_that_reads_anothers_cache(tmp_path):
     engine.release([slot])
     got = torch.cat(got).cpu()
     assert float((got - want).abs().max()) <= 1e-4 * float(want.abs().max())
+
+
+# ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_windowed_layer_has_storage_of_its_own_and_gives_pages_back(dtype, tmp_path):
+    """Layer 1 of a tiny Qwen3 sees only the last 70 positions: it gets a cache group of its own whose pages are
+    freed as they fall behind the window, and the logits match the plain model with the same window."""
+    from dataclasses import replace
+    from dryft_amd import Engine, register_architecture
+    from dryft_amd.config import LayerSpec, PartSpec, Qwen3Config
+    from dryft_amd.engine.replay import Replayer
+    from dryft_amd.models import known_architectures
+    from dryft_amd.models.qwen3 import qwen3_plan
+    from helpers import TINY_B, collect_positions, make_model_dir, read_model_dir, trace_batches, trace_whole
+    import json
+    WINDOW = 70
+
+    def windowed_plan(cfg):
+        plan = qwen3_plan(cfg)
+        layers = list(plan.layers)
+        parts = dict(layers[1].parts)
+        parts["mixer"] = PartSpec(parts["mixer"].kind, dict(parts["mixer"].args, window=WINDOW), parts["mixer"].tensors)
+        layers[1] = LayerSpec(layers[1].block, parts)
+        return replace(plan, layers=tuple(layers))
+
+    if "Qwen3Windowed" not in known_architectures():
+        register_architecture("Qwen3Windowed", Qwen3Config, windowed_plan)
+    path = make_model_dir(str(tmp_path / "m"), TINY_B, seed=6, norm_std=0.1)
+    with open(os.path.join(path, "config.json"), "w") as f:
+        json.dump(dict(TINY_B, architectures=["Qwen3Windowed"]), f)
+    raw, weights = read_model_dir(path)
+    w = {k: v.double() for k, v in weights.items()}
+
+    def plain_logits(toks):
+        T, d, eps = len(toks), raw["head_dim"], raw["rms_norm_eps"]
+        cos, sin = P.rope_tables(d, raw["rope_theta"], T, torch.float64)
+        x = w["model.embed_tokens.weight"][torch.tensor(toks)]
+        for i in range(raw["num_hidden_layers"]):
+            p = f"model.layers.{i}."
+            h = P.rms_norm(x, w[p + "input_layernorm.weight"], eps)
+            q = P.apply_rope(P.rms_norm((h @ w[p + "self_attn.q_proj.weight"].T).view(T, 8, d), w[p + "self_attn.q_norm.weight"], eps), cos, sin)
+            k = P.apply_rope(P.rms_norm((h @ w[p + "self_attn.k_proj.weight"].T).view(T, 2, d), w[p + "self_attn.k_norm.weight"], eps), cos, sin)
+            v = (h @ w[p + "self_attn.v_proj.weight"].T).view(T, 2, d)
+            o = P.causal_gqa_attention(q, k, v, 1 / math.sqrt(d), WINDOW if i == 1 else None)
+            x = x + o.reshape(T, -1) @ w[p + "self_attn.o_proj.weight"].T
+            x = x + P.swiglu(P.rms_norm(x, w[p + "post_attention_layernorm.weight"], eps), w, p)
+        return (P.rms_norm(x, w["model.norm.weight"], eps) @ w["lm_head.weight"].T).float()
+
+    engine = Engine(path, dtype=dtype, max_batch=4, max_len=512, max_tokens=64 * 14, use_graph=False)
+    groups = engine.cache.kv_groups
+    assert len(groups) == 2 and sorted(len(g.lines) for g in groups) == [1, 2]
+    windowed = next(g for g in groups if g.need.window == WINDOW)
+    full = next(g for g in groups if g.need.window is None)
+    reqs = {"a": random_tokens(300, raw["vocab_size"], seed=1), "b": random_tokens(75, raw["vocab_size"], seed=2)}
+    want = {rid: plain_logits(toks) for rid, toks in reqs.items()}
+    limit = 1e-4 if dtype == "float32" else 3e-2
+    for records in (list(trace_whole(reqs)), list(trace_batches([{"a": (reqs["a"], 230), "b": (reqs["b"], 70)}]))):
+        r = Replayer(engine)
+        outputs = {}
+        least_free = windowed.table.pool.n_pages
+        for rec in records:
+            lg = r.run_step(rec)
+            if lg is not None and lg.shape[0]:
+                outputs[rec["step"]] = lg.float().cpu()
+            least_free = min(least_free, windowed.table.pool.free_count)
+            for slot in r.slot_of.values():        # a live sequence never holds more than the window needs
+                assert len(windowed.table.held_pages(slot)) <= (WINDOW + 63) // 64 + 1
+        for (rid, pos), row in collect_positions(records, outputs).items():
+            ref = want[rid]
+            err = float((row - ref[pos]).abs().max()) / float(ref.abs().max())
+            assert err <= limit, f"{rid}@{pos}: {err}"
+        assert windowed.table.pool.free_count == windowed.table.pool.n_pages
+        assert full.table.pool.free_count == full.table.pool.n_pages
