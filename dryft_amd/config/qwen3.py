@@ -3,7 +3,7 @@
 Field names are the ``config.json`` key names. The keys read and the options
 refused follow the reference (engine/dryft_qwen3/config.py:137-155): read are
 the sizes, ``rms_norm_eps``, ``rope_theta``, ``tie_word_embeddings`` and
-``max_position_embeddings``; ``hidden_act`` must be ``silu``, ``attention_bias``
+``max_position_embeddings`` (optional here: it only bounds lengths); ``hidden_act`` must be ``silu``, ``attention_bias``
 false, ``rope_scaling`` null, ``use_sliding_window`` false, and the q heads a
 multiple of the kv heads. ``head_dim`` falls back to ``hidden_size //
 num_attention_heads`` (config.py:142). Unlike the reference no checkpoint is
@@ -30,7 +30,7 @@ class Qwen3Config:
     rms_norm_eps: float
     rope_theta: float
     tie_word_embeddings: bool
-    max_position_embeddings: int
+    max_position_embeddings: int | None = None      # only bounds lengths; absent: no bound from the model
 
     architecture = "Qwen3ForCausalLM"
 
@@ -68,7 +68,8 @@ class Qwen3Config:
             rms_norm_eps=r.number("rms_norm_eps"),
             rope_theta=r.number("rope_theta"),
             tie_word_embeddings=r.boolean("tie_word_embeddings", default=False),
-            max_position_embeddings=r.integer("max_position_embeddings"),
+            max_position_embeddings=(r.integer("max_position_embeddings")
+                                     if raw.get("max_position_embeddings") is not None else None),
         )
         r.require("hidden_act", lambda v: v == "silu", "silu", "only 'silu' is supported")
         r.require("attention_bias", lambda v: v is False, False, "projection biases are not supported")
@@ -84,7 +85,7 @@ class Qwen3Config:
 
     def to_dict(self) -> dict[str, Any]:
         """The ``config.json`` content that reads back as this configuration."""
-        d = asdict(self)
+        d = {k: v for k, v in asdict(self).items() if v is not None}
         d.update(architectures=[self.architecture], model_type="qwen3", hidden_act="silu",
                  attention_bias=False, rope_scaling=None, use_sliding_window=False,
                  torch_dtype="bfloat16")

@@ -22,12 +22,16 @@ class Architecture:
 
 
 _REGISTRY: dict[str, Architecture] = {}
+_MODEL_TYPES: dict[str, str] = {}      # config.json "model_type" -> architecture name, for files without "architectures"
 
 
-def register_architecture(name: str, config_class: Any, plan: Callable[[Any], ModelPlan]) -> None:
+def register_architecture(name: str, config_class: Any, plan: Callable[[Any], ModelPlan],
+                          model_type: str | None = None) -> None:
     if name in _REGISTRY:
         raise ValueError(f"architecture {name!r} is already registered")
     _REGISTRY[name] = Architecture(name, config_class, plan)
+    if model_type is not None:
+        _MODEL_TYPES[model_type] = name
 
 
 def known_architectures() -> list[str]:
@@ -36,6 +40,8 @@ def known_architectures() -> list[str]:
 
 def resolve_architecture(raw_config: dict[str, Any]) -> Architecture:
     names = raw_config.get("architectures")
+    if names is None and raw_config.get("model_type") in _MODEL_TYPES:
+        names = [_MODEL_TYPES[raw_config["model_type"]]]          # a config.json that only says model_type
     if not isinstance(names, list) or not names or not isinstance(names[0], str):
         raise ConfigError("config.json", [
             f"architectures: expected a list naming the model class, got {names!r}; known: {known_architectures()}"])

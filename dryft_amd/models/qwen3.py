@@ -62,7 +62,7 @@ def qwen3_plan(cfg: Qwen3Config) -> ModelPlan:
     )
 
 
-register_architecture(Qwen3Config.architecture, Qwen3Config, qwen3_plan)
+register_architecture(Qwen3Config.architecture, Qwen3Config, qwen3_plan, model_type="qwen3")
 
 _PRESET_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "presets")
 

@@ -29,6 +29,16 @@ def test_head_dim_defaults_to_hidden_over_heads():
     assert Qwen3Config.from_dict(raw).tie_word_embeddings is False      # reference default (config.py:153)
 
 
+def test_optional_keys_and_model_type_fallback():
+    raw = {k: v for k, v in TINY_B.items() if k not in ("max_position_embeddings", "hidden_act", "attention_bias",
+                                                        "architectures")}
+    cfg = Qwen3Config.from_dict(raw)
+    assert cfg.max_position_embeddings is None and "max_position_embeddings" not in cfg.to_dict()
+    assert resolve_architecture(raw).name == "Qwen3ForCausalLM"          # found through model_type "qwen3"
+    del raw["num_key_value_heads"]
+    assert Qwen3Config.from_dict(raw).num_key_value_heads == 8            # as many kv heads as query heads
+
+
 def test_one_error_lists_every_problem():
     raw = dict(TINY_B, hidden_act="gelu", attention_bias=True, rope_scaling={"type": "yarn"}, use_sliding_window=True,
                num_key_value_heads=3, rms_norm_eps="tiny")
