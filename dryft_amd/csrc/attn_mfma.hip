@@ -378,54 +378,65 @@ __global__ __launch_bounds__(256, (GP * KB <= 8 && KB <= 4) ? 2 : 1) void attn_c
 // unnormalised partial (o, m, l); the combine kernel merges splits in a fixed order, so results do
 // not depend on timing.
 // One q or k head of one row, as the fused projection left it: RMSNorm over the head (optional), then the
-// rotation of pairs (j, j + rot/2), with the same roundings as the stand-alone kernel (rope_kv.hip). One wave;
-// `tmp` is the wave's own LDS scratch of head_dim floats (head_dim <= 256). The result is written as bfloat16 to
-// `dst` (in LDS) and, if given, to `dst2` (in global memory). All loads are issued before anything waits on them.
-__device__ __forceinline__ void wave_norm_rope(const bf16_t* __restrict__ src, const void* __restrict__ w, int w_f32,
-                                               int has_norm, float eps, const bf16_t* __restrict__ cos_t,
-                                               const bf16_t* __restrict__ sin_t, int rot, int pos, int head_dim,
-                                               float* tmp, bf16_t* dst, bf16_t* dst2) {
+// rotation of pairs (j, j + rot/2), with the same roundings as the stand-alone kernel (rope_kv.hip). One wave, in
+// two halves so that a caller can put other loads between them: `head_load` issues every load (head_dim <= 256:
+// at most 4 values per lane), `head_finish` computes. `tmp` is the wave's own LDS scratch of head_dim floats. The
+// result is written as bfloat16 to `dst` (in LDS) and, if given, to `dst2` (in global memory).
+struct HeadRegs {
+  float x[4], wt[4], cs[4], sn[4];
+};
+
+__device__ __forceinline__ void head_load(HeadRegs& r, const bf16_t* __restrict__ src, const void* __restrict__ w,
+                                          int w_f32, int has_norm, const bf16_t* __restrict__ cos_t,
+                                          const bf16_t* __restrict__ sin_t, int rot, int pos, int head_dim) {
   const int lane = threadIdx.x % WAVE;
   const int half = rot / 2;
-  float x[4], cs[4], sn[4], wt[4];
 #pragma unroll
   for (int u = 0; u < 4; ++u) {
     const int i = lane + WAVE * u;
     const bool in = i < head_dim;
-    x[u] = in ? bf16_to_float(src[i]) : 0.f;
-    wt[u] = (in && has_norm) ? load_vector(w, i, w_f32) : 1.f;
+    r.x[u] = in ? bf16_to_float(src[i]) : 0.f;
+    r.wt[u] = (in && has_norm) ? load_vector(w, i, w_f32) : 1.f;
     const int j = i < half ? i : i - half;
-    cs[u] = (in && i < rot) ? bf16_to_float(cos_t[(int64_t)pos * half + j]) : 1.f;
-    sn[u] = (in && i < rot) ? bf16_to_float(sin_t[(int64_t)pos * half + j]) : 0.f;
+    r.cs[u] = (in && i < rot) ? bf16_to_float(cos_t[(int64_t)pos * half + j]) : 1.f;
+    r.sn[u] = (in && i < rot) ? bf16_to_float(sin_t[(int64_t)pos * half + j]) : 0.f;
   }
+}
+
+__device__ __forceinline__ void head_finish(HeadRegs& r, int has_norm, float eps, int rot, int head_dim, float* tmp,
+                                            bf16_t* dst, bf16_t* dst2) {
+  const int lane = threadIdx.x % WAVE;
+  const int half = rot / 2;
   if (has_norm) {
     float ss = 0.f;
 #pragma unroll
-    for (int u = 0; u < 4; ++u) ss += x[u] * x[u];
+    for (int u = 0; u < 4; ++u) ss += r.x[u] * r.x[u];
     ss = wave_sum(ss);
     const float inv = rsqrtf(ss / (float)head_dim + eps);
 #pragma unroll
-    for (int u = 0; u < 4; ++u) x[u] = rounded_as<bf16_t>(rounded_as<bf16_t>(x[u] * inv) * wt[u]);
+    for (int u = 0; u < 4; ++u) r.x[u] = rounded_as<bf16_t>(rounded_as<bf16_t>(r.x[u] * inv) * r.wt[u]);
   }
 #pragma unroll
   for (int u = 0; u < 4; ++u)
-    if (lane + WAVE * u < head_dim) tmp[lane + WAVE * u] = x[u];
+    if (lane + WAVE * u < head_dim) tmp[lane + WAVE * u] = r.x[u];
   __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "workgroup");
   __builtin_amdgcn_wave_barrier();
 #pragma unroll
   for (int u = 0; u < 4; ++u) {
     const int i = lane + WAVE * u;
     if (i >= head_dim) continue;
-    float o = x[u];
+    float o = r.x[u];
     if (i < rot) {
       const float other = tmp[i < half ? i + half : i - half];
-      const float a = rounded_as<bf16_t>(o * cs[u]), b = rounded_as<bf16_t>(other * sn[u]);
+      const float a = rounded_as<bf16_t>(o * r.cs[u]), b = rounded_as<bf16_t>(other * r.sn[u]);
       o = i < half ? a - b : a + b;
     }
-    const bf16_t r = float_to_bf16(o);
-    dst[i] = r;
-    if (dst2 != nullptr) dst2[i] = r;
+    const bf16_t v = float_to_bf16(o);
+    dst[i] = v;
+    if (dst2 != nullptr) dst2[i] = v;
   }
+  __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "workgroup");   // the next head of this wave reuses tmp
+  __builtin_amdgcn_wave_barrier();
 }
 
 // What the fused form of the split kernel needs to do the work of the norm/rotation/append kernel itself.
@@ -482,31 +493,45 @@ __global__ __launch_bounds__(64 * SPLIT_WAVES, 2) void attn_split_kernel(
   PageK<KB> kf;
   PageV<KB> vf;
   int page = pg <= pg1 ? table[pg] : -1;
-  if (page >= 0) load_page_k<KB, FULL>(kf, k_pages + ((int64_t)page * n_kv + kvh) * page_elems, head_dim);
   RowBlock<KB> st;
   const bool fused_on = fused.qkv != nullptr;
   // exactly one split has the row's own page among its pages (splits past the sequence's end have none)
   const bool owns_last = fused_on && slot >= 0 && pg_first <= pg_hi && pg1 == pg_hi;
   if (fused_on) {
-    // The row's q, k and v come straight from the projection (the first page of keys is already on its way). The
-    // waves norm and rotate the query heads this workgroup serves into LDS. The workgroup whose pages include the
-    // row's own position also norms and rotates the new key, appends key and value to the cache, and keeps both in
-    // LDS: the wave that reads that page puts them into its operands itself, so nothing has to wait for memory.
+    // The row's q, k and v come straight from the projection. The waves norm and rotate the query heads this
+    // workgroup serves into LDS. The workgroup whose pages include the row's own position also norms and rotates
+    // the new key, appends key and value to the cache, and keeps both in LDS: the wave that reads that page puts
+    // them into its operands itself, so nothing has to wait for memory. The loads of a wave's first head are
+    // issued before those of its first page of keys and waited for first, so the two latencies overlap.
     float* tmp = &merge_o[wave][0][0];                          // free until the merge
+    const bf16_t* src_row = fused.qkv + row * fused.stride;
+    HeadRegs first;
+    const bool has_first = slot >= 0 && wave < group;
+    if (has_first)
+      head_load(first, src_row + (int64_t)(kvh * group + wave) * head_dim, fused.q_w, fused.w_f32, fused.has_norm,
+                fused.cos_t, fused.sin_t, fused.rot, pos, head_dim);
+    if (page >= 0) load_page_k<KB, FULL>(kf, k_pages + ((int64_t)page * n_kv + kvh) * page_elems, head_dim);
+    if (has_first)
+      head_finish(first, fused.has_norm, fused.eps, fused.rot, head_dim, tmp, &q_lds[wave][0], nullptr);
     if (slot >= 0) {
-      const bf16_t* src_row = fused.qkv + row * fused.stride;
-      for (int r = wave; r < group; r += SPLIT_WAVES)
-        wave_norm_rope(src_row + (int64_t)(kvh * group + r) * head_dim, fused.q_w, fused.w_f32, fused.has_norm,
-                       fused.eps, fused.cos_t, fused.sin_t, fused.rot, pos, head_dim, tmp, &q_lds[r][0], nullptr);
+      for (int r = wave + SPLIT_WAVES; r < group; r += SPLIT_WAVES) {
+        HeadRegs more;
+        head_load(more, src_row + (int64_t)(kvh * group + r) * head_dim, fused.q_w, fused.w_f32, fused.has_norm,
+                  fused.cos_t, fused.sin_t, fused.rot, pos, head_dim);
+        head_finish(more, fused.has_norm, fused.eps, fused.rot, head_dim, tmp, &q_lds[r][0], nullptr);
+      }
       if (owns_last) {
         const int page_last = table[pg_hi];
         const int64_t base = ((int64_t)max(page_last, 0) * n_kv + kvh) * page_elems;
         const int at = pos % PAGE_TOKENS;
         const bool store = fused.write_kv && page_last >= 0;
-        if (wave == SPLIT_WAVES - 1)
-          wave_norm_rope(src_row + (int64_t)(n_heads + kvh) * head_dim, fused.k_w, fused.w_f32, fused.has_norm,
-                         fused.eps, fused.cos_t, fused.sin_t, fused.rot, pos, head_dim, tmp, &kv_new[0][0],
-                         store ? k_pages_w + base + (int64_t)at * head_dim : nullptr);
+        if (wave == SPLIT_WAVES - 1) {
+          HeadRegs key;
+          head_load(key, src_row + (int64_t)(n_heads + kvh) * head_dim, fused.k_w, fused.w_f32, fused.has_norm,
+                    fused.cos_t, fused.sin_t, fused.rot, pos, head_dim);
+          head_finish(key, fused.has_norm, fused.eps, fused.rot, head_dim, tmp, &kv_new[0][0],
+                      store ? k_pages_w + base + (int64_t)at * head_dim : nullptr);
+        }
         if (wave == SPLIT_WAVES - 2) {
           const bf16_t* vs = src_row + (int64_t)(n_heads + n_kv + kvh) * head_dim;
           for (int i = lane; i < head_dim; i += WAVE) {
@@ -520,6 +545,7 @@ __global__ __launch_bounds__(64 * SPLIT_WAVES, 2) void attn_split_kernel(
     __syncthreads();
     init_rows<KB>(st, &q_lds[c][0], row_valid && slot >= 0, head_dim);
   } else {
+    if (page >= 0) load_page_k<KB, FULL>(kf, k_pages + ((int64_t)page * n_kv + kvh) * page_elems, head_dim);
     init_rows<KB>(st, q + (row * n_heads + head) * head_dim, row_valid && slot >= 0, head_dim);
   }
   while (pg <= pg1) {
