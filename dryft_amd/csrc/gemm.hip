@@ -290,6 +290,219 @@ DRYFT_API int dryft_gemm_skinny_swiglu_bf16(const void* x, int64_t x_stride, con
   return DRYFT_LAUNCH_CHECK();
 }
 
+// ----------------------------------------------------------------------------------------- stream
+// The same product for at most 16 activation rows, with the memory traffic shaped for the cache in front of
+// the matrix cores: a load instruction of gemm_skinny touches 16 rows, 64 bytes of each (half a cache line),
+// for the weights and again for the activations, and the rate at which the vector cache looks lines up, not
+// HBM, bounds it as soon as there are several activation rows. Here a wave reads whole lines (GB * 128
+// contiguous bytes of a row per group of GB blocks of K, two or four rows per instruction), parks them in
+// its own piece of LDS and takes the matrix-core operands from there. The next group's loads are in flight
+// while the current one is multiplied. Rows beyond N or M are read from a clamped, valid row and never
+// stored; values beyond the wave's share of K are zeros.
+template <int GB, int NW>
+struct StreamShape {
+  static constexpr int ROW_BYTES = GB * 128;            // of one row in one group
+  static constexpr int STRIDE = ROW_BYTES + 16;         // in LDS: rows 16 bytes apart in the banks
+  static constexpr int ROWS_PER_LOAD = 1024 / ROW_BYTES;
+  static constexpr int LANES_PER_ROW = WAVE / ROWS_PER_LOAD;
+  static constexpr int LOADS = 16 / ROWS_PER_LOAD;      // instructions per tile of 16 rows
+  static constexpr int TILE_BYTES = 16 * STRIDE;
+  static constexpr int WAVE_BYTES = (NW + 1) * TILE_BYTES;
+  static constexpr int LDS_BYTES = 4 * WAVE_BYTES;
+};
+
+template <int I>
+struct StaticIndex {
+  static constexpr int value = I;
+};
+template <int N, int I = 0, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (I < N) {
+    f(StaticIndex<I>{});
+    static_for<N, I + 1>(f);
+  }
+}
+
+template <int GB, int NW, int DEPTH, bool SWIGLU, typename O>
+__global__ __launch_bounds__(256) void gemm_stream_kernel(const bf16_t* __restrict__ x, int64_t x_stride,
+                                                          const bf16_t* __restrict__ w, O* __restrict__ y,
+                                                          float* __restrict__ partials, int M, int N, int K) {
+  typedef StreamShape<GB, NW> S;
+  extern __shared__ __align__(16) unsigned char stream_lds[];
+  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE, c = lane % 16, g = lane / 16;
+  const int lr = lane / S::LANES_PER_ROW, lp = lane % S::LANES_PER_ROW;   // row within a load, 16-byte piece of it
+  const int n0 = blockIdx.x * 16;
+  const int splits = gridDim.y, units = splits * 4, unit = blockIdx.y * 4 + wave;
+  const int kblocks = (K + 63) / 64, per = (kblocks + units - 1) / units;
+  const int kb0 = min(kblocks, unit * per), kb1 = min(kblocks, kb0 + per);
+  const int k_begin = kb0 * 64, k_end = min(kb1 * 64, K);
+  unsigned char* mine = stream_lds + wave * S::WAVE_BYTES;
+  f32x4 acc[NW];
+#pragma unroll
+  for (int t = 0; t < NW; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+  // where each load instruction of this lane starts (element offsets at k = 0)
+  int64_t w_at[NW][S::LOADS], x_at[S::LOADS];
+#pragma unroll
+  for (int i = 0; i < S::LOADS; ++i) {
+    const int r = S::ROWS_PER_LOAD * i + lr;
+#pragma unroll
+    for (int t = 0; t < NW; ++t) w_at[t][i] = (int64_t)((SWIGLU ? t * N : 0) + min(n0 + r, N - 1)) * K + 8 * lp;
+    x_at[i] = (int64_t)min(r, M - 1) * x_stride + 8 * lp;
+  }
+  const int x_loads = (M + S::ROWS_PER_LOAD - 1) / S::ROWS_PER_LOAD;
+  // DEPTH groups are in flight: slot d of the registers holds group d, d + DEPTH, ... of the wave's share
+  bf16x8 wa[DEPTH][NW][S::LOADS], xa[DEPTH][S::LOADS];
+#pragma unroll
+  for (int d = 0; d < DEPTH; ++d)
+#pragma unroll
+    for (int i = 0; i < S::LOADS; ++i) xa[d][i] = zero8g();
+  auto fetch = [&](auto slot, int k0) {
+    constexpr int d = decltype(slot)::value;
+    if (k0 + GB * 64 <= k_end) {
+#pragma unroll
+      for (int i = 0; i < S::LOADS; ++i) {
+#pragma unroll
+        for (int t = 0; t < NW; ++t) wa[d][t][i] = *(const bf16x8*)(w + w_at[t][i] + k0);
+        if (i < x_loads) xa[d][i] = *(const bf16x8*)(x + x_at[i] + k0);
+      }
+    } else {                                            // the wave's last, partial group
+      const bool in = k0 + 8 * lp < k_end;
+#pragma unroll
+      for (int i = 0; i < S::LOADS; ++i) {
+#pragma unroll
+        for (int t = 0; t < NW; ++t) wa[d][t][i] = in ? *(const bf16x8*)(w + w_at[t][i] + k0) : zero8g();
+        if (i < x_loads) xa[d][i] = in ? *(const bf16x8*)(x + x_at[i] + k0) : zero8g();
+      }
+    }
+  };
+  auto multiply = [&](auto slot, int k0) {
+    constexpr int d = decltype(slot)::value;
+    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "workgroup");   // the previous group's operand reads are done
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int i = 0; i < S::LOADS; ++i) {
+      const int at = (S::ROWS_PER_LOAD * i + lr) * S::STRIDE + 16 * lp;
+#pragma unroll
+      for (int t = 0; t < NW; ++t) *(bf16x8*)(mine + t * S::TILE_BYTES + at) = wa[d][t][i];
+      *(bf16x8*)(mine + NW * S::TILE_BYTES + at) = xa[d][i];
+    }
+    if (k0 + DEPTH * GB * 64 < k_end) fetch(slot, k0 + DEPTH * GB * 64);
+    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "workgroup");
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int u = 0; u < 2 * GB; ++u) {                   // 32 values of K at a time
+      const int at = c * S::STRIDE + 64 * u + 16 * g;
+      const bf16x8 b = *(const bf16x8*)(mine + NW * S::TILE_BYTES + at);
+#pragma unroll
+      for (int t = 0; t < NW; ++t) {
+        const bf16x8 a = *(const bf16x8*)(mine + t * S::TILE_BYTES + at);
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[t], 0, 0, 0);
+      }
+    }
+  };
+  static_for<DEPTH>([&](auto slot) {
+    const int k0 = k_begin + decltype(slot)::value * GB * 64;
+    if (k0 < k_end) fetch(slot, k0);
+  });
+  for (int k0 = k_begin; k0 < k_end; k0 += DEPTH * GB * 64)
+    static_for<DEPTH>([&](auto slot) {
+      const int kk = k0 + decltype(slot)::value * GB * 64;
+      if (kk < k_end) multiply(slot, kk);
+    });
+  __syncthreads();                                        // every wave is done with its staging area
+  f32x4 (*red)[NW][WAVE] = (f32x4 (*)[NW][WAVE])stream_lds;
+#pragma unroll
+  for (int t = 0; t < NW; ++t) red[wave][t][lane] = acc[t];
+  __syncthreads();
+  if (wave != 0) return;
+  const int m = c;
+  if (SWIGLU) {
+    // gate and up of the same (n, m) sit in the same lane (reference: kernels/silu_mul.py:29-32)
+    f32x4 gate = red[0][0][lane], up = red[0][NW - 1][lane];
+#pragma unroll
+    for (int wv = 1; wv < 4; ++wv) {
+      gate += red[wv][0][lane];
+      up += red[wv][NW - 1][lane];
+    }
+    if (m >= M) return;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int n = n0 + 4 * g + i;
+      if (n >= N) continue;
+      const float gv = rounded_as<bf16_t>(gate[i]), uv = rounded_as<bf16_t>(up[i]);
+      const float sv = rounded_as<bf16_t>(gv / (1.f + expf(-gv)));
+      store_from_float(y + (int64_t)m * N + n, sv * uv);
+    }
+    return;
+  }
+  f32x4 s = red[0][0][lane];                              // waves in the order 0..3, as in gemm_skinny
+  s += red[1][0][lane];
+  s += red[2][0][lane];
+  s += red[3][0][lane];
+  if (m >= M) return;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int n = n0 + 4 * g + i;
+    if (n >= N) continue;
+    if (splits > 1)
+      partials[((int64_t)blockIdx.y * M + m) * N + n] = s[i];
+    else
+      store_from_float(y + (int64_t)m * N + n, s[i]);
+  }
+}
+
+template <int GB, int NW, int DEPTH, bool SWIGLU, typename O>
+static int launch_stream(const void* x, int64_t x_stride, const void* w, void* y, float* partials, int M, int N, int K,
+                         int splits, hipStream_t stream) {
+  typedef StreamShape<GB, NW> S;
+  static bool raised = false;                             // more dynamic LDS than the default limit allows
+  auto kernel = gemm_stream_kernel<GB, NW, DEPTH, SWIGLU, O>;
+  if (!raised) {
+    if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, S::LDS_BYTES) != hipSuccess)
+      return -2;
+    raised = true;
+  }
+  dim3 grid((N + 15) / 16, splits), block(256);
+  hipLaunchKernelGGL(kernel, grid, block, S::LDS_BYTES, stream, (const bf16_t*)x, x_stride, (const bf16_t*)w, (O*)y,
+                     partials, M, N, K);
+  return DRYFT_LAUNCH_CHECK();
+}
+
+// M <= 16. splits > 1: float partial sums go to partials[splits, M, N] and y is not written.
+DRYFT_API int dryft_gemm_stream_bf16(const void* x, int64_t x_stride, const void* w, void* y, float* partials, int M,
+                                     int N, int K, int group_blocks, int depth, int splits, int out_f32, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (M > 16 || K <= 0 || K % 8 || x_stride % 8 || splits < 1 || splits > 64) return -1;
+  if (splits > 1 && partials == nullptr) return -1;
+#define ST(GBV, DV)                                                                                               \
+  return out_f32 ? launch_stream<GBV, 1, DV, false, float>(x, x_stride, w, y, partials, M, N, K, splits, stream)  \
+                 : launch_stream<GBV, 1, DV, false, bf16_t>(x, x_stride, w, y, partials, M, N, K, splits, stream)
+  switch (depth * 10 + group_blocks) {
+    case 11: ST(1, 1);
+    case 12: ST(2, 1);
+    case 21: ST(1, 2);
+    case 22: ST(2, 2);
+    default: return -1;
+  }
+#undef ST
+}
+
+// M <= 16. y[M, N] = T(T(silu(x . Wg^T)) * (x . Wu^T)) with W = [Wg; Wu] of 2N rows
+DRYFT_API int dryft_gemm_stream_swiglu_bf16(const void* x, int64_t x_stride, const void* w, void* y, int M, int N,
+                                            int K, int group_blocks, int depth, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (M > 16 || K <= 0 || K % 8 || x_stride % 8) return -1;
+#define SW(GBV, DV) return launch_stream<GBV, 2, DV, true, bf16_t>(x, x_stride, w, y, nullptr, M, N, K, 1, stream)
+  switch (depth * 10 + group_blocks) {
+    case 11: SW(1, 1);
+    case 12: SW(2, 1);
+    case 21: SW(1, 2);
+    case 22: SW(2, 2);
+    default: return -1;
+  }
+#undef SW
+}
+
 // y = T(sum_s partials[s]) in the order s = 0, 1, ...
 template <typename O>
 __global__ void sum_partials_kernel(const float* __restrict__ partials, O* __restrict__ y, int64_t n, int splits) {

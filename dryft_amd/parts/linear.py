@@ -6,8 +6,9 @@ engine/dryft_qwen3/model.py:153, 179-180, 237, 258-261). Here:
 * float32: this library's own kernel, plain multiply-adds, so the 32-bit path has no
   reduced-precision matrix mode anywhere;
 * bfloat16, at most 16 rows (decoding at small batch) and the output head up to 64 rows:
-  this library's weight-streaming matrix-core kernel, which can leave its result as
-  float32 partial sums over K for the consumer to add;
+  this library's weight-streaming matrix-core kernels (up to 16 rows the one that stages
+  whole cache lines through LDS), which can leave their result as float32 partial sums
+  over K for the consumer to add;
 * bfloat16, more rows (prompts, decoding at large batch): the vendor library through
   ``torch.mm``, as in the reference; sizes it or the skinny kernel cannot take go to the
   plain kernel.
@@ -22,6 +23,7 @@ from .base import Partials
 
 SKINNY_ROWS = 64          # the most rows the skinny kernel takes
 SKINNY_BEST = 16          # up to here it beats the vendor library on every projection shape measured
+STREAM_ROWS = 16          # the most rows the line-staging variant takes
 _TARGET_WORKGROUPS = 320   # a little more than one per compute unit
 _BLOCKS_PER_WAVE = 10      # 64-value blocks of K a wave should walk at most
 
@@ -57,14 +59,21 @@ def linear(x: torch.Tensor, w: torch.Tensor, *, out_dtype: torch.dtype | None = 
     library_ok = k % 8 == 0 and n % 8 == 0 and x.is_contiguous()
     if m <= SKINNY_ROWS and skinny_ok(x, w) and (m <= SKINNY_BEST or out_dtype == torch.float32 or not library_ok):
         ntw, splits = skinny_plan(m, n, k)
+        stream = m <= STREAM_ROWS
         if splits > 1:
             partials = torch.empty((splits, m, n), dtype=torch.float32, device=x.device)
-            ops.gemm_skinny_bf16(x, w, None, partials, ntw, splits)
+            if stream:
+                ops.gemm_stream_bf16(x, w, None, partials, splits=splits)
+            else:
+                ops.gemm_skinny_bf16(x, w, None, partials, ntw, splits)
             if allow_partials:
                 return Partials(partials, splits)
             return ops.sum_partials(partials, torch.empty((m, n), dtype=out_dtype, device=x.device), splits)
         out = torch.empty((m, n), dtype=out_dtype, device=x.device)
-        ops.gemm_skinny_bf16(x, w, out, None, ntw, 1)
+        if stream:
+            ops.gemm_stream_bf16(x, w, out)
+        else:
+            ops.gemm_skinny_bf16(x, w, out, None, ntw, 1)
         return out
     if out_dtype == torch.float32:
         out = torch.empty((m, n), dtype=torch.float32, device=x.device)

@@ -11,7 +11,7 @@ import torch
 from ..csrc import ops
 from . import register_part
 from .base import FeedForward, matrix
-from .linear import SKINNY_BEST, linear, skinny_ok
+from .linear import STREAM_ROWS, linear, skinny_ok
 
 
 class SwiGLU(FeedForward):
@@ -33,8 +33,8 @@ class SwiGLU(FeedForward):
 
     def forward(self, h, ctx):
         act = torch.empty((h.shape[0], self.inter), dtype=h.dtype, device=h.device)
-        if h.dtype == torch.bfloat16 and h.shape[0] <= SKINNY_BEST and skinny_ok(h, self.w_gate_up):
-            ops.gemm_skinny_swiglu_bf16(h, self.w_gate_up, act)       # product and activation in one kernel
+        if h.dtype == torch.bfloat16 and h.shape[0] <= STREAM_ROWS and skinny_ok(h, self.w_gate_up):
+            ops.gemm_stream_swiglu_bf16(h, self.w_gate_up, act)       # product and activation in one kernel
         else:
             ops.silu_mul(linear(h, self.w_gate_up), act)
         return linear(act, self.w_down, allow_partials=True)

@@ -385,6 +385,53 @@ def test_gemm_skinny_swiglu(m, inter, k):
     close(out, want, torch.bfloat16, what="fused swiglu")
 
 
+@pytest.mark.parametrize("m", [1, 2, 3, 8, 11, 16])
+@pytest.mark.parametrize("n,k", [(2560, 2560), (384, 96), (331, 80), (256, 9728), (48, 136), (17, 8), (100, 1000)])
+@pytest.mark.parametrize("group,depth,splits", [(2, 2, 1), (2, 1, 1), (1, 2, 1), (1, 1, 3), (2, 2, 4), (2, 1, 16)])
+def test_gemm_stream(m, n, k, group, depth, splits):
+    torch.manual_seed(m + n + k)
+    x, w = torch.randn(m, k).to(torch.bfloat16), (torch.randn(n, k) / math.sqrt(k)).to(torch.bfloat16)
+    want = x.double() @ w.double().T
+    o = ops()
+    if splits == 1:
+        out = torch.empty(m, n, dtype=torch.float32, device=DEV)
+        o.gemm_stream_bf16(x.to(DEV), w.to(DEV), out, None, group, 1, depth)
+        close(out, want, torch.float32, what="stream float32 out")
+        outb = torch.empty(m, n, dtype=torch.bfloat16, device=DEV)
+        o.gemm_stream_bf16(x.to(DEV), w.to(DEV), outb, None, group, 1, depth)
+        close(outb, want, torch.bfloat16, ulps=1.0, what="stream bfloat16 out")
+    else:
+        parts = torch.full((splits, m, n), float("nan"), dtype=torch.float32, device=DEV)
+        o.gemm_stream_bf16(x.to(DEV), w.to(DEV), None, parts, group, splits, depth)
+        out = o.sum_partials(parts, torch.empty(m, n, dtype=torch.float32, device=DEV), splits)
+        close(out, want, torch.float32, what="stream split-K")
+
+
+def test_gemm_stream_strided_rows():
+    """Activation rows that are a slice of a wider matrix (row stride larger than K)."""
+    torch.manual_seed(3)
+    wide = torch.randn(5, 3 * 96).to(torch.bfloat16).to(DEV)
+    x = wide[:, 96:192]
+    w = (torch.randn(200, 96) / 10).to(torch.bfloat16).to(DEV)
+    out = torch.empty(5, 200, dtype=torch.float32, device=DEV)
+    ops().gemm_stream_bf16(x, w, out, None, 2, 1)
+    close(out, x.double().cpu() @ w.double().cpu().T, torch.float32, what="stream strided x")
+
+
+@pytest.mark.parametrize("m", [1, 5, 8, 16])
+@pytest.mark.parametrize("inter,k", [(9728, 2560), (224, 96), (136, 80), (37 * 8, 72)])
+@pytest.mark.parametrize("group,depth", [(1, 1), (2, 1), (2, 2), (1, 2)])
+def test_gemm_stream_swiglu(m, inter, k, group, depth):
+    torch.manual_seed(m + inter)
+    x = torch.randn(m, k).to(torch.bfloat16)
+    w = (torch.randn(2 * inter, k) * 2 / math.sqrt(k)).to(torch.bfloat16)
+    gu = (x.double() @ w.double().T).to(torch.bfloat16).float()            # the unfused path rounds the product first
+    want = (torch.nn.functional.silu(gu[:, :inter]).to(torch.bfloat16).float() * gu[:, inter:]).to(torch.bfloat16)
+    out = torch.empty(m, inter, dtype=torch.bfloat16, device=DEV)
+    ops().gemm_stream_swiglu_bf16(x.to(DEV), w.to(DEV), out, group, depth)
+    close(out, want, torch.bfloat16, what="stream swiglu")
+
+
 def test_linear_dispatch_matches_everywhere():
     """The same product through every route the linear helper can take."""
     from dryft_amd.parts.linear import linear
