@@ -596,40 +596,36 @@ __global__ __launch_bounds__(64 * SPLIT_WAVES, 2) void attn_split_kernel(
     page = page_next;
   }
   // merge the four waves' results: o = sum_w 2^(m_w - m) o_w, l likewise
+  if (row_valid) {
 #pragma unroll
-  for (int dt = 0; dt < 2 * KB; ++dt)
+    for (int dt = 0; dt < 2 * KB; ++dt)
 #pragma unroll
-    for (int i = 0; i < 4; ++i) merge_o[wave][c][16 * dt + 4 * g + i] = st.o[dt][i];
-  if (g == 0) {
-    merge_ml[wave][c][0] = st.m;
-    merge_ml[wave][c][1] = st.l;
+      for (int i = 0; i < 4; ++i) merge_o[wave][c][16 * dt + 4 * g + i] = st.o[dt][i];
+    if (g == 0) {
+      merge_ml[wave][c][0] = st.m;
+      merge_ml[wave][c][1] = st.l;
+    }
   }
   __syncthreads();
-  const int tid = threadIdx.x;
-  for (int r = 0; r < 16; ++r) {
-    if (hb * 16 + r >= group) break;
+  const int rows = min(16, group - hb * 16);
+  for (int idx = threadIdx.x; idx < rows * head_dim; idx += blockDim.x) {     // all heads of the block at once
+    const int r = idx / head_dim, d = idx % head_dim;
     float m = -INFINITY;
 #pragma unroll
     for (int w = 0; w < SPLIT_WAVES; ++w) m = fmaxf(m, merge_ml[w][r][0]);
-    float wgt[SPLIT_WAVES], l = 0.f;
+    float o = 0.f, l = 0.f;
 #pragma unroll
     for (int w = 0; w < SPLIT_WAVES; ++w) {
       const float mw = merge_ml[w][r][0];
-      wgt[w] = mw == -INFINITY ? 0.f : exp2f(mw - m);
-      l += wgt[w] * merge_ml[w][r][1];
+      const float wgt = mw == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mw - m);
+      l += wgt * merge_ml[w][r][1];
+      o += wgt * merge_o[w][r][d];
     }
-    const int h = kvh * group + hb * 16 + r;
-    float* po = part_o + (((int64_t)seq * n_heads + h) * n_splits + split) * head_dim;
-    for (int d = tid; d < head_dim; d += blockDim.x) {
-      float o = 0.f;
-#pragma unroll
-      for (int w = 0; w < SPLIT_WAVES; ++w) o += wgt[w] * merge_o[w][r][d];
-      po[d] = o;
-    }
-    if (tid == 0) {
-      float* pml = part_ml + (((int64_t)seq * n_heads + h) * n_splits + split) * 2;
-      pml[0] = m;       // in units of log2(e)
-      pml[1] = l;
+    const int64_t at = ((int64_t)seq * n_heads + kvh * group + hb * 16 + r) * n_splits + split;
+    part_o[at * head_dim + d] = o;
+    if (d == 0) {
+      part_ml[at * 2] = m;       // in units of log2(e)
+      part_ml[at * 2 + 1] = l;
     }
   }
 }

@@ -26,7 +26,7 @@ from . import register_part
 from .base import Mixer, StepContext, matrix
 from .linear import linear
 
-_SPLIT_TARGET_WAVES = 1024
+_RESIDENT_WORKGROUPS = 512     # of the split kernel: two per compute unit (its registers allow no more)
 _MAX_SPLITS = 32
 
 
@@ -110,9 +110,13 @@ class GQAAttention(Mixer):
         return linear(out.view(rows, self.q_dim), self.w_o, allow_partials=True)
 
     def decode_splits(self, n_seqs: int, max_kv_len: int) -> int:
-        """How many ways each sequence's keys are split so the chip has enough waves to hide latency."""
+        """How many ways each sequence's keys are split: as many as run at the same time, and no more.
+
+        Workgroups beyond what the chip holds at once start when the first ones end, which costs more than
+        the longer walk of fewer, larger splits.
+        """
         blocks = self.n_kv * ((self.n_heads // self.n_kv + 15) // 16)
-        want = (_SPLIT_TARGET_WAVES + n_seqs * blocks - 1) // (n_seqs * blocks)
+        want = _RESIDENT_WORKGROUPS // (n_seqs * blocks)
         span = self.window if self.window else max_kv_len
         pages = max(1, (span + 63) // 64)
         return max(1, min(want, _MAX_SPLITS, pages))
