@@ -64,7 +64,17 @@ __global__ __launch_bounds__(512) void add_rmsnorm_vec_kernel(const T* __restric
       load8_as_float(res + base + i, v[r]);
       if (n_partials > 0) {
         float d[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-        for (int p = 0; p < n_partials; ++p) {
+        int p = 0;
+        for (; p + 4 <= n_partials; p += 4) {             // four loads in flight; added in the order 0, 1, ...
+          float t[4][8];
+#pragma unroll
+          for (int u = 0; u < 4; ++u) load8_as_float(delta + (p + u) * partial_stride + base + i, t[u]);
+#pragma unroll
+          for (int u = 0; u < 4; ++u)
+#pragma unroll
+            for (int j = 0; j < 8; ++j) d[j] += t[u][j];
+        }
+        for (; p < n_partials; ++p) {
           float t[8];
           load8_as_float(delta + p * partial_stride + base + i, t);
 #pragma unroll

@@ -45,6 +45,23 @@ def skinny_plan(m: int, n: int, k: int) -> tuple[int, int]:
     return ntw, splits
 
 
+_STREAM_BLOCKS_PER_WAVE = 5     # measured on the projection shapes of 4B to 32B models inside captured graphs:
+_STREAM_WORKGROUPS = 1536       # short walks over K, as long as the launch stays under about six workgroups a unit
+
+
+def stream_plan(n: int, k: int, may_split: bool) -> tuple[int, int, int]:
+    """(splits of K across workgroups, blocks per group, groups in flight) for the line-staging kernel.
+
+    Splitting pays only where the consumer adds the partial sums up on its way (a pass of their own
+    costs more than the split gains).
+    """
+    tiles = (n + 15) // 16
+    k_blocks = (k + 63) // 64
+    want = (k_blocks + 4 * _STREAM_BLOCKS_PER_WAVE - 1) // (4 * _STREAM_BLOCKS_PER_WAVE)
+    splits = max(1, min(want, _STREAM_WORKGROUPS // tiles, k_blocks // 8, 16)) if may_split else 1
+    return (splits, 1, 2) if splits > 1 else (1, 2, 2)
+
+
 def skinny_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
     return x.shape[1] % 8 == 0 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0
 
@@ -58,12 +75,15 @@ def linear(x: torch.Tensor, w: torch.Tensor, *, out_dtype: torch.dtype | None = 
         return ops.gemm_tiled(x, w, torch.empty((m, n), dtype=torch.float32, device=x.device))
     library_ok = k % 8 == 0 and n % 8 == 0 and x.is_contiguous()
     if m <= SKINNY_ROWS and skinny_ok(x, w) and (m <= SKINNY_BEST or out_dtype == torch.float32 or not library_ok):
-        ntw, splits = skinny_plan(m, n, k)
         stream = m <= STREAM_ROWS
+        if stream:
+            splits, group, depth = stream_plan(n, k, allow_partials)
+        else:
+            ntw, splits = skinny_plan(m, n, k)
         if splits > 1:
             partials = torch.empty((splits, m, n), dtype=torch.float32, device=x.device)
             if stream:
-                ops.gemm_stream_bf16(x, w, None, partials, splits=splits)
+                ops.gemm_stream_bf16(x, w, None, partials, group, splits, depth)
             else:
                 ops.gemm_skinny_bf16(x, w, None, partials, ntw, splits)
             if allow_partials:
@@ -71,7 +91,7 @@ def linear(x: torch.Tensor, w: torch.Tensor, *, out_dtype: torch.dtype | None = 
             return ops.sum_partials(partials, torch.empty((m, n), dtype=out_dtype, device=x.device), splits)
         out = torch.empty((m, n), dtype=out_dtype, device=x.device)
         if stream:
-            ops.gemm_stream_bf16(x, w, out)
+            ops.gemm_stream_bf16(x, w, out, None, group, 1, depth)
         else:
             ops.gemm_skinny_bf16(x, w, out, None, ntw, 1)
         return out
