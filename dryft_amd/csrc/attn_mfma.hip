@@ -462,7 +462,7 @@ __global__ __launch_bounds__(64 * SPLIT_WAVES, 2) void attn_split_kernel(
     const int* __restrict__ page_table, int max_pages, const int* __restrict__ seq_slot,
     const int* __restrict__ cu_rows, const int* __restrict__ kv_len, float* __restrict__ part_o,
     float* __restrict__ part_ml, int n_heads, int n_kv, int head_dim, float scale, int window, int n_splits,
-    FusedQKV fused, bf16_t* __restrict__ k_pages_w, bf16_t* __restrict__ v_pages_w) {
+    FusedQKV fused, bf16_t* __restrict__ k_pages_w, bf16_t* __restrict__ v_pages_w, bf16_t* __restrict__ out) {
   __shared__ float merge_o[SPLIT_WAVES][16][32 * KB + 1];
   __shared__ float merge_ml[SPLIT_WAVES][16][2];
   __shared__ __attribute__((aligned(16))) bf16_t q_lds[16][32 * KB];
@@ -621,6 +621,10 @@ __global__ __launch_bounds__(64 * SPLIT_WAVES, 2) void attn_split_kernel(
       l += wgt * merge_ml[w][r][1];
       o += wgt * merge_o[w][r][d];
     }
+    if (n_splits == 1) {                                   // nothing to combine: this is the result
+      out[(row * n_heads + kvh * group + hb * 16 + r) * head_dim + d] = float_to_bf16(l > 0.f ? o / l : 0.f);
+      continue;
+    }
     const int64_t at = ((int64_t)seq * n_heads + kvh * group + hb * 16 + r) * n_splits + split;
     part_o[at * head_dim + d] = o;
     if (d == 0) {
@@ -737,7 +741,8 @@ static int launch_split(const void* q, const void* k_pages, const void* v_pages,
 #define LAUNCH_SPLIT(FULLV)                                                                                        \
   hipLaunchKernelGGL((attn_split_kernel<KB, FULLV>), grid, block, 0, stream, (const bf16_t*)q, (const bf16_t*)k_pages, \
                      (const bf16_t*)v_pages, page_table, max_pages, seq_slot, cu_rows, kv_len, part_o, part_ml,    \
-                     n_heads, n_kv, head_dim, scale, window, n_splits, fused, (bf16_t*)k_pages, (bf16_t*)v_pages)
+                     n_heads, n_kv, head_dim, scale, window, n_splits, fused, (bf16_t*)k_pages, (bf16_t*)v_pages,       \
+                     (bf16_t*)out)
   if (head_dim % 32 == 0) {
     DISPATCH_KB(head_dim / 32, LAUNCH_SPLIT(true));
   } else {
@@ -745,7 +750,7 @@ static int launch_split(const void* q, const void* k_pages, const void* v_pages,
   }
 #undef LAUNCH_SPLIT
   int rc = DRYFT_LAUNCH_CHECK();
-  if (rc) return rc;
+  if (rc || n_splits == 1) return rc;
   hipLaunchKernelGGL(attn_combine_kernel, dim3(n_seqs, n_heads), dim3(128), 0, stream, part_o, part_ml, seq_slot,
                      cu_rows, (bf16_t*)out, n_heads, head_dim, n_splits);
   return DRYFT_LAUNCH_CHECK();
