@@ -503,6 +503,184 @@ DRYFT_API int dryft_gemm_stream_swiglu_bf16(const void* x, int64_t x_stride, con
 #undef SW
 }
 
+// ------------------------------------------------------------------------------------------- wide
+// The same product for 17 to 64 activation rows (decoding at larger batch). Here the activations weigh as much
+// as the weights, so a workgroup shares them: its four waves stage the rows of x for one group of K in LDS once
+// (double-buffered, one barrier per group), each wave streams 16 weight rows of its own through its own piece of
+// LDS (whole cache lines per load, as in gemm_stream) and multiplies them with all MT tiles of 16 rows of x.
+// K is split across workgroups only (float partial sums for the consumer to add), never across the waves of one.
+// With SWIGLU a workgroup owns 32 outputs: waves 0 and 1 hold their gate rows, waves 2 and 3 their up rows, and
+// the two halves meet through LDS for T(T(silu(gate)) * up) (reference: kernels/silu_mul.py:29-32).
+template <int MT, int GB, bool SWIGLU, typename O>
+__global__ __launch_bounds__(256) void gemm_wide_kernel(const bf16_t* __restrict__ x, int64_t x_stride,
+                                                        const bf16_t* __restrict__ w, O* __restrict__ y,
+                                                        float* __restrict__ partials, int M, int N, int K) {
+  typedef StreamShape<GB, 1> S;
+  extern __shared__ __align__(16) unsigned char wide_lds[];
+  unsigned char* mine = wide_lds + (threadIdx.x / WAVE) * S::TILE_BYTES;          // this wave's weight tile
+  unsigned char* shared = wide_lds + 4 * S::TILE_BYTES;                           // [2][4 tiles] of x
+  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE, c = lane % 16, g = lane / 16;
+  const int lr = lane / S::LANES_PER_ROW, lp = lane % S::LANES_PER_ROW;
+  const int cols = SWIGLU ? 32 : 64;                       // outputs a workgroup owns
+  const int n0 = blockIdx.x * cols + 16 * (SWIGLU ? wave % 2 : wave);             // first output of this wave
+  const int w_row0 = (SWIGLU && wave >= 2 ? N : 0) + n0;   // its first weight row (W = [Wg; Wu] with SWIGLU)
+  const int w_last = (SWIGLU && wave >= 2 ? 2 * N : N) - 1;
+  const int splits = gridDim.y;
+  const int kblocks = (K + 63) / 64, per = (kblocks + splits - 1) / splits;
+  const int kb0 = min(kblocks, (int)blockIdx.y * per), kb1 = min(kblocks, kb0 + per);
+  const int k_begin = kb0 * 64, k_end = min(kb1 * 64, K);
+  f32x4 acc[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  int w_row[S::LOADS], x_row[S::LOADS];
+#pragma unroll
+  for (int i = 0; i < S::LOADS; ++i) {
+    const int r = S::ROWS_PER_LOAD * i + lr;
+    w_row[i] = min(w_row0 + r, w_last);
+    x_row[i] = min(16 * wave + r, M - 1);
+  }
+  const bf16_t* w_lane = w + 8 * lp;
+  const bf16_t* x_lane = x + 8 * lp;
+  const bool stages_x = 16 * wave < M;                     // this wave's tile of x has rows at all
+  bf16x8 wa[S::LOADS], xa[S::LOADS];
+#pragma unroll
+  for (int i = 0; i < S::LOADS; ++i) xa[i] = zero8g();
+  auto fetch = [&](int k0) {
+    const bool in = k0 + 8 * lp < k_end;                   // false only in the last, partial group
+#pragma unroll
+    for (int i = 0; i < S::LOADS; ++i) {
+      wa[i] = in ? *(const bf16x8*)(w_lane + (int64_t)w_row[i] * K + k0) : zero8g();
+      if (stages_x) xa[i] = in ? *(const bf16x8*)(x_lane + (int64_t)x_row[i] * x_stride + k0) : zero8g();
+    }
+  };
+  if (k_begin < k_end) fetch(k_begin);
+  int buf = 0;
+  for (int k0 = k_begin; k0 < k_end; k0 += GB * 64, buf ^= 1) {
+    unsigned char* xs = shared + buf * 4 * S::TILE_BYTES;
+    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "workgroup");   // this wave's reads of its weight tile are done
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int i = 0; i < S::LOADS; ++i) {
+      const int at = (S::ROWS_PER_LOAD * i + lr) * S::STRIDE + 16 * lp;
+      *(bf16x8*)(mine + at) = wa[i];
+      if (stages_x) *(bf16x8*)(xs + wave * S::TILE_BYTES + at) = xa[i];
+    }
+    if (k0 + GB * 64 < k_end) fetch(k0 + GB * 64);
+    __syncthreads();                                         // all tiles of x of this group are in place
+#pragma unroll
+    for (int u = 0; u < 2 * GB; ++u) {
+      const int at = c * S::STRIDE + 64 * u + 16 * g;
+      const bf16x8 a = *(const bf16x8*)(mine + at);
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        const bf16x8 b = *(const bf16x8*)(xs + mt * S::TILE_BYTES + at);
+        acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[mt], 0, 0, 0);
+      }
+    }
+  }
+  // acc[mt][i] is output n0 + 4g + i of activation row 16 mt + c
+  if (SWIGLU) {
+    __syncthreads();                                         // the buffers of x are free: up passes through them
+    f32x4 (*pass)[MT][WAVE] = (f32x4 (*)[MT][WAVE])shared;
+    if (wave >= 2) {
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) pass[wave - 2][mt][lane] = acc[mt];
+    }
+    __syncthreads();
+    if (wave >= 2) return;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      const f32x4 up = pass[wave][mt][lane];
+      const int m = 16 * mt + c;
+      if (m >= M) continue;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int n = n0 + 4 * g + i;
+        if (n >= N) continue;
+        const float gv = rounded_as<bf16_t>(acc[mt][i]), uv = rounded_as<bf16_t>(up[i]);
+        const float sv = rounded_as<bf16_t>(gv / (1.f + expf(-gv)));
+        store_from_float(y + (int64_t)m * N + n, sv * uv);
+      }
+    }
+    return;
+  }
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int m = 16 * mt + c;
+    if (m >= M) continue;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int n = n0 + 4 * g + i;
+      if (n >= N) continue;
+      if (splits > 1)
+        partials[((int64_t)blockIdx.y * M + m) * N + n] = acc[mt][i];
+      else
+        store_from_float(y + (int64_t)m * N + n, acc[mt][i]);
+    }
+  }
+}
+
+template <int MT, int GB, bool SWIGLU, typename O>
+static int launch_wide(const void* x, int64_t x_stride, const void* w, void* y, float* partials, int M, int N, int K,
+                       int splits, hipStream_t stream) {
+  typedef StreamShape<GB, 1> S;
+  constexpr int lds = 12 * S::TILE_BYTES;                  // four weight tiles, two buffers of four tiles of x
+  static bool raised = false;                              // more dynamic LDS than the default limit allows
+  auto kernel = gemm_wide_kernel<MT, GB, SWIGLU, O>;
+  if (lds > 64 * 1024 && !raised) {
+    if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess) return -2;
+    raised = true;
+  }
+  const int cols = SWIGLU ? 32 : 64;
+  dim3 grid((N + cols - 1) / cols, splits), block(256);
+  hipLaunchKernelGGL(kernel, grid, block, lds, stream, (const bf16_t*)x, x_stride, (const bf16_t*)w, (O*)y, partials, M,
+                     N, K);
+  return DRYFT_LAUNCH_CHECK();
+}
+
+// M <= 64. splits > 1: float partial sums go to partials[splits, M, N] and y is not written.
+DRYFT_API int dryft_gemm_wide_bf16(const void* x, int64_t x_stride, const void* w, void* y, float* partials, int M,
+                                   int N, int K, int group_blocks, int splits, int out_f32, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (M > 64 || K <= 0 || K % 8 || x_stride % 8 || splits < 1 || splits > 64) return -1;
+  if (splits > 1 && partials == nullptr) return -1;
+#define WD(MTV, GBV)                                                                                           \
+  return out_f32 ? launch_wide<MTV, GBV, false, float>(x, x_stride, w, y, partials, M, N, K, splits, stream)   \
+                 : launch_wide<MTV, GBV, false, bf16_t>(x, x_stride, w, y, partials, M, N, K, splits, stream)
+  switch (((M + 15) / 16) * 10 + group_blocks) {
+    case 11: WD(1, 1);
+    case 12: WD(1, 2);
+    case 21: WD(2, 1);
+    case 22: WD(2, 2);
+    case 31: WD(3, 1);
+    case 32: WD(3, 2);
+    case 41: WD(4, 1);
+    case 42: WD(4, 2);
+    default: return -1;
+  }
+#undef WD
+}
+
+// M <= 64. y[M, N] = T(T(silu(x . Wg^T)) * (x . Wu^T)) with W = [Wg; Wu] of 2N rows
+DRYFT_API int dryft_gemm_wide_swiglu_bf16(const void* x, int64_t x_stride, const void* w, void* y, int M, int N, int K,
+                                          int group_blocks, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (M > 64 || K <= 0 || K % 8 || x_stride % 8) return -1;
+#define WS(MTV, GBV) return launch_wide<MTV, GBV, true, bf16_t>(x, x_stride, w, y, nullptr, M, N, K, 1, stream)
+  switch (((M + 15) / 16) * 10 + group_blocks) {
+    case 11: WS(1, 1);
+    case 12: WS(1, 2);
+    case 21: WS(2, 1);
+    case 22: WS(2, 2);
+    case 31: WS(3, 1);
+    case 32: WS(3, 2);
+    case 41: WS(4, 1);
+    case 42: WS(4, 2);
+    default: return -1;
+  }
+#undef WS
+}
+
 // y = T(sum_s partials[s]) in the order s = 0, 1, ...
 template <typename O>
 __global__ void sum_partials_kernel(const float* __restrict__ partials, O* __restrict__ y, int64_t n, int splits) {

@@ -9,7 +9,10 @@ engine/dryft_qwen3/model.py:153, 179-180, 237, 258-261). Here:
   this library's weight-streaming matrix-core kernels (up to 16 rows the one that stages
   whole cache lines through LDS), which can leave their result as float32 partial sums
   over K for the consumer to add;
-* bfloat16, more rows (prompts, decoding at large batch): the vendor library through
+* bfloat16, 17 to 64 rows into a product whose consumer adds partial sums (the projections
+  back to the hidden width): this library's shared-activation kernel with K split across
+  workgroups;
+* bfloat16, otherwise (prompts, decoding at large batch): the vendor library through
   ``torch.mm``, as in the reference; sizes it or the skinny kernel cannot take go to the
   plain kernel.
 """
@@ -62,6 +65,17 @@ def stream_plan(n: int, k: int, may_split: bool) -> tuple[int, int, int]:
     return (splits, 1, 2) if splits > 1 else (1, 2, 2)
 
 
+WIDE_ROWS = 64                  # the most rows the shared-activation kernel takes
+_WIDE_BLOCKS = 8                # blocks of K a workgroup of it should walk
+
+
+def wide_splits(n: int, k: int) -> int:
+    """Splits of K for the shared-activation kernel where the consumer adds the partial sums."""
+    tiles = (n + 63) // 64
+    k_blocks = (k + 63) // 64
+    return max(1, min((k_blocks + _WIDE_BLOCKS - 1) // _WIDE_BLOCKS, 1024 // tiles, k_blocks // 4, 16))
+
+
 def skinny_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
     return x.shape[1] % 8 == 0 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0
 
@@ -95,6 +109,14 @@ def linear(x: torch.Tensor, w: torch.Tensor, *, out_dtype: torch.dtype | None = 
         else:
             ops.gemm_skinny_bf16(x, w, out, None, ntw, 1)
         return out
+    if allow_partials and m <= WIDE_ROWS and skinny_ok(x, w):
+        # 17 to 64 rows into a narrow output (the projections back to the hidden width): the vendor library has
+        # too few tiles to fill the chip, this kernel splits K and leaves the sum to the consumer
+        splits = wide_splits(n, k)
+        if splits > 1:
+            partials = torch.empty((splits, m, n), dtype=torch.float32, device=x.device)
+            ops.gemm_wide_bf16(x, w, None, partials, 2, splits)
+            return Partials(partials, splits)
     if out_dtype == torch.float32:
         out = torch.empty((m, n), dtype=torch.float32, device=x.device)
         if skinny_ok(x, w):

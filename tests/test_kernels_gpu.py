@@ -432,6 +432,42 @@ def test_gemm_stream_swiglu(m, inter, k, group, depth):
     close(out, want, torch.bfloat16, what="stream swiglu")
 
 
+@pytest.mark.parametrize("m", [1, 16, 17, 31, 33, 48, 64])
+@pytest.mark.parametrize("n,k", [(2560, 2560), (384, 96), (331, 80), (256, 9728), (48, 136), (17, 8), (100, 1000)])
+@pytest.mark.parametrize("group,splits", [(2, 1), (1, 1), (2, 3), (1, 4), (2, 16)])
+def test_gemm_wide(m, n, k, group, splits):
+    torch.manual_seed(m + n + k)
+    x, w = torch.randn(m, k).to(torch.bfloat16), (torch.randn(n, k) / math.sqrt(k)).to(torch.bfloat16)
+    want = x.double() @ w.double().T
+    o = ops()
+    if splits == 1:
+        out = torch.empty(m, n, dtype=torch.float32, device=DEV)
+        o.gemm_wide_bf16(x.to(DEV), w.to(DEV), out, None, group, 1)
+        close(out, want, torch.float32, what="wide float32 out")
+        outb = torch.empty(m, n, dtype=torch.bfloat16, device=DEV)
+        o.gemm_wide_bf16(x.to(DEV), w.to(DEV), outb, None, group, 1)
+        close(outb, want, torch.bfloat16, ulps=1.0, what="wide bfloat16 out")
+    else:
+        parts = torch.full((splits, m, n), float("nan"), dtype=torch.float32, device=DEV)
+        o.gemm_wide_bf16(x.to(DEV), w.to(DEV), None, parts, group, splits)
+        out = o.sum_partials(parts, torch.empty(m, n, dtype=torch.float32, device=DEV), splits)
+        close(out, want, torch.float32, what="wide split-K")
+
+
+@pytest.mark.parametrize("m", [5, 17, 40, 64])
+@pytest.mark.parametrize("inter,k", [(9728, 2560), (224, 96), (136, 80), (37 * 8, 72), (40, 64)])
+@pytest.mark.parametrize("group", [1, 2])
+def test_gemm_wide_swiglu(m, inter, k, group):
+    torch.manual_seed(m + inter)
+    x = torch.randn(m, k).to(torch.bfloat16)
+    w = (torch.randn(2 * inter, k) * 2 / math.sqrt(k)).to(torch.bfloat16)
+    gu = (x.double() @ w.double().T).to(torch.bfloat16).float()            # the unfused path rounds the product first
+    want = (torch.nn.functional.silu(gu[:, :inter]).to(torch.bfloat16).float() * gu[:, inter:]).to(torch.bfloat16)
+    out = torch.empty(m, inter, dtype=torch.bfloat16, device=DEV)
+    ops().gemm_wide_swiglu_bf16(x.to(DEV), w.to(DEV), out, group)
+    close(out, want, torch.bfloat16, what="wide swiglu")
+
+
 def test_linear_dispatch_matches_everywhere():
     """The same product through every route the linear helper can take."""
     from dryft_amd.parts.linear import linear
