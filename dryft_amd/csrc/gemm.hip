@@ -4,10 +4,9 @@
 //  * gemm_tiled:  any M, N, K, float accumulation by plain fused multiply-adds. With float inputs it
 //    is the true 32-bit product (no reduced-precision matrix mode); with bfloat16 inputs it takes the
 //    sizes the matrix-core kernel refuses.
-//  * gemm_skinny: bfloat16, M <= 64 rows (decoding, output head): every weight is read once, from
-//    global memory straight into the A operand of v_mfma_f32_16x16x32_bf16; the four waves of a
-//    workgroup split K, and further workgroups may split K again into float partial sums that the
-//    consumer adds in a fixed order.
+//  * gemm_stream (M <= 16) and gemm_wide (M <= 64): bfloat16, few rows (decoding, output head): every
+//    weight is read once and multiplied on the matrix cores; K may be split across workgroups into
+//    float partial sums that the consumer adds in a fixed order.
 #include "common.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
@@ -85,7 +84,7 @@ DRYFT_API int dryft_gemm_tiled(const void* x, int64_t x_stride, const void* w, v
   return DRYFT_LAUNCH_CHECK();
 }
 
-// ----------------------------------------------------------------------------------------- skinny
+// ----------------------------------------------------------------------------------------- few rows
 __device__ __forceinline__ bf16x8 zero8g() {
   bf16x8 z;
 #pragma unroll
@@ -93,210 +92,17 @@ __device__ __forceinline__ bf16x8 zero8g() {
   return z;
 }
 
-// A wave computes C^T[n, m] = W[n, :] . x[m, :] for NTW tiles of 16 weight rows and MT tiles of 16
-// activation rows, over its share of K, 64 values of K per step: a lane reads two 16-byte pieces of its
-// weight row (the four lanes of a row cover 64 contiguous bytes per piece) and the same of its activation
-// row. Rows beyond N or M are read from a clamped, valid row and their results are never stored, so the
-// main loop has no guards and is unrolled to keep many loads in flight. With SWIGLU the two weight tiles
-// of a wave are rows [n0, n0+16) of the first half (gate) and of the second half (up) of W, and the
-// epilogue stores T(T(silu(gate)) * up) for the N = rows/2 outputs (reference: kernels/silu_mul.py:29-32).
-#define SKINNY_UNROLL 4
-template <int MT, int NTW, bool SWIGLU, typename O>
-__global__ __launch_bounds__(256) void gemm_skinny_kernel(const bf16_t* __restrict__ x, int64_t x_stride,
-                                                          const bf16_t* __restrict__ w, O* __restrict__ y,
-                                                          float* __restrict__ partials, int M, int N, int K) {
-  __shared__ f32x4 red[4][MT * NTW][WAVE];
-  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE, c = lane % 16, g = lane / 16;
-  const int n0 = blockIdx.x * 16 * (SWIGLU ? 1 : NTW);
-  const int splits = gridDim.y, units = splits * 4, unit = blockIdx.y * 4 + wave;
-  const int kblocks = (K + 63) / 64, per = (kblocks + units - 1) / units;
-  const int kb0 = min(kblocks, unit * per), kb1 = min(kblocks, kb0 + per);
-  const int kb1_full = min(kb1, K / 64);              // blocks that lie wholly inside K
-  f32x4 acc[NTW][MT];
-#pragma unroll
-  for (int nt = 0; nt < NTW; ++nt)
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) acc[nt][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
-  const bf16_t* wp[NTW];
-#pragma unroll
-  for (int nt = 0; nt < NTW; ++nt) {
-    const int n = SWIGLU ? nt * N + min(n0 + c, N - 1) : min(n0 + 16 * nt + c, N - 1);
-    wp[nt] = w + (int64_t)n * K + 8 * g;
-  }
-  const bf16_t* xp[MT];
-#pragma unroll
-  for (int mt = 0; mt < MT; ++mt) xp[mt] = x + (int64_t)min(16 * mt + c, M - 1) * x_stride + 8 * g;
-  int kb = kb0;
-  for (; kb + SKINNY_UNROLL <= kb1_full; kb += SKINNY_UNROLL) {   // all loads of several blocks first, then the products
-    bf16x8 a[SKINNY_UNROLL][NTW][2], b[SKINNY_UNROLL][MT][2];
-#pragma unroll
-    for (int u = 0; u < SKINNY_UNROLL; ++u) {
-      const int k = (kb + u) * 64;
-#pragma unroll
-      for (int nt = 0; nt < NTW; ++nt) {
-        a[u][nt][0] = *(const bf16x8*)(wp[nt] + k);
-        a[u][nt][1] = *(const bf16x8*)(wp[nt] + k + 32);
-      }
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
-        b[u][mt][0] = *(const bf16x8*)(xp[mt] + k);
-        b[u][mt][1] = *(const bf16x8*)(xp[mt] + k + 32);
-      }
-    }
-#pragma unroll
-    for (int u = 0; u < SKINNY_UNROLL; ++u)
-#pragma unroll
-      for (int nt = 0; nt < NTW; ++nt)
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-          acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][nt][0], b[u][mt][0], acc[nt][mt], 0, 0, 0);
-          acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][nt][1], b[u][mt][1], acc[nt][mt], 0, 0, 0);
-        }
-  }
-  for (; kb < kb1_full; ++kb) {
-    const int k = kb * 64;
-#pragma unroll
-    for (int nt = 0; nt < NTW; ++nt)
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
-        const bf16x8 a0 = *(const bf16x8*)(wp[nt] + k), a1 = *(const bf16x8*)(wp[nt] + k + 32);
-        const bf16x8 b0 = *(const bf16x8*)(xp[mt] + k), b1 = *(const bf16x8*)(xp[mt] + k + 32);
-        acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, b0, acc[nt][mt], 0, 0, 0);
-        acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, b1, acc[nt][mt], 0, 0, 0);
-      }
-  }
-  if (kb0 <= K / 64 && K / 64 < kb1) {                // the last, partial block of K (K is a multiple of 8)
-    const int k = (K / 64) * 64;
-    const bool ok0 = k + 8 * g < K, ok1 = k + 32 + 8 * g < K;
-#pragma unroll
-    for (int nt = 0; nt < NTW; ++nt)
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
-        const bf16x8 a0 = ok0 ? *(const bf16x8*)(wp[nt] + k) : zero8g();
-        const bf16x8 b0 = ok0 ? *(const bf16x8*)(xp[mt] + k) : zero8g();
-        const bf16x8 a1 = ok1 ? *(const bf16x8*)(wp[nt] + k + 32) : zero8g();
-        const bf16x8 b1 = ok1 ? *(const bf16x8*)(xp[mt] + k + 32) : zero8g();
-        acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, b0, acc[nt][mt], 0, 0, 0);
-        acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, b1, acc[nt][mt], 0, 0, 0);
-      }
-  }
-#pragma unroll
-  for (int nt = 0; nt < NTW; ++nt)
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) red[wave][nt * MT + mt][lane] = acc[nt][mt];
-  __syncthreads();
-  if (SWIGLU) {
-    // activation-row tile mt is finished by wave mt % 4: gate and up of the same (n, m) sit in the same lane
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      if (mt % 4 != wave) continue;
-      f32x4 gate = red[0][mt][lane], up = red[0][MT + mt][lane];
-#pragma unroll
-      for (int wv = 1; wv < 4; ++wv) {
-        gate += red[wv][mt][lane];
-        up += red[wv][MT + mt][lane];
-      }
-      const int m = 16 * mt + c;
-      if (m >= M) continue;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int n = n0 + 4 * g + i;
-        if (n >= N) continue;
-        const float gv = rounded_as<bf16_t>(gate[i]), uv = rounded_as<bf16_t>(up[i]);
-        const float sv = rounded_as<bf16_t>(gv / (1.f + expf(-gv)));
-        store_from_float(y + (int64_t)m * N + n, sv * uv);
-      }
-    }
-    return;
-  }
-  // tile t is summed (waves in order 0..3) and stored by wave t % 4
-#pragma unroll
-  for (int t = 0; t < MT * NTW; ++t) {
-    if (t % 4 != wave) continue;
-    f32x4 s = red[0][t][lane];
-    s += red[1][t][lane];
-    s += red[2][t][lane];
-    s += red[3][t][lane];
-    const int nt = t / MT, mt = t % MT;
-    const int m = 16 * mt + c;
-    if (m >= M) continue;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int n = n0 + 16 * nt + 4 * g + i;
-      if (n >= N) continue;
-      if (splits > 1)
-        partials[((int64_t)blockIdx.y * M + m) * N + n] = s[i];
-      else
-        store_from_float(y + (int64_t)m * N + n, s[i]);
-    }
-  }
-}
-
-template <int MT, int NTW>
-static int launch_skinny(const void* x, int64_t x_stride, const void* w, void* y, float* partials, int M, int N, int K,
-                         int splits, int out_f32, hipStream_t stream) {
-  dim3 grid((N + 16 * NTW - 1) / (16 * NTW), splits), block(256);
-  if (out_f32)
-    hipLaunchKernelGGL((gemm_skinny_kernel<MT, NTW, false, float>), grid, block, 0, stream, (const bf16_t*)x, x_stride,
-                       (const bf16_t*)w, (float*)y, partials, M, N, K);
-  else
-    hipLaunchKernelGGL((gemm_skinny_kernel<MT, NTW, false, bf16_t>), grid, block, 0, stream, (const bf16_t*)x,
-                       x_stride, (const bf16_t*)w, (bf16_t*)y, partials, M, N, K);
-  return DRYFT_LAUNCH_CHECK();
-}
-
-// splits > 1: float partial sums go to partials[splits, M, N] and y is not written.
-DRYFT_API int dryft_gemm_skinny_bf16(const void* x, int64_t x_stride, const void* w, void* y, float* partials, int M,
-                                     int N, int K, int ntw, int splits, int out_f32, hipStream_t stream) {
-  if (M <= 0 || N <= 0) return 0;
-  if (M > 64 || K <= 0 || K % 8 || x_stride % 8 || splits < 1 || splits > 64) return -1;
-  if (splits > 1 && partials == nullptr) return -1;
-  const int mt = (M + 15) / 16;
-#define SK(MTV, NTWV) return launch_skinny<MTV, NTWV>(x, x_stride, w, y, partials, M, N, K, splits, out_f32, stream)
-  switch (mt * 10 + ntw) {
-    case 11: SK(1, 1);
-    case 12: SK(1, 2);
-    case 14: SK(1, 4);
-    case 21: SK(2, 1);
-    case 22: SK(2, 2);
-    case 24: SK(2, 4);
-    case 31: SK(3, 1);
-    case 32: SK(3, 2);
-    case 34: SK(3, 4);
-    case 41: SK(4, 1);
-    case 42: SK(4, 2);
-    case 44: SK(4, 4);
-    default: return -1;
-  }
-#undef SK
-}
-
-// y[M, N] = T(T(silu(x . Wg^T)) * (x . Wu^T)) with W = [Wg; Wu] of 2N rows
-DRYFT_API int dryft_gemm_skinny_swiglu_bf16(const void* x, int64_t x_stride, const void* w, void* y, int M, int N,
-                                            int K, hipStream_t stream) {
-  if (M <= 0 || N <= 0) return 0;
-  if (M > 64 || K <= 0 || K % 8 || x_stride % 8) return -1;
-  dim3 grid((N + 15) / 16, 1), block(256);
-#define SW(MTV)                                                                                                    \
-  hipLaunchKernelGGL((gemm_skinny_kernel<MTV, 2, true, bf16_t>), grid, block, 0, stream, (const bf16_t*)x, x_stride, \
-                     (const bf16_t*)w, (bf16_t*)y, (float*)nullptr, M, N, K)
-  switch ((M + 15) / 16) {
-    case 1: SW(1); break;
-    case 2: SW(2); break;
-    case 3: SW(3); break;
-    default: SW(4); break;
-  }
-#undef SW
-  return DRYFT_LAUNCH_CHECK();
-}
-
-// ----------------------------------------------------------------------------------------- stream
-// The same product for at most 16 activation rows, with the memory traffic shaped for the cache in front of
-// the matrix cores: a load instruction of gemm_skinny touches 16 rows, 64 bytes of each (half a cache line),
-// for the weights and again for the activations, and the rate at which the vector cache looks lines up, not
-// HBM, bounds it as soon as there are several activation rows. Here a wave reads whole lines (GB * 128
-// contiguous bytes of a row per group of GB blocks of K, two or four rows per instruction), parks them in
-// its own piece of LDS and takes the matrix-core operands from there. The next group's loads are in flight
+// gemm_stream: at most 16 activation rows. A wave computes C^T[n, m] = W[n, :] . x[m, :] for 16 weight rows
+// with v_mfma_f32_16x16x32_bf16 over its share of K; the four waves of a workgroup split K, and further
+// workgroups may split it again into float partial sums. Every weight is read once, and the memory traffic
+// is shaped for the cache in front of the matrix cores: loading the operands straight into the matrix-core
+// layout touches 16 rows, 64 bytes of each (half a cache line), per instruction, for the weights and again for
+// the activations, and the rate at which the vector cache looks lines up, not HBM, then bounds the kernel as
+// soon as there are several activation rows. So a wave reads whole lines (GB * 128 contiguous bytes of a row
+// per group of GB blocks of K, four or eight rows per instruction), parks them in its own piece of LDS and
+// takes the matrix-core operands from there. With SWIGLU the two weight tiles of a wave are rows [n0, n0+16)
+// of the first half (gate) and of the second half (up) of W, and the epilogue stores T(T(silu(gate)) * up)
+// for the N = rows/2 outputs (reference: kernels/silu_mul.py:29-32). The next group's loads are in flight
 // while the current one is multiplied. Rows beyond N or M are read from a clamped, valid row and never
 // stored; values beyond the wave's share of K are zeros.
 template <int GB, int NW>
@@ -417,7 +223,7 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(const bf16_t* __restri
   if (wave != 0) return;
   const int m = c;
   if (SWIGLU) {
-    // gate and up of the same (n, m) sit in the same lane (reference: kernels/silu_mul.py:29-32)
+    // gate and up of the same (n, m) sit in the same lane
     f32x4 gate = red[0][0][lane], up = red[0][NW - 1][lane];
 #pragma unroll
     for (int wv = 1; wv < 4; ++wv) {
@@ -435,7 +241,7 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(const bf16_t* __restri
     }
     return;
   }
-  f32x4 s = red[0][0][lane];                              // waves in the order 0..3, as in gemm_skinny
+  f32x4 s = red[0][0][lane];                              // waves in the order 0..3
   s += red[1][0][lane];
   s += red[2][0][lane];
   s += red[3][0][lane];

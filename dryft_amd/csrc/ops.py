@@ -32,8 +32,6 @@ _SIGNATURES = {
                   "dryft_attn_decode_fused_bf16": [_P, _L, _P, _P, _I, _I, _F, _P, _P, _I, _I, _P, _P, _P, _I, _P, _P,
                                                    _P, _I, _P, _P, _I, _P, _I, _I, _I, _F, _I, _P]},
     "gemm": {"dryft_gemm_tiled": [_P, _L, _P, _P, _I, _I, _I, _I, _I, _P],
-             "dryft_gemm_skinny_bf16": [_P, _L, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
-             "dryft_gemm_skinny_swiglu_bf16": [_P, _L, _P, _P, _I, _I, _I, _P],
              "dryft_gemm_stream_bf16": [_P, _L, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
              "dryft_gemm_stream_swiglu_bf16": [_P, _L, _P, _P, _I, _I, _I, _I, _I, _P],
              "dryft_gemm_wide_bf16": [_P, _L, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
@@ -345,45 +343,6 @@ def gemm_tiled(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Ten
         m1 = min(m, m0 + 65535 * 64)
         _check(_fn("gemm", "dryft_gemm_tiled")(_ptr(x[m0:m1]), x.stride(0), _ptr(w), _ptr(out[m0:m1]), m1 - m0, n, k,
                                                is_f32, out_f32, _stream()), "gemm_tiled")
-    return out
-
-
-def gemm_skinny_bf16(x, w, out, partials=None, ntw: int = 1, splits: int = 1) -> None:
-    """``x [M<=64, K] @ w[N, K].T``; with ``splits > 1`` the result is left as ``partials[splits, M, N]``."""
-    _gpu(x, "x", torch.bfloat16)
-    _gpu(w, "w", torch.bfloat16)
-    m, k = x.shape
-    n = w.shape[0]
-    _require(w.shape == (n, k) and w.is_contiguous() and x.stride(1) == 1, "gemm_skinny: x [M,K] row-major, w [N,K] contiguous")
-    _require(m <= 64 and k % 8 == 0 and x.stride(0) % 8 == 0, f"gemm_skinny: needs M <= 64 and K % 8 == 0, got M={m} K={k}")
-    _require(x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0, "gemm_skinny: operands must be 16-byte aligned")
-    out_f32 = 0
-    if splits > 1:
-        _gpu(partials, "partials", torch.float32)
-        _require(partials.numel() >= splits * m * n and partials.is_contiguous(), "gemm_skinny: partials too small")
-    else:
-        _gpu(out, "out")
-        out_f32 = 1 if out.dtype == torch.float32 else 0
-        _require(out.shape == (m, n) and out.is_contiguous() and out.dtype in (torch.float32, torch.bfloat16),
-                 f"gemm_skinny: out must be contiguous [{m},{n}]")
-    _check(_fn("gemm", "dryft_gemm_skinny_bf16")(_ptr(x), x.stride(0), _ptr(w), _ptr(out), _ptr(partials), m, n, k,
-                                                 int(ntw), int(splits), out_f32, _stream()), "gemm_skinny_bf16")
-
-
-def gemm_skinny_swiglu_bf16(x, w_gate_up, out) -> torch.Tensor:
-    """``silu(x @ Wg.T) * (x @ Wu.T)`` for ``w_gate_up = [Wg; Wu]``, at most 64 rows, in one kernel."""
-    _gpu(x, "x", torch.bfloat16)
-    _gpu(w_gate_up, "w_gate_up", torch.bfloat16)
-    _gpu(out, "out", torch.bfloat16)
-    m, k = x.shape
-    two_n = w_gate_up.shape[0]
-    _require(two_n % 2 == 0 and w_gate_up.shape == (two_n, k) and w_gate_up.is_contiguous() and x.stride(1) == 1,
-             "gemm_skinny_swiglu: x [M,K] row-major, w [2N,K] contiguous")
-    _require(m <= 64 and k % 8 == 0 and x.stride(0) % 8 == 0, f"gemm_skinny_swiglu: needs M <= 64 and K % 8 == 0, got M={m} K={k}")
-    _require(x.data_ptr() % 16 == 0 and w_gate_up.data_ptr() % 16 == 0, "gemm_skinny_swiglu: operands must be 16-byte aligned")
-    _require(out.shape == (m, two_n // 2) and out.is_contiguous(), f"gemm_skinny_swiglu: out must be [{m},{two_n // 2}]")
-    _check(_fn("gemm", "dryft_gemm_skinny_swiglu_bf16")(_ptr(x), x.stride(0), _ptr(w_gate_up), _ptr(out), m, two_n // 2, k,
-                                                        _stream()), "gemm_skinny_swiglu_bf16")
     return out
 
 
