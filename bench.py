@@ -96,20 +96,19 @@ def main() -> int:
 
     def decode_rate(batch: int, steps: int, warmup: int):
         """(tokens/s, ms per step, mean context) for `steps` decode steps after a 2,048-token prefill."""
-        slots = engine.acquire(batch)
+        stream = engine.generate(prompts(batch), warmup + steps + 1)      # the library's own generation loop
         try:
-            engine.reserve(slots, [PROMPT + warmup + steps + 1] * batch)
-            tokens = engine.start(slots, prompts(batch), 0)
-            for i in range(warmup):
-                tokens = engine.advance(slots, tokens, 1 + i)
+            next(stream)                                                  # the prompts' step
+            for _ in range(warmup):
+                next(stream)
             sync()
             t0 = time.perf_counter()
-            for i in range(steps):
-                tokens = engine.advance(slots, tokens, 1 + warmup + i)
+            for _ in range(steps):
+                next(stream)
             sync()
             dt = time.perf_counter() - t0
         finally:
-            engine.release(slots)
+            stream.close()
         context = PROMPT + warmup + (steps + 1) / 2.0
         return batch * steps / dt, dt / steps * 1e3, context
 

@@ -44,6 +44,16 @@ def require_gpu(device) -> torch.device:
     return device
 
 
+class PendingStep:
+    """A launched decoding step: where its chosen tokens will be, and when."""
+
+    def __init__(self, n: int, device: torch.device):
+        self.chosen = torch.empty(n, dtype=torch.int32, device=device)
+        self.host = torch.empty(n, dtype=torch.int32).pin_memory()
+        self.done = torch.cuda.Event()
+        self.sampler_state = None
+
+
 class Engine:
     def __init__(self, model_path: str | None = None, *, config: dict[str, Any] | None = None,
                  seed: int | None = None, norm_std: float = 0.0, dtype: str = "bfloat16", max_batch: int = 32,
@@ -79,6 +89,7 @@ class Engine:
         self.use_graph = bool(use_graph)
         self._graphs: dict[int, DecodeGraph] = {}
         self._sampler = Sampler()
+        self._last_choice: torch.Tensor | None = None
         if verbose:
             log(f"{arch.name} ready in {time.time() - t0:.1f}s: weights {self.model.weight_bytes() / 2**30:.2f} GiB, "
                 f"cache {self.cache.bytes() / 2**30:.2f} GiB for {self.max_tokens} tokens")
@@ -102,21 +113,57 @@ class Engine:
         return self._choose(logits, len(slots))
 
     def advance(self, slots: list[int], tokens: list[int], step_index: int) -> list[int]:
+        if self.use_graph:
+            return self.advance_end(self.advance_begin(slots, tokens, step_index))
+        return self._advance_eager(slots, tokens)
+
+    @property
+    def chains(self) -> bool:
+        """Can a step be launched before the one before it has been read? (Captured graphs only.)"""
+        return self.use_graph
+
+    def advance_begin(self, slots: list[int], tokens: list[int] | None, step_index: int) -> "PendingStep":
+        """Launches one more token each and returns without waiting. ``tokens`` None: every sequence goes on
+        with the token the step launched before this one chose for it, handed over on the device."""
         n = len(slots)
         graph = self._graph_for(n)
-        if graph is not None:
-            live = [s for s in slots if s >= 0]
-            self.cache.begin_step(live, [1] * len(live))
-            logits = graph.replay(slots, tokens)
-            self.cache.end_step(live, [1] * len(live))
+        live = [s for s in slots if s >= 0]
+        self.cache.begin_step(live, [1] * len(live))
+        if tokens is None:
+            if self._last_choice is None or self._last_choice.numel() != n:
+                raise RuntimeError("no previous step of this batch to take the tokens from")
+            logits = graph.replay(slots, self._last_choice)
         else:
-            # dead sequences keep their row so that rows and sequences stay aligned
-            logits = self.stepper.step([SeqStep(s, [t], [0]) for s, t in zip(slots, tokens)])
-            if len(logits) != n:
-                full = torch.zeros((n, logits.shape[1]), dtype=logits.dtype, device=logits.device)
-                idx = torch.tensor([i for i, s in enumerate(slots) if s >= 0], dtype=torch.long, device=logits.device)
-                full[idx] = logits
-                logits = full
+            logits = graph.replay(slots, tokens)
+        self.cache.end_step(live, [1] * len(live))
+        pending = PendingStep(n, self.device)
+        pending.sampler_state = self._sampler.state()
+        uniforms = None if self._sampler.greedy else self._sampler.draw(n)
+        self._sampler.choose(logits, uniforms, out=pending.chosen)
+        pending.host.copy_(pending.chosen, non_blocking=True)
+        pending.done.record()
+        self._last_choice = pending.chosen
+        return pending
+
+    def advance_end(self, pending: "PendingStep") -> list[int]:
+        """The tokens a launched step chose (waits for that step only)."""
+        pending.done.synchronize()
+        return pending.host.tolist()
+
+    def advance_drop(self, pending: "PendingStep") -> None:
+        """Forgets the step launched last: its random numbers count as not drawn."""
+        self._sampler.restore(pending.sampler_state)
+        self._last_choice = None
+
+    def _advance_eager(self, slots: list[int], tokens: list[int]) -> list[int]:
+        n = len(slots)
+        # dead sequences keep their row so that rows and sequences stay aligned
+        logits = self.stepper.step([SeqStep(s, [t], [0]) for s, t in zip(slots, tokens)])
+        if len(logits) != n:
+            full = torch.zeros((n, logits.shape[1]), dtype=logits.dtype, device=logits.device)
+            idx = torch.tensor([i for i, s in enumerate(slots) if s >= 0], dtype=torch.long, device=logits.device)
+            full[idx] = logits
+            logits = full
         return self._choose(logits, n)
 
     def _choose(self, logits: torch.Tensor, n: int) -> list[int]:

@@ -31,6 +31,12 @@ class StepBackend(Protocol):
     def advance(self, slots: list[int], tokens: list[int], step_index: int) -> list[int]:
         """One more token each; ``slots[i] == -1`` marks a sequence that has ended."""
 
+    # A backend whose ``chains`` is true can also launch a step without waiting for it:
+    #   advance_begin(slots, tokens or None, step_index) -> handle    (None: the tokens the step launched
+    #                                                                  before this one chose, kept on the device)
+    #   advance_end(handle) -> list[int]
+    #   advance_drop(handle)                                           (a launched step whose result nobody wants)
+
 
 def check_request(prompts: Sequence[Sequence[int]], max_new_tokens: int, max_len: int) -> None:
     for i, p in enumerate(prompts):
@@ -57,6 +63,9 @@ def generate_batch(backend: StepBackend, prompts: list[list[int]], max_new_token
         backend.reserve(slots, [len(p) + max_new_tokens - 1 for p in prompts])
         running = [True] * n
         tokens = backend.start(slots, [list(p) for p in prompts], 0)
+        if getattr(backend, "chains", False):
+            yield from _chained_steps(backend, slots, running, tokens, max_new_tokens, stops)
+            return
         for step in range(max_new_tokens):
             if step > 0:
                 live_slots = [s if r else -1 for s, r in zip(slots, running)]
@@ -70,6 +79,43 @@ def generate_batch(backend: StepBackend, prompts: list[list[int]], max_new_token
                 return
     finally:
         backend.release(slots)
+
+
+def _chained_steps(backend, slots: list[int], running: list[bool], tokens: list[int], max_new_tokens: int,
+                   stops: set[int]) -> Iterator[list[int]]:
+    """The same steps with one launched ahead: step ``s + 1`` starts before the host has seen what step ``s``
+    chose, on the tokens that step ``s`` left on the device. A sequence that step ``s`` ends therefore still runs
+    in step ``s + 1`` (its place in the cache was reserved anyway); that token is dropped and it sits out from
+    step ``s + 2`` on. What is yielded is exactly what the unchained loop yields.
+    """
+    n = len(slots)
+
+    def decide(step_tokens: list[int]) -> list[int]:
+        out = [int(t) if r else FILL for t, r in zip(step_tokens, running)]
+        for i in range(n):
+            if running[i] and out[i] in stops:
+                running[i] = False
+        return out
+
+    out = decide(tokens)                                      # step 0: the prompts' step
+    yield out
+    if max_new_tokens == 1 or not any(running):
+        return
+    live = [s if r else -1 for s, r in zip(slots, running)]
+    ahead = backend.advance_begin(live, [t if r else 0 for t, r in zip(tokens, running)], 1)
+    try:
+        for step in range(1, max_new_tokens):
+            current, ahead = ahead, None
+            if step + 1 < max_new_tokens:                     # launched on what is known now; see above
+                live = [s if r else -1 for s, r in zip(slots, running)]
+                ahead = backend.advance_begin(live, None, step + 1)
+            out = decide(backend.advance_end(current))
+            yield out
+            if not any(running):
+                return
+    finally:
+        if ahead is not None:                                 # launched, never read: it takes back what it drew
+            backend.advance_drop(ahead)
 
 
 def plan_batches(n_requests: int, max_batch: int) -> list[range]:

@@ -28,7 +28,11 @@ class DecodeGraph:
                                              max_tiles=self.batch, max_kv_len=stepper.cache.max_len, host=None)
         self.logits: torch.Tensor | None = None
         self.graph: torch.cuda.CUDAGraph | None = None
-        self._stage = torch.zeros(2 * self.batch, dtype=torch.int32).pin_memory()
+        # Host-side staging for tokens and slots. Steps may be launched one ahead of the host reading their
+        # results, so a buffer must not be rewritten while an earlier step's copy may still be waiting: four
+        # take turns, and a step is only launched once the step before the previous one has been waited for.
+        self._stages = [torch.zeros(2 * self.batch, dtype=torch.int32).pin_memory() for _ in range(4)]
+        self._turn = 0
 
     def _body(self) -> torch.Tensor:
         hidden = self.stepper.run(self.buf, self.ctx)
@@ -48,13 +52,20 @@ class DecodeGraph:
             self.logits = self._body()
         self.graph = graph
 
-    def replay(self, slots: list[int], tokens: list[int]) -> torch.Tensor:
-        """Logits ``[batch, vocab]`` of one more token each; rows of dead sequences hold nothing of use."""
+    def replay(self, slots: list[int], tokens: list[int] | torch.Tensor) -> torch.Tensor:
+        """Logits ``[batch, vocab]`` of one more token each; rows of dead sequences hold nothing of use.
+
+        ``tokens`` are given by the host, or as an int32 tensor on the device (a previous step's choice).
+        """
         n = self.batch
-        stage = self._stage
-        stage[:n] = torch.from_numpy(np.asarray(tokens, dtype=np.int32))
+        stage = self._stages[self._turn]
+        self._turn = (self._turn + 1) % len(self._stages)
         stage[n:] = torch.from_numpy(np.asarray(slots, dtype=np.int32))
-        self.buf.tokens.copy_(stage[:n], non_blocking=True)
+        if isinstance(tokens, torch.Tensor):
+            self.buf.tokens.copy_(tokens, non_blocking=True)
+        else:
+            stage[:n] = torch.from_numpy(np.asarray(tokens, dtype=np.int32))
+            self.buf.tokens.copy_(stage[:n], non_blocking=True)
         self.buf.seq_slot.copy_(stage[n:], non_blocking=True)
         self.graph.replay()
         return self.logits

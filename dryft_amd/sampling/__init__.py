@@ -32,6 +32,13 @@ class Sampler:
         """The step's uniform numbers in [0, 1), one per sequence of the batch (CPU, float32)."""
         return torch.rand(n, generator=self._gen, dtype=torch.float32)
 
+    def state(self) -> torch.Tensor:
+        """Where the stream of uniform numbers stands; ``restore`` goes back there."""
+        return self._gen.get_state()
+
+    def restore(self, state: torch.Tensor) -> None:
+        self._gen.set_state(state)
+
     def choose(self, logits: torch.Tensor, uniforms: torch.Tensor | None = None,
                out: torch.Tensor | None = None) -> torch.Tensor:
         """Token ids (int32, on the device) for float32 logits ``[rows, vocab]`` on the device."""

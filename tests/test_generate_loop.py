@@ -113,3 +113,86 @@ def test_batches_one_after_another():
     acquires = [e for e in be.log if e[0] == "acquire"]
     assert [len(a[1]) for a in acquires] == [3, 3, 1]
     assert acquires[1][1] == acquires[0][1]                    # the second batch uses the first one's slots again
+
+
+class Chained(Scripted):
+    """The same model with steps that can be launched before the one before them has been read.
+
+    A launched step keeps its result until it is asked for; ``tokens=None`` means "go on with what the
+    step launched before this one chose", which the loop must only use when that is what it would have fed.
+    """
+
+    chains = True
+
+    def __init__(self, **kw):
+        super().__init__(**kw)
+        self.drawn = 0                                          # stands for the sampler's stream of random numbers
+        self.in_flight = 0
+        self.previous = None
+
+    def advance_begin(self, slots, tokens, step_index):
+        if self.fail_at == step_index:
+            raise RuntimeError("boom")
+        assert self.in_flight <= 1, "more than one step ahead"
+        if tokens is None:
+            assert self.previous is not None
+            tokens = self.previous
+        self.log.append(("advance", tuple(slots), tuple(tokens)))
+        for s, t in zip(slots, tokens):
+            if s >= 0:
+                assert t == self.last[s], "a chained step must go on with the token chosen before it"
+        before = dict(self.last), self.drawn
+        result = self._next(slots)
+        self.drawn += 1
+        self.previous = result
+        self.in_flight += 1
+        return {"result": result, "before": before}
+
+    def advance_end(self, handle):
+        self.in_flight -= 1
+        return handle["result"]
+
+    def advance_drop(self, handle):
+        self.in_flight -= 1
+        self.drawn = handle["before"][1]
+        self.log.append(("drop",))
+
+
+@pytest.mark.parametrize("stops", [(), (22, 9), (3,), (7,), (6, 21, 8)])
+@pytest.mark.parametrize("limit", [1, 2, 3, 6])
+def test_chained_loop_yields_what_the_plain_loop_yields(stops, limit):
+    prompts = [[5], [20], [7]]
+    plain = list(generate_batch(Scripted(), prompts, limit, stop_token_ids=stops))
+    be = Chained()
+    assert list(generate_batch(be, prompts, limit, stop_token_ids=stops)) == plain
+    assert sorted(be.free) == [0, 1, 2, 3] and be.in_flight == 0
+    # every random number drawn belongs to a step that was yielded: a step launched in vain gives its own back
+    assert be.drawn == len(plain) - 1
+
+
+def test_chained_loop_lets_an_ended_sequence_run_one_step_more_and_then_sit_out():
+    be = Chained()
+    steps = list(generate_batch(be, [[5], [20], [7]], 6, stop_token_ids=[22]))
+    assert [s[1] for s in steps] == [21, 22, FILL, FILL, FILL, FILL]
+    advances = [e for e in be.log if e[0] == "advance"]
+    assert advances[1][1] == (0, 1, 2)                         # launched before 22 was seen
+    assert advances[2][1] == (0, -1, 2)                        # from then on it sits out
+
+
+def test_chained_loop_releases_and_drops_when_the_caller_stops_early_or_a_step_fails():
+    be = Chained()
+    gen = generate_batch(be, [[1], [2]], 5)
+    next(gen)
+    next(gen)
+    gen.close()
+    assert sorted(be.free) == [0, 1, 2, 3] and be.in_flight == 0 and ("drop",) in be.log
+    be = Chained(fail_at=3)
+    with pytest.raises(RuntimeError, match="boom"):
+        list(generate_batch(be, [[1], [2]], 5))
+    assert sorted(be.free) == [0, 1, 2, 3]
+
+
+def test_chained_batches_one_after_another():
+    be = Chained(max_batch=3)
+    out = generate_all(be, [[10 * i] for i in range(7)], 3, stop_token_ids=[32])
+    assert out == [[1, 2, 3], [11, 12, 13], [21, 22, 23], [31, 32], [41, 42, 43], [51, 52, 53], [61, 62, 63]]

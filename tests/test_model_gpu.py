@@ -327,6 +327,30 @@ def test_stop_tokens_and_more_requests_than_slots(cases, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+def test_steps_launched_ahead_change_nothing(cases, dtype):
+    """With captured graphs the loop launches a step before it has read the one before. Stop tokens (seen one
+    step late), sampling (random numbers drawn ahead, given back when a step is dropped) and batch after batch
+    must give what the engine gives that finishes every step before it starts the next."""
+    case = cases["B"]
+    prompts = [random_tokens(n, case.vocab, seed=90 + n) for n in (3, 17, 8, 40, 5, 11, 26)]
+    ahead = case.engine(dtype, max_batch=3, max_len=128, use_graph=True)
+    plain_loop = case.engine(dtype, max_batch=3, max_len=128, use_graph=False)
+    assert ahead.chains and not plain_loop.chains
+    free_run = plain_loop.generate_all(prompts, 9, temperature=0.7, sample_seed=11)
+    stops = [free_run[0][2], free_run[4][5], free_run[6][0]]
+    for kw in (dict(), dict(temperature=0.7, sample_seed=11), dict(temperature=0.7, sample_seed=11, stop_token_ids=stops),
+               dict(stop_token_ids=[plain_loop.generate_all(prompts, 9)[2][4]])):
+        want = plain_loop.generate_all(prompts, 9, **kw)
+        assert ahead.generate_all(prompts, 9, **kw) == want, f"differs with {kw}"
+        assert list(ahead.generate(prompts[:3], 9, **kw)) == list(plain_loop.generate(prompts[:3], 9, **kw))
+    early = ahead.generate(prompts[:3], 9)
+    next(early), next(early)
+    early.close()                                             # a step is in flight: it is dropped, slots come back
+    assert ahead.cache.slots.free_count == 3
+    assert ahead.generate_all(prompts, 9) == plain_loop.generate_all(prompts, 9)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_graph_replay_equals_eager(cases, dtype):
     """A captured decoding step gives bit-identical logits to the same step run eagerly."""
     case = cases["B"]
