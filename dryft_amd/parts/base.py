@@ -63,6 +63,12 @@ class Partials:
     data: torch.Tensor
     count: int
 
+    def summed(self, dtype: torch.dtype) -> torch.Tensor:
+        """The product itself, ``[rows, width]``: for a consumer that cannot add the partial sums on its way."""
+        from ..csrc import ops
+        out = torch.empty(self.data.shape[1:], dtype=dtype, device=self.data.device)
+        return ops.sum_partials(self.data, out, self.count)
+
 
 class Part:
     """Base of all parts. ``tensor_specs`` maps logical names to (shape, role, init)."""

@@ -51,7 +51,7 @@ def wide_splits(n: int, k: int) -> int:
     return max(1, min((k_blocks + _WIDE_BLOCKS - 1) // _WIDE_BLOCKS, 1024 // tiles, k_blocks // 4, 16))
 
 
-def skinny_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
+def few_rows_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
     """Can the few-row kernels read these operands? (16-byte pieces of rows.)"""
     return x.shape[1] % 8 == 0 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0
 
@@ -63,7 +63,7 @@ def linear(x: torch.Tensor, w: torch.Tensor, *, out_dtype: torch.dtype | None = 
     out_dtype = out_dtype or x.dtype
     if x.dtype == torch.float32:
         return ops.gemm_tiled(x, w, torch.empty((m, n), dtype=torch.float32, device=x.device))
-    few_ok = skinny_ok(x, w)
+    few_ok = few_rows_ok(x, w)
     library_ok = k % 8 == 0 and n % 8 == 0 and x.is_contiguous() and out_dtype == x.dtype
     if m <= STREAM_ROWS and few_ok:
         splits, group, depth = stream_plan(n, k, allow_partials)

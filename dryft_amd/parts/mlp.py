@@ -11,7 +11,7 @@ import torch
 from ..csrc import ops
 from . import register_part
 from .base import FeedForward, matrix
-from .linear import STREAM_ROWS, linear, skinny_ok
+from .linear import STREAM_ROWS, linear, few_rows_ok
 
 
 class SwiGLU(FeedForward):
@@ -33,7 +33,7 @@ class SwiGLU(FeedForward):
 
     def forward(self, h, ctx):
         act = torch.empty((h.shape[0], self.inter), dtype=h.dtype, device=h.device)
-        if h.dtype == torch.bfloat16 and h.shape[0] <= STREAM_ROWS and skinny_ok(h, self.w_gate_up):
+        if h.dtype == torch.bfloat16 and h.shape[0] <= STREAM_ROWS and few_rows_ok(h, self.w_gate_up):
             ops.gemm_stream_swiglu_bf16(h, self.w_gate_up, act)       # product and activation in one kernel
         else:
             ops.silu_mul(linear(h, self.w_gate_up), act)

@@ -73,7 +73,8 @@ def test_swiglu_part(dtype):
         h = torch.randn(rows, 80).to(dtype)
         out = ffn.forward(h.to(DEV), None)
         if isinstance(out, Partials):
-            out = out.data[: out.count].sum(0)
+            assert torch.equal(out.summed(torch.float32), out.data[: out.count].sum(0)) or out.count > 2
+            out = out.summed(torch.float32)
         want = P.swiglu(h.double(), {"mlp." + k + ".weight": v.double() for k, v in w.items()}, "")
         close(out, want, dtype, f"swiglu rows={rows}")
 
