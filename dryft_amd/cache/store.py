@@ -3,7 +3,10 @@
 Key/value groups: ``k`` of shape ``[lines, pages, kv_heads, 64, head_dim]`` and ``v``
 of shape ``[lines, pages, kv_heads, head_dim, 64]`` (transposed within a page) in the
 compute dtype, so one (page, kv head) is one contiguous tile of 64 keys or values and
-both matrix products of attention read contiguous runs along their contraction index. The reference's layout is
+both matrix products of attention read contiguous runs along their contraction index.
+The 64 columns of a page of values hold its positions in the order the matrix cores take
+them (``value_column``: position ``16a + 4g + i`` of a block of 32 sits in column
+``8g + 4a + i``), which only the kernels that write and read pages need to know. The reference's layout is
 ``[layers, rows, kv_heads, L_cap, head_dim]`` (engine/dryft_qwen3/cache.py:3-6);
 the page indirection replaces its fixed ``L_cap`` per row. State groups:
 ``[lines, slots, *shape]``. Storage is zero-initialised once so that bytes no
@@ -48,7 +51,7 @@ class KVGroup:
         self.need, self.lines = need, list(lines)
         shape = (len(lines), n_pages, need.num_kv_heads, PAGE_TOKENS, need.head_dim)
         self.k = torch.zeros(shape, dtype=dtype, device=device)
-        # values are kept transposed within a page: [.., head_dim, 64]
+        # values are kept transposed within a page: [.., head_dim, 64], columns in the kernels' own order
         self.v = torch.zeros(shape[:3] + (need.head_dim, PAGE_TOKENS), dtype=dtype, device=device)
         self.table = PageTable(n_slots, n_pages, max_pages, need.window)
         self.table_dev = torch.full((n_slots, max_pages), -1, dtype=torch.int32, device=device)

@@ -66,7 +66,7 @@ struct PageK {
 };
 template <int KB>
 struct PageV {
-  bf16x4 v[2 * KB][2][2];
+  bf16x8 v[2 * KB][2];      // [tile of 16 features][block of 32 positions]: the lane's 8 values, see value_column
 };
 
 // FULL: head_dim == 32 * KB. Otherwise features at or beyond head_dim are read from a clamped, valid address:
@@ -92,9 +92,7 @@ __device__ __forceinline__ void load_page_v(PageV<KB>& f, const bf16_t* __restri
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
       const int d = FULL ? 16 * dt + c : min(16 * dt + c, head_dim - 1);
-      const bf16_t* vp = v_page + d * PAGE_TOKENS + 32 * h + 4 * g;
-      f.v[dt][h][0] = *(const bf16x4*)vp;
-      f.v[dt][h][1] = *(const bf16x4*)(vp + 16);
+      f.v[dt][h] = load8(v_page + d * PAGE_TOKENS + 32 * h + 8 * g);
     }
 }
 
@@ -164,15 +162,7 @@ __device__ __forceinline__ void page_values(RowBlock<KB>& st, const bf16x8 (&p)[
   for (int dt = 0; dt < 2 * KB; ++dt) {
     if (rescale) st.o[dt] *= alpha;
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      bf16x8 a;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        a[i] = f.v[dt][h][0][i];
-        a[4 + i] = f.v[dt][h][1][i];
-      }
-      st.o[dt] = MFMA16(a, p[h], st.o[dt]);
-    }
+    for (int h = 0; h < 2; ++h) st.o[dt] = MFMA16(f.v[dt][h], p[h], st.o[dt]);
   }
 }
 
@@ -223,9 +213,7 @@ __device__ __forceinline__ void lds_page_v(PageV<KB>& f, const bf16_t* v_lds, in
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
       const int d = FULL ? 16 * dt + c : min(16 * dt + c, head_dim - 1);
-      const bf16_t* vp = v_lds + d * (PAGE_TOKENS + V_PAD) + 32 * h + 4 * g;
-      f.v[dt][h][0] = *(const bf16x4*)vp;
-      f.v[dt][h][1] = *(const bf16x4*)(vp + 16);
+      f.v[dt][h] = load8(v_lds + d * (PAGE_TOKENS + V_PAD) + 32 * h + 8 * g);
     }
 }
 
@@ -537,7 +525,7 @@ __global__ __launch_bounds__(64 * SPLIT_WAVES, 2) void attn_split_kernel(
           for (int i = lane; i < head_dim; i += WAVE) {
             const bf16_t v = vs[i];
             kv_new[1][i] = v;
-            if (store) v_pages_w[base + (int64_t)i * PAGE_TOKENS + at] = v;
+            if (store) v_pages_w[base + (int64_t)i * PAGE_TOKENS + value_column(at)] = v;
           }
         }
       }
@@ -568,7 +556,7 @@ __global__ __launch_bounds__(64 * SPLIT_WAVES, 2) void attn_split_kernel(
               }
             }
         }
-        const int rem = at % 32, hsel = at / 32, half_sel = rem / 16, gsel = (rem % 16) / 4, isel = rem % 4;
+        const int col = value_column(at), hsel = col / 32, gsel = (col % 32) / 8, esel = col % 8;
         if (g == gsel) {
 #pragma unroll
           for (int dt = 0; dt < 2 * KB; ++dt) {
@@ -577,10 +565,8 @@ __global__ __launch_bounds__(64 * SPLIT_WAVES, 2) void attn_split_kernel(
 #pragma unroll
             for (int h = 0; h < 2; ++h)
 #pragma unroll
-              for (int hf = 0; hf < 2; ++hf)
-#pragma unroll
-                for (int i = 0; i < 4; ++i)
-                  if (h == hsel && hf == half_sel && i == isel) vf.v[dt][h][hf][i] = nv;
+              for (int e = 0; e < 8; ++e)
+                if (h == hsel && e == esel) vf.v[dt][h][e] = nv;
           }
         }
       }

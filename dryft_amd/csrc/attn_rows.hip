@@ -64,7 +64,7 @@ __global__ void attn_rows_kernel(const T* __restrict__ q, const T* __restrict__ 
       for (int jj = 0; jj < n; ++jj) {
         const int pg = pages[jj / PAGE_TOKENS];
         if (pg < 0) continue;
-        const T* vp = v_pages + (((int64_t)pg * n_kv + kvh) * head_dim + tid) * PAGE_TOKENS + jj % PAGE_TOKENS;
+        const T* vp = v_pages + (((int64_t)pg * n_kv + kvh) * head_dim + tid) * PAGE_TOKENS + value_column(jj % PAGE_TOKENS);
         acc += ps[jj] * load_as_float(vp);
       }
     }

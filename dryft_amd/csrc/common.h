@@ -108,4 +108,14 @@ __device__ __forceinline__ int page_of(const int* page_table, int max_pages, int
   return page_table[(int64_t)slot * max_pages + pos / PAGE_TOKENS];
 }
 
+// A page of values is [head_dim][64]: a row per feature, a column per position of the page, with the positions
+// of each block of 32 in the order in which the matrix cores want them. The first attention product leaves a
+// lane group g with the scores of positions 4g..4g+3 and 16+4g..16+4g+3 of a block, and the second product
+// takes the values of exactly those positions from one lane; in this order they are 16 contiguous bytes.
+// Position 16a + 4g + i of a block (a in 0..1, g in 0..3, i in 0..3) sits in column 8g + 4a + i of it.
+__host__ __device__ __forceinline__ int value_column(int pos_in_page) {
+  const int o = pos_in_page & 31;
+  return (pos_in_page & 32) + 8 * ((o >> 2) & 3) + 4 * (o >> 4) + (o & 3);
+}
+
 #define DRYFT_LAUNCH_CHECK() (int)hipGetLastError()

@@ -48,7 +48,7 @@ __global__ void qk_norm_rope_kv_kernel(const T* __restrict__ qkv, int64_t qkv_st
   }
   if (!is_q && !is_k) {
     const int kvh = job - n_heads - n_kv;
-    T* dst = v_pages + ((int64_t)page * n_kv + kvh) * head_dim * PAGE_TOKENS + in_page;
+    T* dst = v_pages + ((int64_t)page * n_kv + kvh) * head_dim * PAGE_TOKENS + value_column(in_page);
     for (int i = lane; i < head_dim; i += WAVE) dst[(int64_t)i * PAGE_TOKENS] = src[i];
     return;
   }
@@ -134,7 +134,7 @@ __global__ __launch_bounds__(256) void qk_norm_rope_vec_kernel(const T* __restri
     const int page = page_of(page_table, max_pages, slot, pos);
     if (page < 0) return;
     T* vd = v_pages + (((int64_t)page * n_kv + (job - n_heads - n_kv)) * head_dim + 8 * part) * PAGE_TOKENS +
-            pos % PAGE_TOKENS;
+            value_column(pos % PAGE_TOKENS);
     const T* vs = qkv + row * qkv_stride + (int64_t)job * head_dim + 8 * part;
 #pragma unroll
     for (int j = 0; j < 8; ++j) vd[(int64_t)j * PAGE_TOKENS] = vs[j];
@@ -169,9 +169,11 @@ __global__ __launch_bounds__(256) void qk_norm_rope_vec_kernel(const T* __restri
   store8_from_float(dst, o);
 }
 
-// Values of a step with many rows: a workgroup takes 64 consecutive rows of one kv head, turns the tile in LDS
-// and writes runs of 8 consecutive positions with one 16-byte store where they lie together in a page. (The
-// per-row kernel above writes a row's values 128 bytes apart.) head_dim must be a multiple of 8.
+// Values of a step with many rows: a workgroup takes 64 consecutive rows of one kv head and turns the tile in
+// LDS. Where 32 consecutive rows are one aligned block of 32 positions of one page (the usual case in a long
+// prompt), a thread writes 8 columns of a feature's row with one 16-byte store: they are two runs of four
+// consecutive positions (see value_column). Otherwise values go one by one. (The per-row kernel above writes a
+// row's values 128 bytes apart.) head_dim must be a multiple of 8.
 #define V_TILE_ROWS 64
 #define V_TILE_LD (V_TILE_ROWS + 8)
 template <typename T>
@@ -181,7 +183,9 @@ __global__ __launch_bounds__(256) void v_tile_write_kernel(const T* __restrict__
                                                            const int* __restrict__ page_table, int max_pages,
                                                            int n_rows, int n_kv, int head_dim) {
   extern __shared__ __attribute__((aligned(16))) unsigned char v_tile_raw[];
-  __shared__ int64_t dest[V_TILE_ROWS];
+  __shared__ int64_t base[V_TILE_ROWS];                     // start of the row's page for this kv head, or -1
+  __shared__ int in_page[V_TILE_ROWS];                      // the row's position within its page
+  __shared__ int block_ok[V_TILE_ROWS / 32];
   T* tile = (T*)v_tile_raw;                                 // [head_dim][V_TILE_LD]: already transposed
   const int r0 = blockIdx.x * V_TILE_ROWS, kvh = blockIdx.y;
   const int rows = min(V_TILE_ROWS, n_rows - r0);
@@ -195,31 +199,44 @@ __global__ __launch_bounds__(256) void v_tile_write_kernel(const T* __restrict__
   }
   if (threadIdx.x < V_TILE_ROWS) {
     int64_t where = -1;
+    int at = 0;
     if ((int)threadIdx.x < rows) {
       const int slot = row_slot[r0 + threadIdx.x], pos = row_pos[r0 + threadIdx.x];
       if (slot >= 0) {
         const int page = page_of(page_table, max_pages, slot, pos);
-        if (page >= 0) where = ((int64_t)page * n_kv + kvh) * head_dim * PAGE_TOKENS + pos % PAGE_TOKENS;
+        if (page >= 0) where = ((int64_t)page * n_kv + kvh) * head_dim * PAGE_TOKENS;
+        at = pos % PAGE_TOKENS;
       }
     }
-    dest[threadIdx.x] = where;
+    base[threadIdx.x] = where;
+    in_page[threadIdx.x] = at;
+  }
+  __syncthreads();
+  if (threadIdx.x < V_TILE_ROWS / 32) {                     // is this block of 32 rows one aligned block of a page?
+    const int t0 = 32 * threadIdx.x;
+    bool ok = base[t0] >= 0 && in_page[t0] % 32 == 0;
+    for (int j = 1; j < 32; ++j) ok = ok && base[t0 + j] == base[t0] && in_page[t0 + j] == in_page[t0] + j;
+    block_ok[threadIdx.x] = ok;
   }
   __syncthreads();
   for (int e = threadIdx.x; e < head_dim * (V_TILE_ROWS / 8); e += blockDim.x) {
-    const int d = e / (V_TILE_ROWS / 8), t0 = (e % (V_TILE_ROWS / 8)) * 8;
-    const int64_t w0 = dest[t0];
-    bool together = w0 >= 0 && (w0 % 8) == 0;
-#pragma unroll
-    for (int j = 1; j < 8; ++j) together = together && dest[t0 + j] == w0 + j;
-    const T* src = tile + d * V_TILE_LD + t0;
-    if (together) {
+    const int d = e / (V_TILE_ROWS / 8), piece = e % (V_TILE_ROWS / 8);   // 8 columns of feature d
+    const int blk = piece / 4, g = piece % 4, t0 = 32 * blk;
+    if (block_ok[blk]) {
+      const T* src = tile + d * V_TILE_LD + t0 + 4 * g;     // positions 4g.. and 16+4g.. of the block
       float v[8];
-      load8_as_float(src, v);
-      store8_from_float(v_pages + w0 + (int64_t)d * PAGE_TOKENS, v);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        v[i] = load_as_float(src + i);
+        v[4 + i] = load_as_float(src + 16 + i);
+      }
+      store8_from_float(v_pages + base[t0] + (int64_t)d * PAGE_TOKENS + in_page[t0] + 8 * g, v);
     } else {
 #pragma unroll
-      for (int j = 0; j < 8; ++j)
-        if (dest[t0 + j] >= 0) v_pages[dest[t0 + j] + (int64_t)d * PAGE_TOKENS] = src[j];
+      for (int j = 0; j < 8; ++j) {
+        const int t = t0 + 8 * g + j;
+        if (base[t] >= 0) v_pages[base[t] + (int64_t)d * PAGE_TOKENS + value_column(in_page[t])] = tile[d * V_TILE_LD + t];
+      }
     }
   }
 }

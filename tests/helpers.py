@@ -71,6 +71,14 @@ def random_tokens(n: int, vocab: int, seed: int) -> list[int]:
     return [int(t) for t in rng.integers(0, vocab, size=n)]
 
 
+def value_columns() -> torch.Tensor:
+    """Column of a page of values that holds each of its 64 positions: within a block of 32, position
+    ``16a + 4g + i`` sits in column ``8g + 4a + i`` (the order in which attention's second product takes them)."""
+    pos = torch.arange(64)
+    o = pos % 32
+    return (pos // 32) * 32 + 8 * ((o // 4) % 4) + 4 * (o // 16) + o % 4
+
+
 def build_pages(k: torch.Tensor, v: torch.Tensor, lengths, n_pages: int, n_slots: int, seed: int = 0,
                 poison: float | None = None):
     """Scatter dense keys/values ``[B, L, nKV, D]`` into shuffled pages.
@@ -88,6 +96,7 @@ def build_pages(k: torch.Tensor, v: torch.Tensor, lengths, n_pages: int, n_slots
     k_pages = torch.full((n_pages, n_kv, 64, D), fill, dtype=k.dtype)
     v_pages_t = torch.full((n_pages, n_kv, D, 64), fill, dtype=v.dtype)
     table = torch.full((n_slots, max_pages), -1, dtype=torch.int32)
+    cols = value_columns()
     nxt = 0
     for b in range(B):
         n = int(lengths[b])
@@ -96,7 +105,7 @@ def build_pages(k: torch.Tensor, v: torch.Tensor, lengths, n_pages: int, n_slots
             table[slots[b], pg] = page
             lo, hi = pg * 64, min(n, pg * 64 + 64)
             k_pages[page, :, : hi - lo] = k[b, lo:hi].transpose(0, 1)
-            v_pages_t[page, :, :, : hi - lo] = v[b, lo:hi].permute(1, 2, 0)
+            v_pages_t[page][:, :, cols[: hi - lo]] = v[b, lo:hi].permute(1, 2, 0)
     return k_pages, v_pages_t.reshape(n_pages, n_kv, 64, D), table, slots
 
 

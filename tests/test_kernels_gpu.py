@@ -8,7 +8,7 @@ import numpy as np
 import pytest
 import torch
 
-from helpers import bf16_tolerance, build_pages
+from helpers import bf16_tolerance, build_pages, value_columns
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -155,10 +155,42 @@ def test_qk_norm_rope_kv(dtype, n_heads, n_kv, D, theta):
         page = int(table[row_slot[r], row_pos[r] // 64])
         at = int(row_pos[r]) % 64
         close(kp[page, :, at], k_want[r], dtype, what=f"k row {r}")
-        assert torch.equal(vp[page, :, :, at], v[r]), f"v row {r} must be copied unchanged"
+        col = int(value_columns()[at])                        # values sit in the column the second product wants
+        assert torch.equal(vp[page, :, :, col], v[r]), f"v row {r} must be copied unchanged"
         kp[page, :, at] = 0
-        vp[page, :, :, at] = 0
+        vp[page, :, :, col] = 0
     assert not kp.any() and not vp.any(), "the kernel wrote outside the rows' places"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("n_kv,D", [(2, 128), (3, 48), (1, 16)])
+def test_values_of_many_rows_land_in_their_columns(dtype, n_kv, D):
+    """A step of many rows writes values tile by tile: whole aligned blocks of 32 positions with vector
+    stores, everything else one by one. Three sequences: from position 0, from the middle of a block, dead."""
+    torch.manual_seed(D)
+    n_heads, n_slots, max_pages, n_pages = n_kv, 4, 4, 16
+    spans = [(2, 0, 150), (0, 37, 50), (-1, 0, 9), (3, 64, 70)]            # (slot, first position, rows)
+    row_slot = torch.tensor([s for s, _, n in spans for _ in range(n)], dtype=torch.int32)
+    row_pos = torch.tensor([p0 + i for _, p0, n in spans for i in range(n)], dtype=torch.int32)
+    rows = len(row_slot)
+    qkv = torch.randn(rows, (n_heads + 2 * n_kv) * D).to(dtype)
+    w = torch.ones(D).to(dtype)
+    cos, sin = torch.ones(max_pages * 64, D // 2).to(dtype), torch.zeros(max_pages * 64, D // 2).to(dtype)
+    table = torch.tensor(np.random.default_rng(1).permutation(n_pages).reshape(n_slots, max_pages), dtype=torch.int32)
+    k_pages = torch.zeros(n_pages, n_kv, 64, D, dtype=dtype, device=DEV)
+    v_pages = torch.zeros(n_pages, n_kv, D, 64, dtype=dtype, device=DEV)
+    q_out = torch.empty(rows, n_heads, D, dtype=dtype, device=DEV)
+    ops().qk_norm_rope_kv(qkv.to(DEV), w.to(DEV), w.to(DEV), 1e-6, cos.to(DEV), sin.to(DEV), D, row_slot.to(DEV),
+                          row_pos.to(DEV), q_out, k_pages, v_pages, table.to(DEV), True, n_heads, n_kv, D)
+    v = qkv[:, (n_heads + n_kv) * D:].view(rows, n_kv, D)
+    vp, cols = v_pages.cpu(), value_columns()
+    for r in range(rows):
+        if row_slot[r] < 0:
+            continue
+        page, col = int(table[row_slot[r], row_pos[r] // 64]), int(cols[int(row_pos[r]) % 64])
+        assert torch.equal(vp[page, :, :, col], v[r]), f"v row {r}"
+        vp[page, :, :, col] = 0
+    assert not vp.any(), "values were written outside the rows' places"
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
