@@ -34,11 +34,11 @@ def _add_model_options(ap: argparse.ArgumentParser) -> None:
     ap.add_argument("--no-graph", action="store_true", help="run decoding steps without graph capture")
 
 
-def _engine(args, max_batch: int):
+def _engine(args, max_batch: int, max_tokens: int | None = None):
     from . import Engine
     from .models.qwen3 import load_preset
 
-    kw = dict(dtype=args.dtype, max_batch=args.max_batch or max_batch, max_len=args.max_len,
+    kw = dict(dtype=args.dtype, max_batch=args.max_batch or max_batch, max_len=args.max_len, max_tokens=max_tokens,
               use_graph=not args.no_graph, verbose=True)
     preset = "tiny-a" if args.tiny else args.preset
     if preset:
@@ -108,7 +108,8 @@ def cmd_bench(args) -> int:
     workloads = [w.split(",") for w in (args.workload or ["b1,1,512,32", "b4,4,2048,32", "b16,16,512,128"])]
     workloads = [(n, int(b), int(i), int(o)) for n, b, i, o in workloads]
     args.max_len = max(args.max_len, max(i + o for _, _, i, o in workloads))
-    engine = _engine(args, max(b for _, b, _, _ in workloads))
+    # the cache holds the largest workload, not the largest batch times the longest sequence
+    engine = _engine(args, max(b for _, b, _, _ in workloads), max(b * (-(-(i + o) // 64) * 64) for _, b, i, o in workloads))
     rng = random.Random(args.seed)
     vocab = engine.config.vocab_size
     for name, b, inp, out in workloads:
