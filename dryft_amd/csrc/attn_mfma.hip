@@ -41,8 +41,19 @@ template <int KB>  // KB = ceil(head_dim / 32)
 struct RowBlock {
   bf16x8 q[KB];          // B operand of the first product, per 32 features
   f32x4 o[2 * KB];       // O^T tiles of 16 features each
-  float m, l;            // running maximum and sum of the lane's own row (l % 16)
+  // Running reference maximum of the lane's own row (lane % 16), the same in the four lanes that share a row,
+  // and this lane's part of the row's running sum: the four parts are only added up by row_sum() at the end.
+  float m, l;
 };
+
+// The row's sum of probabilities from its four lanes' parts (all lanes of the wave must call it).
+template <int KB>
+__device__ __forceinline__ float row_sum(const RowBlock<KB>& st) {
+  float l = st.l;
+  l += __shfl_xor(l, 16, WAVE);
+  l += __shfl_xor(l, 32, WAVE);
+  return l;
+}
 
 template <int KB>
 __device__ __forceinline__ void init_rows(RowBlock<KB>& st, const bf16_t* q_row, bool row_valid, int head_dim) {
@@ -107,15 +118,21 @@ __device__ __forceinline__ void page_scores(f32x4 (&s)[4], const PageK<KB>& f, c
   }
 }
 
-// Online softmax over the page's scores: updates the row's running maximum and sum, returns the factor by
-// which the row's accumulator must shrink and leaves the probabilities in `p` as the second product's B operand.
-// `scale_log2` turns a raw score into units of log2(e); st.m is kept in those units. MASKED: some key of the
-// page may be hidden from some row (the page of the diagonal, a window's edge, the end of the sequence).
+// Online softmax over the page's scores, in the form that keeps lanes from talking to each other: the row's
+// reference maximum st.m only moves when some row of the wave has met a score more than MAX_SLACK above it, so
+// in the steady state a lane neither exchanges maxima nor rescales; probabilities are 2^(s - m) with m at most
+// that much below the true maximum (they stay far inside float and bfloat16 range), and each lane adds its own
+// scores to its own part of the sum. Leaves the probabilities in `p` as the second product's B operand and
+// returns the factor by which the row's accumulator must shrink; `moved` tells (the same for the whole wave)
+// whether any factor differs from 1. `scale_log2` turns a raw score into units of log2(e); st.m is kept in those
+// units. MASKED: some key of the page may be hidden from some row (the page of the diagonal, a window's edge,
+// the end of the sequence).
+#define MAX_SLACK 8.f
 template <int KB, bool MASKED>
 __device__ __forceinline__ float page_softmax(RowBlock<KB>& st, f32x4 (&s)[4], bf16x8 (&p)[2], float scale_log2,
-                                              int key0, int lo_row, int hi_row) {
+                                              int key0, int lo_row, int hi_row, bool& moved) {
   const int g = (threadIdx.x % WAVE) / 16;
-  float tile_max = -INFINITY;
+  float lane_max = -INFINITY;
 #pragma unroll
   for (int t = 0; t < 4; ++t)
 #pragma unroll
@@ -124,26 +141,30 @@ __device__ __forceinline__ float page_softmax(RowBlock<KB>& st, f32x4 (&s)[4], b
         const int j = key0 + 16 * t + 4 * g + i;
         if (!(j >= lo_row && j <= hi_row)) s[t][i] = -INFINITY;
       }
-      tile_max = fmaxf(tile_max, s[t][i]);
+      lane_max = fmaxf(lane_max, s[t][i]);
     }
-  tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, WAVE));
-  tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, WAVE));
-  const float m_new = fmaxf(st.m, tile_max * scale_log2);   // scale > 0, so the maximum commutes with it
-  const float m_safe = m_new == -INFINITY ? 0.f : m_new;    // a row that has seen no key yet stays empty
-  const float alpha = fast_exp2(st.m - m_safe);              // exp2(-inf) = 0 for such a row
+  lane_max *= scale_log2;                                     // scale > 0, so the maximum commutes with it
+  float alpha = 1.f;
+  moved = __any(lane_max > st.m + MAX_SLACK);                 // also true for a row's first visible key (m = -inf)
+  if (moved) {
+    float row_max = fmaxf(lane_max, __shfl_xor(lane_max, 16, WAVE));
+    row_max = fmaxf(row_max, __shfl_xor(row_max, 32, WAVE));
+    const float m_new = fmaxf(st.m, row_max);
+    alpha = m_new == -INFINITY ? 1.f : fast_exp2(st.m - m_new);   // exp2(-inf) = 0: nothing was summed before
+    st.l *= alpha;
+    st.m = m_new;
+  }
+  const float m_ref = st.m == -INFINITY ? 0.f : st.m;          // a row that has seen no key yet stays empty
   float sum = 0.f;
 #pragma unroll
   for (int t = 0; t < 4; ++t)
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const float e = fast_exp2(fmaf(s[t][i], scale_log2, -m_safe));   // -inf stays -inf: e = 0
+      const float e = fast_exp2(fmaf(s[t][i], scale_log2, -m_ref));   // -inf stays -inf: e = 0
       s[t][i] = e;
       sum += e;
     }
-  sum += __shfl_xor(sum, 16, WAVE);
-  sum += __shfl_xor(sum, 32, WAVE);
-  st.l = st.l * alpha + sum;
-  st.m = m_new;
+  st.l += sum;
 #pragma unroll
   for (int h = 0; h < 2; ++h)
 #pragma unroll
@@ -156,22 +177,25 @@ __device__ __forceinline__ float page_softmax(RowBlock<KB>& st, f32x4 (&s)[4], b
 
 // O^T = alpha * O^T + V^T P^T
 template <int KB>
-__device__ __forceinline__ void page_values(RowBlock<KB>& st, const bf16x8 (&p)[2], float alpha, const PageV<KB>& f) {
-  const bool rescale = __any(alpha != 1.f);                   // once the maxima have settled nothing changes
+__device__ __forceinline__ void page_values(RowBlock<KB>& st, const bf16x8 (&p)[2], float alpha, bool moved,
+                                            const PageV<KB>& f) {
+  if (moved) {                                                // rare once the maxima have settled
 #pragma unroll
-  for (int dt = 0; dt < 2 * KB; ++dt) {
-    if (rescale) st.o[dt] *= alpha;
+    for (int dt = 0; dt < 2 * KB; ++dt) st.o[dt] *= alpha;
+  }
+#pragma unroll
+  for (int dt = 0; dt < 2 * KB; ++dt)
 #pragma unroll
     for (int h = 0; h < 2; ++h) st.o[dt] = MFMA16(f.v[dt][h], p[h], st.o[dt]);
-  }
 }
 
 template <int KB, bool MASKED>
 __device__ __forceinline__ void page_update_impl(RowBlock<KB>& st, f32x4 (&s)[4], const PageV<KB>& f, float scale_log2,
                                                  int key0, int lo_row, int hi_row) {
   bf16x8 p[2];
-  const float alpha = page_softmax<KB, MASKED>(st, s, p, scale_log2, key0, lo_row, hi_row);
-  page_values<KB>(st, p, alpha, f);
+  bool moved;
+  const float alpha = page_softmax<KB, MASKED>(st, s, p, scale_log2, key0, lo_row, hi_row, moved);
+  page_values<KB>(st, p, alpha, moved, f);
 }
 
 // `masked` must be the same for all lanes of the wave.
@@ -324,6 +348,7 @@ __global__ __launch_bounds__(256, (GP * KB <= 8 && KB <= 4) ? 2 : 1) void attn_c
                           (window > 0 && key0 < pos0 + 15 - window + 1);
       bf16x8 p[GP][2];
       float alpha[GP];
+      bool moved[GP];
       {
         PageK<KB> kf;                      // the keys are dead once every head has its probabilities,
         lds_page_k<KB, FULL>(kf, k_lds, head_dim);
@@ -331,20 +356,23 @@ __global__ __launch_bounds__(256, (GP * KB <= 8 && KB <= 4) ? 2 : 1) void attn_c
         for (int hh = 0; hh < GP; ++hh) {
           f32x4 s[4];
           page_scores<KB>(s, kf, st[hh]);
-          alpha[hh] = masked ? page_softmax<KB, true>(st[hh], s, p[hh], scale_log2, key0, lo_row, pos_row)
-                             : page_softmax<KB, false>(st[hh], s, p[hh], scale_log2, key0, lo_row, pos_row);
+          alpha[hh] = masked ? page_softmax<KB, true>(st[hh], s, p[hh], scale_log2, key0, lo_row, pos_row, moved[hh])
+                             : page_softmax<KB, false>(st[hh], s, p[hh], scale_log2, key0, lo_row, pos_row, moved[hh]);
         }
       }
       PageV<KB> vf;                        // so the values can take their registers
       lds_page_v<KB, FULL>(vf, v_lds, head_dim);
 #pragma unroll
-      for (int hh = 0; hh < GP; ++hh) page_values<KB>(st[hh], p[hh], alpha[hh], vf);
+      for (int hh = 0; hh < GP; ++hh) page_values<KB>(st[hh], p[hh], alpha[hh], moved[hh], vf);
     }
   }
+  float row_l[GP];
+#pragma unroll
+  for (int hh = 0; hh < GP; ++hh) row_l[hh] = row_sum<KB>(st[hh]);
   if (row_valid) {
 #pragma unroll
     for (int hh = 0; hh < GP; ++hh) {
-      const float inv = 1.f / st[hh].l;
+      const float inv = 1.f / row_l[hh];
       bf16_t* o = out + (row * n_heads + head0 + hh) * head_dim;
 #pragma unroll
       for (int dt = 0; dt < 2 * KB; ++dt) {
@@ -582,6 +610,7 @@ __global__ __launch_bounds__(64 * SPLIT_WAVES, 2) void attn_split_kernel(
     page = page_next;
   }
   // merge the four waves' results: o = sum_w 2^(m_w - m) o_w, l likewise
+  const float l_wave = row_sum<KB>(st);
   if (row_valid) {
 #pragma unroll
     for (int dt = 0; dt < 2 * KB; ++dt)
@@ -589,7 +618,7 @@ __global__ __launch_bounds__(64 * SPLIT_WAVES, 2) void attn_split_kernel(
       for (int i = 0; i < 4; ++i) merge_o[wave][c][16 * dt + 4 * g + i] = st.o[dt][i];
     if (g == 0) {
       merge_ml[wave][c][0] = st.m;
-      merge_ml[wave][c][1] = st.l;
+      merge_ml[wave][c][1] = l_wave;
     }
   }
   __syncthreads();
