@@ -169,6 +169,96 @@ __global__ __launch_bounds__(256) void qk_norm_rope_vec_kernel(const T* __restri
   store8_from_float(dst, o);
 }
 
+// The same for steps of many rows: one workgroup per row. A thread keeps the rotation factors and norm weights
+// of its 8 features, which are the same for every head, and walks over the row's q and k heads four at a time,
+// so that it issues about a quarter of the loads per head of the kernel above. Value heads are not handled here.
+template <typename T, int LPH>   // lanes per head: head_dim / 8
+__global__ __launch_bounds__(256) void qk_norm_rope_row_kernel(const T* __restrict__ qkv, int64_t qkv_stride,
+                                                               const void* __restrict__ q_w, const void* __restrict__ k_w,
+                                                               int w_f32, int has_norm, float eps,
+                                                               const T* __restrict__ cos_t, const T* __restrict__ sin_t,
+                                                               const int* __restrict__ row_slot,
+                                                               const int* __restrict__ row_pos, T* __restrict__ q_out,
+                                                               T* __restrict__ k_pages, const int* __restrict__ page_table,
+                                                               int max_pages, int write_kv, int n_heads, int n_kv) {
+  constexpr int D = 8 * LPH, PER = 256 / LPH;           // heads a workgroup handles side by side
+  const int64_t row = blockIdx.x;
+  const int part = threadIdx.x % LPH, lane_head = threadIdx.x / LPH;
+  const int slot = row_slot[row], pos = row_pos[row];
+  if (slot < 0) {                                       // a dead row: its q is zero, nothing is cached
+    const float z[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    for (int job = lane_head; job < n_heads; job += PER) store8_from_float(q_out + (row * n_heads + job) * D + 8 * part, z);
+    return;
+  }
+  const bool first = part < LPH / 2;
+  const int64_t at = (int64_t)pos * (D / 2) + 8 * (first ? part : part - LPH / 2);
+  float c[8], sn[8], wq[8], wk[8];
+  load8_as_float(cos_t + at, c);
+  load8_as_float(sin_t + at, sn);
+  if (has_norm) {
+    if (w_f32) {
+      load8_as_float((const float*)q_w + 8 * part, wq);
+      load8_as_float((const float*)k_w + 8 * part, wk);
+    } else {
+      load8_as_float((const bf16_t*)q_w + 8 * part, wq);
+      load8_as_float((const bf16_t*)k_w + 8 * part, wk);
+    }
+  }
+  const int page = write_kv ? page_of(page_table, max_pages, slot, pos) : -1;
+  const int jobs = n_heads + (page >= 0 ? n_kv : 0);    // q heads, then k heads
+  const T* src = qkv + row * qkv_stride + 8 * part;
+  for (int j0 = lane_head; j0 < jobs; j0 += 4 * PER) {
+    float v[4][8];
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (j0 + u * PER < jobs) load8_as_float(src + (int64_t)(j0 + u * PER) * D, v[u]);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int job = j0 + u * PER;                      // the same for the LPH lanes that share a head
+      if (job >= jobs) continue;
+      const bool is_q = job < n_heads;
+      if (has_norm) {
+        float ss = 0.f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) ss += v[u][j] * v[u][j];
+#pragma unroll
+        for (int o = LPH / 2; o > 0; o >>= 1) ss += __shfl_xor(ss, o, WAVE);
+        const float inv = rsqrtf(ss / (float)D + eps);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[u][j] = rounded_as<T>(rounded_as<T>(v[u][j] * inv) * (is_q ? wq[j] : wk[j]));
+      }
+      float o[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float other = __shfl_xor(v[u][j], LPH / 2, WAVE);
+        const float a = rounded_as<T>(v[u][j] * c[j]), b = rounded_as<T>(other * sn[j]);
+        o[j] = first ? a - b : a + b;                    // x1*c - x2*s ; x2*c + x1*s
+      }
+      T* dst = is_q ? q_out + (row * n_heads + job) * D + 8 * part
+                    : k_pages + (((int64_t)page * n_kv + (job - n_heads)) * PAGE_TOKENS + pos % PAGE_TOKENS) * D + 8 * part;
+      store8_from_float(dst, o);
+    }
+  }
+}
+
+template <typename T>
+static void launch_rope_rows(const void* qkv, int64_t qkv_stride, const void* q_w, const void* k_w, int w_f32, int has_norm,
+                             float eps, const void* cos_t, const void* sin_t, const int* row_slot, const int* row_pos,
+                             void* q_out, void* k_pages, const int* page_table, int max_pages, int write_kv, int n_rows,
+                             int n_heads, int n_kv, int head_dim, hipStream_t stream) {
+#define ROWS(LPHV)                                                                                                     \
+  hipLaunchKernelGGL((qk_norm_rope_row_kernel<T, LPHV>), dim3(n_rows), dim3(256), 0, stream, (const T*)qkv, qkv_stride, \
+                     q_w, k_w, w_f32, has_norm, eps, (const T*)cos_t, (const T*)sin_t, row_slot, row_pos, (T*)q_out,   \
+                     (T*)k_pages, page_table, max_pages, write_kv, n_heads, n_kv)
+  switch (head_dim) {
+    case 32: ROWS(4); break;
+    case 64: ROWS(8); break;
+    case 128: ROWS(16); break;
+    default: ROWS(32); break;
+  }
+#undef ROWS
+}
+
 // Values of a step with many rows: a workgroup takes 64 consecutive rows of one kv head and turns the tile in
 // LDS. Where 32 consecutive rows are one aligned block of 32 positions of one page (the usual case in a long
 // prompt), a thread writes 8 columns of a feature's row with one 16-byte store: they are two runs of four
@@ -253,7 +343,16 @@ DRYFT_API int dryft_qk_norm_rope_kv(const void* qkv, int64_t qkv_stride, const v
   // many rows: the values go through the tile kernel
   const int skip_v = (write_kv && n_rows >= 32 && head_dim % 8 == 0 && aligned) ? 1 : 0;
   const bool vec = aligned && rot == head_dim && (head_dim == 32 || head_dim == 64 || head_dim == 128 || head_dim == 256);
-  if (vec) {
+  if (vec && skip_v && n_rows >= 64) {                  // many rows: a workgroup per row
+    if (is_f32)
+      launch_rope_rows<float>(qkv, qkv_stride, q_w, k_w, w_f32, has_norm, eps, cos_t, sin_t, row_slot, row_pos, q_out,
+                              k_pages, page_table, max_pages, write_kv, n_rows, n_heads, n_kv, head_dim, stream);
+    else
+      launch_rope_rows<bf16_t>(qkv, qkv_stride, q_w, k_w, w_f32, has_norm, eps, cos_t, sin_t, row_slot, row_pos, q_out,
+                               k_pages, page_table, max_pages, write_kv, n_rows, n_heads, n_kv, head_dim, stream);
+    int rc = DRYFT_LAUNCH_CHECK();
+    if (rc) return rc;
+  } else if (vec) {
     const int lph = head_dim / 8, per_block = 256 / lph;
     const int with_v = (write_kv && !skip_v) ? 1 : 0;
     const int qk_jobs = n_heads + (write_kv ? (with_v ? 2 : 1) * n_kv : 0);

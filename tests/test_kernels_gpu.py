@@ -109,10 +109,12 @@ def rope_ref(x, cos, sin, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("n_heads,n_kv,D,theta", [(32, 8, 128, 5e6), (6, 3, 48, 1e4), (4, 2, 16, 1e6), (5, 1, 256, 1e5)])
-def test_qk_norm_rope_kv(dtype, n_heads, n_kv, D, theta):
+@pytest.mark.parametrize("n_heads,n_kv,D,theta", [(32, 8, 128, 5e6), (6, 3, 48, 1e4), (4, 2, 16, 1e6), (5, 1, 256, 1e5),
+                                                  (9, 3, 64, 1e4), (70, 2, 32, 1e4)])
+@pytest.mark.parametrize("rows", [23, 150])                 # few rows, and enough for the kernels of long steps
+def test_qk_norm_rope_kv(dtype, n_heads, n_kv, D, theta, rows):
     torch.manual_seed(D)
-    rows, n_slots, max_pages, n_pages = 23, 7, 6, 42
+    n_slots, max_pages, n_pages = 7, 6, 42
     L = max_pages * 64
     eps = 1e-6
     qkv = (2 * torch.randn(rows, (n_heads + 2 * n_kv) * D)).to(dtype)
