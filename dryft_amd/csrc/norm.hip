@@ -107,7 +107,9 @@ static void launch_norm_vec(const void* res, const void* delta, int n_partials, 
                             int w_f32, void* res_out, void* y, int n_rows, int width, float eps, hipStream_t stream) {
   const int runs_total = width / 8;
   int threads = 64;
-  while (threads < 512 && threads < runs_total) threads *= 2;
+  // few rows: latency counts, one run a thread; many rows: throughput counts, fuller threads in fewer waves
+  const int per_thread = n_rows >= 64 ? 2 : 1;
+  while (threads < 512 && per_thread * threads < runs_total) threads *= 2;
   const int runs = (runs_total + threads - 1) / threads;
   dim3 grid(n_rows), block(threads);
 #define NV(R)                                                                                                        \
