@@ -8,6 +8,7 @@ agent/bench.py:180-192).
     python -m dryft_amd generate --preset tiny-b --weight-seed 0 --random-prompts 3,5,9 --temperature 0.8
     python -m dryft_amd make-model --preset tiny-a --weight-seed 1 --out DIR
     python -m dryft_amd bench --preset qwen3-4b --workload b8,8,2048,64
+    python -m dryft_amd profile --preset qwen3-4b --batch 8 --prompt-len 2048 --steps 8
     python -m dryft_amd replay --model DIR --dtype float32 --out DIR --max-tokens 4096 < steps.jsonl
 """
 
@@ -134,6 +135,67 @@ def cmd_bench(args) -> int:
     return 0
 
 
+def cmd_profile(args) -> int:
+    """Per-kernel table of decoding steps or of one prompt step, from ``torch.profiler`` device events: calls and
+    microseconds per step, share, and for decoding the bandwidth the step's bytes imply (agent/profiler.py:58-89).
+    Decoding steps run without graph capture so that every kernel is visible by name (profiler.py:47-48)."""
+    import torch
+    from torch.profiler import ProfilerActivity, profile
+
+    from .engine.step import SeqStep
+
+    args.no_graph = True
+    args.max_len = max(args.max_len, args.prompt_len + args.steps + 8)
+    engine = _engine(args, args.batch)
+    rng = random.Random(args.seed)
+    vocab = engine.config.vocab_size
+    prompts = [[rng.randrange(vocab) for _ in range(args.prompt_len)] for _ in range(args.batch)]
+    slots = engine.acquire(args.batch)
+    try:
+        engine.reserve(slots, [args.prompt_len + args.steps + 4] * args.batch)
+        if args.prefill:
+            engine.step([SeqStep(s, p, [len(p) - 1]) for s, p in zip(slots, prompts)])       # warm-up, then again
+            engine.release(slots)
+            slots = engine.acquire(args.batch)
+            engine.reserve(slots, [args.prompt_len + args.steps + 4] * args.batch)
+            torch.cuda.synchronize()
+            with profile(activities=[ProfilerActivity.CPU, ProfilerActivity.CUDA]) as prof:
+                engine.step([SeqStep(s, p, [len(p) - 1]) for s, p in zip(slots, prompts)])
+                torch.cuda.synchronize()
+            steps, what = 1, f"one step of {args.batch} prompts of {args.prompt_len} tokens"
+        else:
+            tokens = engine.start(slots, prompts, 0)
+            for i in range(2):
+                tokens = engine.advance(slots, tokens, 1 + i)
+            torch.cuda.synchronize()
+            with profile(activities=[ProfilerActivity.CPU, ProfilerActivity.CUDA]) as prof:
+                for i in range(args.steps):
+                    tokens = engine.advance(slots, tokens, 3 + i)
+                torch.cuda.synchronize()
+            steps, what = args.steps, f"{args.steps} decoding steps of {args.batch} sequences at {args.prompt_len} tokens"
+    finally:
+        engine.release(slots)
+    rows: dict[str, list[float]] = {}
+    for ev in prof.events():
+        if getattr(ev, "device_type", None) is not None and "cuda" in str(ev.device_type).lower():
+            us = float(getattr(ev, "device_time", 0.0) or getattr(ev, "cuda_time", 0.0) or 0.0)
+            entry = rows.setdefault(ev.name, [0, 0.0])
+            entry[0] += 1
+            entry[1] += us
+    total = sum(v[1] for v in rows.values())
+    print(f"{what}: {total / steps:.1f} us of kernels per step")
+    print(f"{'kernel':72s} {'calls/step':>10s} {'us/step':>10s} {'share':>6s}")
+    for name, (count, us) in sorted(rows.items(), key=lambda kv: -kv[1][1])[: args.rows]:
+        print(f"{name[:72]:72s} {count / steps:10.1f} {us / steps:10.1f} {100 * us / max(total, 1e-9):5.1f}%")
+    if not args.prefill and total > 0:
+        cfg = engine.config
+        weights = engine.model.weight_bytes() - (0 if cfg.tie_word_embeddings else cfg.vocab_size * cfg.hidden_size * 2)
+        cache = args.batch * (args.prompt_len + 2 + args.steps / 2) * cfg.num_hidden_layers * 2 * cfg.kv_dim * 2
+        print(f"implied bandwidth: {(weights + cache) / (total / steps * 1e-6) / 1e9:.0f} GB/s "
+              f"(weights read once, cache of the live sequences)")
+    return 0
+
+
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser(prog="dryft_amd", description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     sub = ap.add_subparsers(dest="command", required=True)
@@ -168,6 +230,16 @@ def main(argv=None) -> int:
     b.add_argument("--seed", type=int, default=0)
     b.add_argument("--workload", action="append", help="name,batch,in,out (may repeat)")
     b.set_defaults(fn=cmd_bench)
+
+    pr = sub.add_parser("profile", help="per-kernel table of decoding steps or of one prompt step")
+    _add_model_options(pr)
+    pr.add_argument("--batch", type=int, default=8)
+    pr.add_argument("--prompt-len", type=int, default=2048)
+    pr.add_argument("--steps", type=int, default=8)
+    pr.add_argument("--prefill", action="store_true", help="profile the prompts' step instead of decoding steps")
+    pr.add_argument("--rows", type=int, default=20, help="kernels to list")
+    pr.add_argument("--seed", type=int, default=0)
+    pr.set_defaults(fn=cmd_profile)
 
     r = sub.add_parser("replay", help="trace replay (same as bin/trace_run)", add_help=False)
     r.set_defaults(fn=None)
