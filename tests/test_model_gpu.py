@@ -25,7 +25,7 @@ DTYPES = ["float32", "bfloat16"]
 # for them the bound is what bfloat16 arithmetic itself does to the plain implementation on the same
 # request (its error against the float64 run, times two), when that is larger.
 TOL = {"float32": 1e-4, "bfloat16": 3e-2}
-LENGTHS = [1, 5, 9, 17, 33, 70, 131, 200]
+LENGTHS = [1, 5, 9, 17, 33, 64, 65, 70, 128, 129, 131, 200]     # 64-token cache pages: edges and one past them
 
 
 class Case:
@@ -152,6 +152,9 @@ def unequal_batches(case):
         {"r131": (r["r131"], 66), "r9": (r["r9"], 8), "r33": (r["r33"], 2)},
         {"r200": (r["r200"], 150), "r70#2": (r["r70"], 6), "r5#2": (r["r5"], 4), "r17#2": (r["r17"], 16),
          "r33#2": (r["r33"], 32)},
+        # prompts that end exactly at a page's edge, one token before and one after it, then cross further edges
+        {"r129": (r["r129"], 65), "r128": (r["r128"], 64), "r65": (r["r65"], 2), "r64": (r["r64"], 1),
+         "r131#2": (r["r131"], 3)},
     ]
 
 
