@@ -108,7 +108,7 @@ static void launch_norm_vec(const void* res, const void* delta, int n_partials, 
   const int runs_total = width / 8;
   int threads = 64;
   // few rows: latency counts, one run a thread; many rows: throughput counts, fuller threads in fewer waves
-  const int per_thread = n_rows >= 64 ? 2 : 1;
+  const int per_thread = n_rows >= 256 ? 2 : 1;
   while (threads < 512 && per_thread * threads < runs_total) threads *= 2;
   const int runs = (runs_total + threads - 1) / threads;
   dim3 grid(n_rows), block(threads);
