@@ -482,3 +482,207 @@ def test_windowed_layer_has_storage_of_its_own_and_gives_pages_back(dtype, tmp_p
             assert err <= limit, f"{rid}@{pos}: {err}"
         assert windowed.table.pool.free_count == windowed.table.pool.n_pages
         assert full.table.pool.free_count == full.table.pool.n_pages
+
+
+# ------------------------------------------------------------------------------------------------
+# A second toy architecture defined here, to show the other two kinds of part: a feed-forward that routes each
+# row to one of several experts (router in float32) and a position encoding of its own (a sinusoid table that
+# its mixer adds to its input). Nothing in the package knows about either.
+@dataclass(frozen=True)
+class RoutedConfig:
+    hidden_size: int
+    vocab_size: int
+    decay: float
+    expert_size: int
+    n_experts: int
+
+    @classmethod
+    def from_dict(cls, raw):
+        return cls(*(raw[k] for k in ("hidden_size", "vocab_size", "decay", "expert_size", "n_experts")))
+
+
+def sinusoid_table(n_positions, width):
+    pos = torch.arange(n_positions, dtype=torch.float64)[:, None]
+    freq = 1.0 / (50.0 ** (torch.arange(0, width, 2, dtype=torch.float64) / width))
+    return torch.cat((torch.sin(pos * freq), torch.cos(pos * freq)), dim=1) * 0.5
+
+
+def routed_plan(cfg):
+    from dryft_amd.config import LayerSpec, ModelPlan, PartSpec, Run
+    H = cfg.hidden_size
+
+    def norm(name):
+        return PartSpec("rmsnorm", dict(size=H, eps=1e-5), {"weight": name})
+
+    def layer(i):
+        return LayerSpec("prenorm", {
+            "mixer_norm": norm(f"l{i}.n1"), "ffn_norm": norm(f"l{i}.n2"),
+            "mixer": PartSpec("toy_positional_mixer", dict(hidden_size=H, decay=cfg.decay, positions="sinusoid"),
+                              {"w_in": f"l{i}.w_in", "w_out": f"l{i}.w_out"}),
+            "ffn": PartSpec("toy_routed_ffn", dict(hidden_size=H, expert_size=cfg.expert_size, n_experts=cfg.n_experts),
+                            {"router": f"l{i}.router", "w1": f"l{i}.w1", "w2": f"l{i}.w2"})})
+
+    return ModelPlan(vocab_size=cfg.vocab_size, hidden_size=H,
+                     embedding=PartSpec("token_embedding", dict(vocab_size=cfg.vocab_size, hidden_size=H), {"weight": "emb"}),
+                     layers=(layer(0), layer(1)), schedule=(Run(0, 0), Run(1, 1)), final_norm=norm("final"),
+                     head=PartSpec("lm_head", dict(vocab_size=cfg.vocab_size, hidden_size=H, tied=True), {}),
+                     positions={"sinusoid": PartSpec("toy_sinusoid_positions", dict(width=H))})
+
+
+def register_routed():
+    from dryft_amd import register_architecture, register_part
+    from dryft_amd.cache import StateNeed
+    from dryft_amd.models import known_architectures
+    from dryft_amd.parts.base import FeedForward, Mixer, PositionEncoding, matrix
+    from dryft_amd.parts.linear import linear
+
+    class SinusoidPositions(PositionEncoding):
+        def __init__(self, width):
+            self.width, self.table = width, None
+
+        def prepare(self, n_positions, dtype, device):
+            if self.table is None or self.table.shape[0] < n_positions or self.table.dtype != dtype:
+                self.table = sinusoid_table(n_positions, self.width).to(dtype).to(device)
+
+    class PositionalMixer(Mixer):
+        """s_t = decay * s_{t-1} + (h_t + table[position_t]) @ w_in; out_t = s_t @ w_out."""
+
+        def __init__(self, hidden_size, decay, positions):
+            self.hidden, self.decay, self.positions = hidden_size, decay, positions
+
+        def tensor_specs(self):
+            return {"w_in": matrix((self.hidden, self.hidden)), "w_out": matrix((self.hidden, self.hidden))}
+
+        def load(self, tensors):
+            self.w_in, self.w_out = tensors["w_in"], tensors["w_out"]
+
+        def cache_need(self):
+            return StateNeed((self.hidden,), "float32")
+
+        def forward(self, h, ctx, line, writes_cache):
+            table = ctx.positions[self.positions].table
+            placed = h + table[ctx.row_pos[: h.shape[0]].clamp(min=0).long()]      # the step's positions, on the device
+            u = linear(placed.contiguous(), self.w_in).float()                     # the library's own products
+            out = torch.zeros_like(u)
+            row = 0
+            for slot, n in zip(ctx.host.slots, ctx.host.q_lens):
+                if slot >= 0:
+                    s = line.state[slot]
+                    for t in range(n):
+                        s = self.decay * s + u[row + t]
+                        out[row + t] = s
+                    line.state[slot] = s
+                row += n
+            return linear(out.to(h.dtype), self.w_out)
+
+    class RoutedFFN(FeedForward):
+        """Each row goes to the expert its router likes best, weighted by the router's probability for it:
+        y = p_e * relu(h @ w1[e].T) @ w2[e].T with p = softmax(h @ router.T) in float32."""
+
+        def __init__(self, hidden_size, expert_size, n_experts):
+            self.hidden, self.inner, self.n = hidden_size, expert_size, n_experts
+
+        def tensor_specs(self):
+            return {"router": matrix((self.n, self.hidden)), "w1": matrix((self.n * self.inner, self.hidden)),
+                    "w2": matrix((self.n * self.hidden, self.inner))}
+
+        def load(self, tensors):
+            self.router = tensors["router"].float()
+            self.w1 = tensors["w1"].view(self.n, self.inner, self.hidden)
+            self.w2 = tensors["w2"].view(self.n, self.hidden, self.inner)
+
+        def forward(self, h, ctx):
+            p = torch.softmax(h.float() @ self.router.T, dim=-1)
+            weight, expert = p.max(dim=-1)
+            out = torch.zeros_like(h)
+            for e in range(self.n):
+                rows = (expert == e).nonzero().flatten()
+                if rows.numel():
+                    inner = torch.relu(linear(h[rows].contiguous(), self.w1[e].contiguous()))
+                    y = linear(inner, self.w2[e].contiguous()).float() * weight[rows, None]
+                    out[rows] = y.to(h.dtype)
+            return out
+
+    if "ToyRoutedLM" not in known_architectures():
+        register_part("toy_sinusoid_positions", SinusoidPositions)
+        register_part("toy_positional_mixer", PositionalMixer)
+        register_part("toy_routed_ffn", RoutedFFN)
+        register_architecture("ToyRoutedLM", RoutedConfig, routed_plan)
+
+
+def routed_plain(cfg, w, tokens):
+    """The routed toy model on one whole sequence in float64; also each position's smallest router margin."""
+    w = {k: v.double() for k, v in w.items()}
+    H, E, I = cfg["hidden_size"], cfg["n_experts"], cfg["expert_size"]
+    T = len(tokens)
+    x = w["emb"][torch.tensor(tokens)]
+    table = sinusoid_table(T, H)
+    margin = torch.full((T,), float("inf"), dtype=torch.float64)
+    for i in range(2):
+        h = P.rms_norm(x, w[f"l{i}.n1"], 1e-5) + table
+        u = h @ w[f"l{i}.w_in"].T
+        s, mixed = torch.zeros(H, dtype=torch.float64), []
+        for t in range(T):
+            s = cfg["decay"] * s + u[t]
+            mixed.append(s)
+        x = x + torch.stack(mixed) @ w[f"l{i}.w_out"].T
+        h = P.rms_norm(x, w[f"l{i}.n2"], 1e-5)
+        p = torch.softmax(h @ w[f"l{i}.router"].T, dim=-1)
+        top = p.topk(2, dim=-1).values
+        margin = torch.minimum(margin, top[:, 0] - top[:, 1])
+        weight, expert = p.max(dim=-1)
+        w1, w2 = w[f"l{i}.w1"].view(E, I, H), w[f"l{i}.w2"].view(E, H, I)
+        y = torch.stack([weight[t] * (torch.relu(h[t] @ w1[expert[t]].T) @ w2[expert[t]].T) for t in range(T)])
+        x = x + y
+    return P.rms_norm(x, w["final"], 1e-5) @ w["emb"].T, margin
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_routed_feed_forward_and_position_encoding_are_registered_built_and_stepped(dtype, tmp_path):
+    from dryft_amd import Engine
+    from dryft_amd.engine.model import DecoderModel
+    from dryft_amd.engine.replay import Replayer
+    from dryft_amd.weights import random_tensors, write_model_dir
+    from helpers import collect_positions, read_model_dir, trace_batches, trace_whole
+    register_routed()
+    raw = {"architectures": ["ToyRoutedLM"], "hidden_size": 48, "vocab_size": 83, "decay": 0.7, "expert_size": 40,
+           "n_experts": 3}
+    model = DecoderModel(routed_plan(RoutedConfig.from_dict(raw)), torch.float32, "cpu")
+    tensors = random_tensors(model.tensor_specs(), 9, torch.bfloat16, std=0.15)
+    for name in tensors:                                     # decided routers: few rows sit near a tie of two experts
+        if "router" in name:
+            tensors[name] = (tensors[name].float() * 8).to(torch.bfloat16)
+    path = write_model_dir(str(tmp_path / "routed"), raw, tensors)
+    _, weights = read_model_dir(path)
+    engine = Engine(path, dtype=dtype, max_batch=4, max_len=256, use_graph=False)
+    assert len(engine.cache.state_groups) == 1 and not engine.cache.kv_groups
+    reqs = {f"t{n}": random_tokens(n, 83, seed=30 + n) for n in (2, 33, 70)}
+    want = {rid: routed_plain(raw, weights, toks) for rid, toks in reqs.items()}
+    experts_used = set()
+    for rid, toks in reqs.items():                           # the test is about routing: more than one expert is used
+        w64 = {k: v.double() for k, v in weights.items()}
+        h0 = P.rms_norm(w64["emb"][torch.tensor(toks)], w64["l0.n1"], 1e-5)
+        experts_used |= set((h0 @ w64["l0.router"].T).argmax(-1).tolist())
+    assert len(experts_used) > 1
+    limit = 1e-4 if dtype == "float32" else 4e-2
+    # a router's choice flips where two experts are nearly tied and the arithmetic is coarse; from such a position
+    # on the two runs follow different experts, so bfloat16 is compared only up to the first close call
+    slack = 0.0 if dtype == "float32" else 0.05
+    traces = [list(trace_whole(reqs)),
+              list(trace_batches([{rid: (toks, min(len(toks) - 1, 20)) for rid, toks in reqs.items()}]))]
+    compared = 0
+    for records in traces:
+        r = Replayer(engine)
+        outputs = {}
+        for rec in records:
+            lg = r.run_step(rec)
+            if lg is not None and lg.shape[0]:
+                outputs[rec["step"]] = lg.float().cpu()
+        for (rid, pos), row in collect_positions(records, outputs).items():
+            ref, margin = want[rid]
+            if bool((margin[: pos + 1] < slack).any()):
+                continue
+            err = float((row - ref[pos].float()).abs().max()) / float(ref.abs().max())
+            assert err <= limit, f"{rid}@{pos}: {err}"
+            compared += 1
+    assert compared >= 100
