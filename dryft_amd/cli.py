@@ -111,6 +111,8 @@ def cmd_bench(args) -> int:
     args.max_len = max(args.max_len, max(i + o for _, _, i, o in workloads))
     # the cache holds the largest workload, not the largest batch times the longest sequence
     engine = _engine(args, max(b for _, b, _, _ in workloads), max(b * (-(-(i + o) // 64) * 64) for _, b, i, o in workloads))
+    if args.tune:
+        engine.tune(sorted({b for _, b, _, _ in workloads} | {b * inp for _, b, inp, _ in workloads}))
     rng = random.Random(args.seed)
     vocab = engine.config.vocab_size
     for name, b, inp, out in workloads:
@@ -227,6 +229,8 @@ def main(argv=None) -> int:
     b = sub.add_parser("bench", help="time whole generate calls on given workloads")
     _add_model_options(b)
     b.add_argument("--samples", type=int, default=5)
+    b.add_argument("--tune", action="store_true",
+                   help="first let the vendor library choose its kernels for the workloads' step sizes")
     b.add_argument("--seed", type=int, default=0)
     b.add_argument("--workload", action="append", help="name,batch,in,out (may repeat)")
     b.set_defaults(fn=cmd_bench)

@@ -98,6 +98,30 @@ class Engine:
     def step(self, seqs: list[SeqStep]) -> torch.Tensor:
         return self.stepper.step(seqs)
 
+    def tune(self, row_counts: Sequence[int]) -> None:
+        """Lets the vendor library choose its kernels for steps of these many rows (a prompt of 2,048 tokens is a
+        step of 2,048 rows; 64 sequences decoding are a step of 64): one step of stand-in tokens for each count,
+        a few seconds each, nothing kept in the cache; counts beyond the longest sequence are spread over several
+        sequences. The choice holds for exactly these counts; any other keeps
+        the library's default. Only the bfloat16 products of more than 64 rows, and some of 17 to 64, are the
+        library's; everything else is untouched."""
+        from ..parts.linear import library_tuning
+        with library_tuning():
+            for rows in row_counts:
+                rows = int(rows)
+                n_seqs = max(1, -(-rows // self.max_len))
+                if rows <= 0 or n_seqs > self.max_batch or -(-rows // 64) * 64 + 64 * n_seqs > self.max_tokens:
+                    raise ValueError(f"a step of {rows} rows does not fit this engine "
+                                     f"({self.max_batch} sequences of {self.max_len}, {self.max_tokens} tokens)")
+                lengths = [rows // n_seqs + (i < rows % n_seqs) for i in range(n_seqs)]
+                slots = self.acquire(n_seqs)
+                try:
+                    self.stepper.step([SeqStep(s, [0] * n, [n - 1]) for s, n in zip(slots, lengths)])
+                    torch.cuda.synchronize()
+                finally:
+                    self.release(slots)
+        self._graphs.clear()            # graphs captured before would keep the kernels chosen then
+
     # ------------------------------------------------------------------ StepBackend
     def acquire(self, n: int) -> list[int]:
         return self.cache.acquire(n)

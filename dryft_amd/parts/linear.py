@@ -19,6 +19,10 @@ engine/dryft_qwen3/model.py:153, 179-180, 237, 258-261). Here:
 
 from __future__ import annotations
 
+import contextlib
+import os
+import tempfile
+
 import torch
 
 from ..csrc import ops
@@ -92,6 +96,26 @@ def linear(x: torch.Tensor, w: torch.Tensor, *, out_dtype: torch.dtype | None = 
             ops.gemm_wide_bf16(x[m0:m0 + WIDE_ROWS], w, out[m0:m0 + WIDE_ROWS], None, 2, 1)
         return out
     return ops.gemm_tiled(x, w, out)
+
+
+@contextlib.contextmanager
+def library_tuning():
+    """While open, the vendor library times its candidate kernels for every product shape it meets for the
+    first time and keeps the fastest; afterwards those shapes use what was kept and nothing more is timed.
+
+    The reference plans the same kind of choice, measured on the real GPU before the timed region
+    (AGENTS.md:567). It is torch's TunableOp; what it finds is written to a file in the temporary folder
+    when the process ends, never to the working directory. Not to be open while a graph is captured.
+    """
+    import torch.cuda.tunable as tunable
+    if not tunable.is_enabled():
+        tunable.set_filename(os.path.join(tempfile.gettempdir(), f"dryft_amd-products-{os.getpid()}.csv"))
+        tunable.enable(True)
+    tunable.tuning_enable(True)
+    try:
+        yield
+    finally:
+        tunable.tuning_enable(False)
 
 
 def linear_modules(dtype: torch.dtype) -> tuple[str, ...]:
