@@ -317,15 +317,17 @@ DRYFT_API int dryft_gemm_stream_swiglu_bf16(const void* x, int64_t x_stride, con
 // K is split across workgroups only (float partial sums for the consumer to add), never across the waves of one.
 // With SWIGLU a workgroup owns 32 outputs: waves 0 and 1 hold their gate rows, waves 2 and 3 their up rows, and
 // the two halves meet through LDS for T(T(silu(gate)) * up) (reference: kernels/silu_mul.py:29-32).
-template <int MT, int GB, bool SWIGLU, typename O>
+template <int MT, int GB, int DEPTH, bool SWIGLU, typename O>
 __global__ __launch_bounds__(256) void gemm_wide_kernel(const bf16_t* __restrict__ x, int64_t x_stride,
                                                         const bf16_t* __restrict__ w, O* __restrict__ y,
                                                         float* __restrict__ partials, int M, int N, int K) {
   typedef StreamShape<GB, 1> S;
+  constexpr int GROUP = GB * 64;                           // values of K in one group
   extern __shared__ __align__(16) unsigned char wide_lds[];
-  unsigned char* mine = wide_lds + (threadIdx.x / WAVE) * S::TILE_BYTES;          // this wave's weight tile
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
+  const int lane = threadIdx.x % WAVE, c = lane % 16, g = lane / 16;
+  unsigned char* mine = wide_lds + wave * S::TILE_BYTES;                          // this wave's weight tile
   unsigned char* shared = wide_lds + 4 * S::TILE_BYTES;                           // [2][4 tiles] of x
-  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE, c = lane % 16, g = lane / 16;
   const int lr = lane / S::LANES_PER_ROW, lp = lane % S::LANES_PER_ROW;
   const int cols = SWIGLU ? 32 : 64;                       // outputs a workgroup owns
   const int n0 = blockIdx.x * cols + 16 * (SWIGLU ? wave % 2 : wave);             // first output of this wave
@@ -338,51 +340,67 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(const bf16_t* __restrict
   f32x4 acc[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
-  int w_row[S::LOADS], x_row[S::LOADS];
+  const bf16_t* w_row[S::LOADS];
+  const bf16_t* x_row[S::LOADS];
 #pragma unroll
   for (int i = 0; i < S::LOADS; ++i) {
     const int r = S::ROWS_PER_LOAD * i + lr;
-    w_row[i] = min(w_row0 + r, w_last);
-    x_row[i] = min(16 * wave + r, M - 1);
+    w_row[i] = w + (int64_t)min(w_row0 + r, w_last) * K;
+    x_row[i] = x + (int64_t)min(16 * wave + r, M - 1) * x_stride;   // a wave beyond the last row stages copies of it
   }
-  const bf16_t* w_lane = w + 8 * lp;
-  const bf16_t* x_lane = x + 8 * lp;
-  const bool stages_x = 16 * wave < M;                     // this wave's tile of x has rows at all
-  bf16x8 wa[S::LOADS], xa[S::LOADS];
-#pragma unroll
-  for (int i = 0; i < S::LOADS; ++i) xa[i] = zero8g();
-  auto fetch = [&](int k0) {
-    const bool in = k0 + 8 * lp < k_end;                   // false only in the last, partial group
+  // DEPTH groups are in flight: slot d of the registers holds group d, d + DEPTH, ... Nothing in the walk is
+  // conditional, so that the compiler counts the loads in flight exactly and waits for one slot's only: a
+  // group beyond the workgroup's share of K is read from the share's last piece (a line that is in the cache
+  // already) and its activations are replaced by zeros.
+  bf16x8 wa[DEPTH][S::LOADS], xa[DEPTH][S::LOADS];
+  auto fetch = [&](auto slot, int k0) {
+    constexpr int d = decltype(slot)::value;
+    const int kk = min(k0 + 8 * lp, k_end - 8);
 #pragma unroll
     for (int i = 0; i < S::LOADS; ++i) {
-      wa[i] = in ? *(const bf16x8*)(w_lane + (int64_t)w_row[i] * K + k0) : zero8g();
-      if (stages_x) xa[i] = in ? *(const bf16x8*)(x_lane + (int64_t)x_row[i] * x_stride + k0) : zero8g();
+      wa[d][i] = *(const bf16x8*)(w_row[i] + kk);
+      xa[d][i] = *(const bf16x8*)(x_row[i] + kk);
     }
   };
-  if (k_begin < k_end) fetch(k_begin);
   int buf = 0;
-  for (int k0 = k_begin; k0 < k_end; k0 += GB * 64, buf ^= 1) {
+  auto step = [&](auto slot, int k0) {
+    constexpr int d = decltype(slot)::value;
+    const bool in = k0 + 8 * lp < k_end;
     unsigned char* xs = shared + buf * 4 * S::TILE_BYTES;
-    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "workgroup");   // this wave's reads of its weight tile are done
+    buf ^= 1;
+    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");   // this wave's reads of its weight tile come first
     __builtin_amdgcn_wave_barrier();
 #pragma unroll
     for (int i = 0; i < S::LOADS; ++i) {
       const int at = (S::ROWS_PER_LOAD * i + lr) * S::STRIDE + 16 * lp;
-      *(bf16x8*)(mine + at) = wa[i];
-      if (stages_x) *(bf16x8*)(xs + wave * S::TILE_BYTES + at) = xa[i];
+      *(bf16x8*)(mine + at) = wa[d][i];
+      *(bf16x8*)(xs + wave * S::TILE_BYTES + at) = in ? xa[d][i] : zero8g();
     }
-    if (k0 + GB * 64 < k_end) fetch(k0 + GB * 64);
+    fetch(slot, k0 + DEPTH * GROUP);
     __syncthreads();                                         // all tiles of x of this group are in place
+    // every operand of the group is asked for before the first product: the reads overlap one another
+    // instead of each product waiting a whole LDS round trip for its own
+    bf16x8 a[2 * GB], b[2 * GB][MT];
 #pragma unroll
     for (int u = 0; u < 2 * GB; ++u) {
       const int at = c * S::STRIDE + 64 * u + 16 * g;
-      const bf16x8 a = *(const bf16x8*)(mine + at);
+      a[u] = *(const bf16x8*)(mine + at);
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
-        const bf16x8 b = *(const bf16x8*)(xs + mt * S::TILE_BYTES + at);
-        acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[mt], 0, 0, 0);
-      }
+      for (int mt = 0; mt < MT; ++mt) b[u][mt] = *(const bf16x8*)(xs + mt * S::TILE_BYTES + at);
     }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int u = 0; u < 2 * GB; ++u)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u], b[u][mt], acc[mt], 0, 0, 0);
+  };
+  if (k_begin < k_end) {
+    static_for<DEPTH>([&](auto slot) {
+      fetch(slot, k_begin + decltype(slot)::value * GROUP);
+      __builtin_amdgcn_sched_barrier(0);                   // slot after slot, the order in which they are waited for
+    });
+    for (int k0 = k_begin; k0 < k_end; k0 += DEPTH * GROUP)
+      static_for<DEPTH>([&](auto slot) { step(slot, k0 + decltype(slot)::value * GROUP); });
   }
   // acc[mt][i] is output n0 + 4g + i of activation row 16 mt + c
   if (SWIGLU) {
@@ -426,13 +444,13 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(const bf16_t* __restrict
   }
 }
 
-template <int MT, int GB, bool SWIGLU, typename O>
+template <int MT, int GB, int DEPTH, bool SWIGLU, typename O>
 static int launch_wide(const void* x, int64_t x_stride, const void* w, void* y, float* partials, int M, int N, int K,
                        int splits, hipStream_t stream) {
   typedef StreamShape<GB, 1> S;
   constexpr int lds = 12 * S::TILE_BYTES;                  // four weight tiles, two buffers of four tiles of x
   static bool raised = false;                              // more dynamic LDS than the default limit allows
-  auto kernel = gemm_wide_kernel<MT, GB, SWIGLU, O>;
+  auto kernel = gemm_wide_kernel<MT, GB, DEPTH, SWIGLU, O>;
   if (lds > 64 * 1024 && !raised) {
     if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess) return -2;
     raised = true;
@@ -445,14 +463,39 @@ static int launch_wide(const void* x, int64_t x_stride, const void* w, void* y, 
 }
 
 // M <= 64. splits > 1: float partial sums go to partials[splits, M, N] and y is not written.
+template <int MT, int GB>
+static int wide_depth(const void* x, int64_t x_stride, const void* w, void* y, float* partials, int M, int N, int K,
+                      int depth, int splits, int out_f32, hipStream_t stream) {
+#define WD(DV)                                                                                                    \
+  return out_f32 ? launch_wide<MT, GB, DV, false, float>(x, x_stride, w, y, partials, M, N, K, splits, stream)    \
+                 : launch_wide<MT, GB, DV, false, bf16_t>(x, x_stride, w, y, partials, M, N, K, splits, stream)
+  switch (depth) {
+    case 1: WD(1);
+    case 2: WD(2);
+    case 3: WD(3);
+    default: return -1;
+  }
+#undef WD
+}
+
+template <int MT, int GB>
+static int wide_swiglu_depth(const void* x, int64_t x_stride, const void* w, void* y, int M, int N, int K, int depth,
+                             hipStream_t stream) {
+  switch (depth) {
+    case 1: return launch_wide<MT, GB, 1, true, bf16_t>(x, x_stride, w, y, nullptr, M, N, K, 1, stream);
+    case 2: return launch_wide<MT, GB, 2, true, bf16_t>(x, x_stride, w, y, nullptr, M, N, K, 1, stream);
+    case 3: return launch_wide<MT, GB, 3, true, bf16_t>(x, x_stride, w, y, nullptr, M, N, K, 1, stream);
+    default: return -1;
+  }
+}
+
 DRYFT_API int dryft_gemm_wide_bf16(const void* x, int64_t x_stride, const void* w, void* y, float* partials, int M,
-                                   int N, int K, int group_blocks, int splits, int out_f32, hipStream_t stream) {
+                                   int N, int K, int group_blocks, int depth, int splits, int out_f32,
+                                   hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (M > 64 || K <= 0 || K % 8 || x_stride % 8 || splits < 1 || splits > 64) return -1;
   if (splits > 1 && partials == nullptr) return -1;
-#define WD(MTV, GBV)                                                                                           \
-  return out_f32 ? launch_wide<MTV, GBV, false, float>(x, x_stride, w, y, partials, M, N, K, splits, stream)   \
-                 : launch_wide<MTV, GBV, false, bf16_t>(x, x_stride, w, y, partials, M, N, K, splits, stream)
+#define WD(MTV, GBV) return wide_depth<MTV, GBV>(x, x_stride, w, y, partials, M, N, K, depth, splits, out_f32, stream)
   switch (((M + 15) / 16) * 10 + group_blocks) {
     case 11: WD(1, 1);
     case 12: WD(1, 2);
@@ -469,10 +512,10 @@ DRYFT_API int dryft_gemm_wide_bf16(const void* x, int64_t x_stride, const void* 
 
 // M <= 64. y[M, N] = T(T(silu(x . Wg^T)) * (x . Wu^T)) with W = [Wg; Wu] of 2N rows
 DRYFT_API int dryft_gemm_wide_swiglu_bf16(const void* x, int64_t x_stride, const void* w, void* y, int M, int N, int K,
-                                          int group_blocks, hipStream_t stream) {
+                                          int group_blocks, int depth, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (M > 64 || K <= 0 || K % 8 || x_stride % 8) return -1;
-#define WS(MTV, GBV) return launch_wide<MTV, GBV, true, bf16_t>(x, x_stride, w, y, nullptr, M, N, K, 1, stream)
+#define WS(MTV, GBV) return wide_swiglu_depth<MTV, GBV>(x, x_stride, w, y, M, N, K, depth, stream)
   switch (((M + 15) / 16) * 10 + group_blocks) {
     case 11: WS(1, 1);
     case 12: WS(1, 2);

@@ -34,8 +34,8 @@ _SIGNATURES = {
     "gemm": {"dryft_gemm_tiled": [_P, _L, _P, _P, _I, _I, _I, _I, _I, _P],
              "dryft_gemm_stream_bf16": [_P, _L, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
              "dryft_gemm_stream_swiglu_bf16": [_P, _L, _P, _P, _I, _I, _I, _I, _I, _P],
-             "dryft_gemm_wide_bf16": [_P, _L, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
-             "dryft_gemm_wide_swiglu_bf16": [_P, _L, _P, _P, _I, _I, _I, _I, _P],
+             "dryft_gemm_wide_bf16": [_P, _L, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
+             "dryft_gemm_wide_swiglu_bf16": [_P, _L, _P, _P, _I, _I, _I, _I, _I, _P],
              "dryft_sum_partials": [_P, _P, _L, _I, _I, _P]},
     "sampling": {"dryft_argmax_rows": [_P, _I, _I, _L, _P, _I, _P, _P, _P],
                  "dryft_sample_rows": [_P, _I, _I, _L, _F, _P, _P, _P]},
@@ -393,11 +393,12 @@ def gemm_stream_swiglu_bf16(x, w_gate_up, out, group_blocks: int = 2, depth: int
     return out
 
 
-def gemm_wide_bf16(x, w, out, partials=None, group_blocks: int = 2, splits: int = 1) -> None:
+def gemm_wide_bf16(x, w, out, partials=None, group_blocks: int = 2, splits: int = 1, depth: int = 2) -> None:
     """``x [M<=64, K] @ w[N, K].T`` by the kernel whose workgroups share the rows of ``x`` in LDS.
 
-    ``group_blocks`` (1 or 2) is how many 64-value blocks of K are staged at a time; with
-    ``splits > 1`` the result is left as ``partials[splits, M, N]``.
+    ``group_blocks`` (1 or 2) is how many 64-value blocks of K are staged at a time and ``depth`` (1 to 3)
+    how many such groups a wave has in flight; with ``splits > 1`` the result is left as
+    ``partials[splits, M, N]``.
     """
     _gpu(x, "x", torch.bfloat16)
     _gpu(w, "w", torch.bfloat16)
@@ -406,7 +407,8 @@ def gemm_wide_bf16(x, w, out, partials=None, group_blocks: int = 2, splits: int 
     _require(w.shape == (n, k) and w.is_contiguous() and x.stride(1) == 1, "gemm_wide: x [M,K] row-major, w [N,K] contiguous")
     _require(m <= 64 and k % 8 == 0 and x.stride(0) % 8 == 0, f"gemm_wide: needs M <= 64 and K % 8 == 0, got M={m} K={k}")
     _require(x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0, "gemm_wide: operands must be 16-byte aligned")
-    _require(group_blocks in (1, 2) and 1 <= splits <= 64, "gemm_wide: group_blocks in 1, 2 and splits in 1..64")
+    _require(group_blocks in (1, 2) and depth in (1, 2, 3) and 1 <= splits <= 64,
+             "gemm_wide: group_blocks in 1, 2, depth in 1..3 and splits in 1..64")
     out_f32 = 0
     if splits > 1:
         _gpu(partials, "partials", torch.float32)
@@ -417,10 +419,10 @@ def gemm_wide_bf16(x, w, out, partials=None, group_blocks: int = 2, splits: int 
         _require(out.shape == (m, n) and out.is_contiguous() and out.dtype in (torch.float32, torch.bfloat16),
                  f"gemm_wide: out must be contiguous [{m},{n}]")
     _check(_fn("gemm", "dryft_gemm_wide_bf16")(_ptr(x), x.stride(0), _ptr(w), _ptr(out), _ptr(partials), m, n, k,
-                                               int(group_blocks), int(splits), out_f32, _stream()), "gemm_wide_bf16")
+                                               int(group_blocks), int(depth), int(splits), out_f32, _stream()), "gemm_wide_bf16")
 
 
-def gemm_wide_swiglu_bf16(x, w_gate_up, out, group_blocks: int = 2) -> torch.Tensor:
+def gemm_wide_swiglu_bf16(x, w_gate_up, out, group_blocks: int = 2, depth: int = 1) -> torch.Tensor:
     """``silu(x @ Wg.T) * (x @ Wu.T)`` for ``w_gate_up = [Wg; Wu]``, at most 64 rows, in one kernel."""
     _gpu(x, "x", torch.bfloat16)
     _gpu(w_gate_up, "w_gate_up", torch.bfloat16)
@@ -432,9 +434,9 @@ def gemm_wide_swiglu_bf16(x, w_gate_up, out, group_blocks: int = 2) -> torch.Ten
     _require(m <= 64 and k % 8 == 0 and x.stride(0) % 8 == 0, f"gemm_wide_swiglu: needs M <= 64 and K % 8 == 0, got M={m} K={k}")
     _require(x.data_ptr() % 16 == 0 and w_gate_up.data_ptr() % 16 == 0, "gemm_wide_swiglu: operands must be 16-byte aligned")
     _require(out.shape == (m, two_n // 2) and out.is_contiguous(), f"gemm_wide_swiglu: out must be [{m},{two_n // 2}]")
-    _require(group_blocks in (1, 2), "gemm_wide_swiglu: group_blocks in 1, 2")
+    _require(group_blocks in (1, 2) and depth in (1, 2, 3), "gemm_wide_swiglu: group_blocks in 1, 2 and depth in 1..3")
     _check(_fn("gemm", "dryft_gemm_wide_swiglu_bf16")(_ptr(x), x.stride(0), _ptr(w_gate_up), _ptr(out), m, two_n // 2, k,
-                                                      int(group_blocks), _stream()), "gemm_wide_swiglu_bf16")
+                                                      int(group_blocks), int(depth), _stream()), "gemm_wide_swiglu_bf16")
     return out
 
 

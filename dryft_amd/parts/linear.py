@@ -32,7 +32,7 @@ STREAM_ROWS = 16                # the most rows the line-staging kernel takes; u
 WIDE_ROWS = 64                  # the most rows the shared-activation kernel takes
 _STREAM_BLOCKS_PER_WAVE = 5     # measured on the projection shapes of 4B to 32B models inside captured graphs:
 _STREAM_WORKGROUPS = 1536       # short walks over K, as long as the launch stays under about six workgroups a unit
-_WIDE_BLOCKS = 8                # blocks of K a workgroup of the shared-activation kernel should walk
+_COMPUTE_UNITS = 256            # of the MI355X
 
 
 def stream_plan(n: int, k: int, may_split: bool) -> tuple[int, int, int]:
@@ -48,11 +48,17 @@ def stream_plan(n: int, k: int, may_split: bool) -> tuple[int, int, int]:
     return (splits, 1, 2) if splits > 1 else (1, 2, 2)
 
 
-def wide_splits(n: int, k: int) -> int:
-    """Splits of K for the shared-activation kernel where the consumer adds the partial sums."""
+def wide_plan(n: int, k: int, may_split: bool) -> tuple[int, int, int]:
+    """(splits of K across workgroups, blocks per group, groups in flight) for the shared-activation kernel.
+
+    Its workgroups are bound by their own compute unit (LDS and barriers), not by memory, so where the
+    consumer adds partial sums the split of K is chosen to give every compute unit one workgroup; measured
+    on the o and down shapes of 4B, 8B and 32B models at 24 and 64 rows.
+    """
     tiles = (n + 63) // 64
     k_blocks = (k + 63) // 64
-    return max(1, min((k_blocks + _WIDE_BLOCKS - 1) // _WIDE_BLOCKS, 1024 // tiles, k_blocks // 4, 16))
+    splits = max(1, min(_COMPUTE_UNITS // tiles, k_blocks // 4, 16)) if may_split else 1
+    return (splits, 1, 3) if splits > 1 else (1, 2, 1)
 
 
 def few_rows_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
@@ -79,21 +85,21 @@ def linear(x: torch.Tensor, w: torch.Tensor, *, out_dtype: torch.dtype | None = 
         ops.gemm_stream_bf16(x, w, out, None, group, 1, depth)
         return out
     if m <= WIDE_ROWS and few_ok:
-        splits = wide_splits(n, k) if allow_partials else 1
+        splits, group, depth = wide_plan(n, k, allow_partials)
         if splits > 1:
             partials = torch.empty((splits, m, n), dtype=torch.float32, device=x.device)
-            ops.gemm_wide_bf16(x, w, None, partials, 2, splits)
+            ops.gemm_wide_bf16(x, w, None, partials, group, splits, depth)
             return Partials(partials, splits)
         if not library_ok:
             out = torch.empty((m, n), dtype=out_dtype, device=x.device)
-            ops.gemm_wide_bf16(x, w, out, None, 2, 1)
+            ops.gemm_wide_bf16(x, w, out, None, group, 1, depth)
             return out
     if library_ok:
         return torch.mm(x, w.t())
     out = torch.empty((m, n), dtype=out_dtype, device=x.device)
     if few_ok:
         for m0 in range(0, m, WIDE_ROWS):
-            ops.gemm_wide_bf16(x[m0:m0 + WIDE_ROWS], w, out[m0:m0 + WIDE_ROWS], None, 2, 1)
+            ops.gemm_wide_bf16(x[m0:m0 + WIDE_ROWS], w, out[m0:m0 + WIDE_ROWS], None, 2, 1, 1)
         return out
     return ops.gemm_tiled(x, w, out)
 

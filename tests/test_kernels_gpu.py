@@ -439,16 +439,17 @@ def test_gemm_wide(m, n, k, group, splits):
     x, w = torch.randn(m, k).to(torch.bfloat16), (torch.randn(n, k) / math.sqrt(k)).to(torch.bfloat16)
     want = x.double() @ w.double().T
     o = ops()
+    depth = 1 + (m + n + splits) % 3                          # groups in flight: every depth meets every shape class
     if splits == 1:
         out = torch.empty(m, n, dtype=torch.float32, device=DEV)
-        o.gemm_wide_bf16(x.to(DEV), w.to(DEV), out, None, group, 1)
+        o.gemm_wide_bf16(x.to(DEV), w.to(DEV), out, None, group, 1, depth)
         close(out, want, torch.float32, what="wide float32 out")
         outb = torch.empty(m, n, dtype=torch.bfloat16, device=DEV)
-        o.gemm_wide_bf16(x.to(DEV), w.to(DEV), outb, None, group, 1)
+        o.gemm_wide_bf16(x.to(DEV), w.to(DEV), outb, None, group, 1, 1 + depth % 3)
         close(outb, want, torch.bfloat16, ulps=1.0, what="wide bfloat16 out")
     else:
         parts = torch.full((splits, m, n), float("nan"), dtype=torch.float32, device=DEV)
-        o.gemm_wide_bf16(x.to(DEV), w.to(DEV), None, parts, group, splits)
+        o.gemm_wide_bf16(x.to(DEV), w.to(DEV), None, parts, group, splits, depth)
         out = o.sum_partials(parts, torch.empty(m, n, dtype=torch.float32, device=DEV), splits)
         close(out, want, torch.float32, what="wide split-K")
 
@@ -463,7 +464,7 @@ def test_gemm_wide_swiglu(m, inter, k, group):
     gu = (x.double() @ w.double().T).to(torch.bfloat16).float()            # the unfused path rounds the product first
     want = (torch.nn.functional.silu(gu[:, :inter]).to(torch.bfloat16).float() * gu[:, inter:]).to(torch.bfloat16)
     out = torch.empty(m, inter, dtype=torch.bfloat16, device=DEV)
-    ops().gemm_wide_swiglu_bf16(x.to(DEV), w.to(DEV), out, group)
+    ops().gemm_wide_swiglu_bf16(x.to(DEV), w.to(DEV), out, group, 1 + (m + inter) % 3)
     close(out, want, torch.bfloat16, what="wide swiglu")
 
 
