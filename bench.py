@@ -148,7 +148,7 @@ def main() -> int:
         for b in (1, 64):
             points[f"decode_b{b}"] = round(decode_rate(b, max(16, args.steps // 2), max(4, args.warmup // 2))[0], 1)
     line = {
-        "metric": "decode tok/s (Qwen3-4B layer sizes, 2,048-token prompts, 4,096-token slots)",
+        "metric": f"decode tok/s ({args.preset} layer sizes, 2,048-token prompts, 4,096-token slots)",
         "value": round(tok_s, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic (random weights, uniform random token ids)",
