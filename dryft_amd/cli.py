@@ -122,7 +122,7 @@ def cmd_bench(args) -> int:
             torch.cuda.synchronize()
             t0 = time.perf_counter()
             first = None
-            for _ in engine.generate(ids, out):
+            for _ in engine.generate(ids, out, temperature=args.temperature, sample_seed=args.seed + sample):
                 if first is None:
                     first = time.perf_counter() - t0
             torch.cuda.synchronize()
@@ -232,6 +232,7 @@ def main(argv=None) -> int:
     b.add_argument("--tune", action="store_true",
                    help="first let the vendor library choose its kernels for the workloads' step sizes")
     b.add_argument("--seed", type=int, default=0)
+    b.add_argument("--temperature", type=float, default=0.0, help="0 = greedy")
     b.add_argument("--workload", action="append", help="name,batch,in,out (may repeat)")
     b.set_defaults(fn=cmd_bench)
 

@@ -38,7 +38,7 @@ _SIGNATURES = {
              "dryft_gemm_wide_swiglu_bf16": [_P, _L, _P, _P, _I, _I, _I, _I, _I, _P],
              "dryft_sum_partials": [_P, _P, _L, _I, _I, _P]},
     "sampling": {"dryft_argmax_rows": [_P, _I, _I, _L, _P, _I, _P, _P, _P],
-                 "dryft_sample_rows": [_P, _I, _I, _L, _F, _P, _P, _P]},
+                 "dryft_sample_rows": [_P, _I, _I, _L, _F, _P, _P, _I, _P, _P, _P]},
 }
 _functions: dict[str, object] = {}
 
@@ -474,6 +474,12 @@ def sample_rows(logits: torch.Tensor, temperature: float, uniforms: torch.Tensor
     rows, vocab = logits.shape
     _require(temperature > 0, "sample_rows: temperature must be positive (use argmax_rows for greedy)")
     _require(logits.stride(1) == 1 and out.numel() >= rows and uniforms.numel() >= rows, "sample_rows: bad operands")
+    chunks = 1 if vocab < 8192 else min(64, vocab // 2048)
+    chunk_max = chunk_sum = None
+    if chunks > 1:
+        chunk_max = torch.empty(rows * chunks, dtype=torch.float32, device=logits.device)
+        chunk_sum = torch.empty(rows * chunks, dtype=torch.float32, device=logits.device)
     _check(_fn("sampling", "dryft_sample_rows")(_ptr(logits), rows, vocab, logits.stride(0), float(temperature),
-                                                _ptr(uniforms), _ptr(out), _stream()), "sample_rows")
+                                                _ptr(uniforms), _ptr(out), chunks, _ptr(chunk_max), _ptr(chunk_sum),
+                                                _stream()), "sample_rows")
     return out

@@ -138,6 +138,102 @@ __global__ __launch_bounds__(64) void argmax_pick_kernel(const float* __restrict
   if (threadIdx.x == 0) out[row] = idx < vocab ? idx : 0;
 }
 
+// Temperature sampling in two stages for wide rows. Stage one: `chunks` workgroups per row each find the maximum
+// of their stretch and the sum of exp((x - max) / T) over it. Stage two, one workgroup per row: the stretches'
+// sums, brought to the row's maximum, are added in index order until the stretch that holds u * total is found;
+// that stretch is then walked in index order, each thread summing a run of its own and one thread finishing
+// inside the run that holds the target. The token is the first index whose running sum exceeds the target, as
+// in the one-stage kernel; the sums are added in another order, so a draw within rounding of a boundary between
+// two tokens may fall on the other side.
+#define PICK_THREADS 256
+
+__global__ __launch_bounds__(256) void sample_chunks_kernel(const float* __restrict__ logits, int vocab,
+                                                            int64_t row_stride, int chunks, float inv_temperature,
+                                                            float* __restrict__ chunk_max, float* __restrict__ chunk_sum) {
+  __shared__ float scratch[16];
+  const int row = blockIdx.x, chunk = blockIdx.y;
+  const int per = (vocab + chunks - 1) / chunks;
+  const int i0 = min(vocab, chunk * per), i1 = min(vocab, i0 + per);
+  const float* r = logits + row * row_stride;
+  float mx = -INFINITY;
+  for (int i = i0 + threadIdx.x; i < i1; i += blockDim.x) mx = fmaxf(mx, r[i]);
+  mx = block_max(mx, scratch);
+  float s = 0.f;
+  if (mx > -INFINITY)
+    for (int i = i0 + threadIdx.x; i < i1; i += blockDim.x) s += expf((r[i] - mx) * inv_temperature);
+  s = block_sum(s, scratch);
+  if (threadIdx.x == 0) {
+    chunk_max[row * chunks + chunk] = mx;
+    chunk_sum[row * chunks + chunk] = s;
+  }
+}
+
+__global__ __launch_bounds__(PICK_THREADS) void sample_pick_kernel(const float* __restrict__ logits, int vocab,
+                                                                   int64_t row_stride, int chunks, float inv_temperature,
+                                                                   const float* __restrict__ chunk_max,
+                                                                   const float* __restrict__ chunk_sum,
+                                                                   const float* __restrict__ uniforms,
+                                                                   int* __restrict__ out) {
+  __shared__ float scratch[16];
+  __shared__ float weight[PICK_THREADS];                   // of a stretch, later of a thread's run
+  __shared__ float s_target, s_before;
+  __shared__ int s_chunk, s_thread;
+  const int row = blockIdx.x, tid = threadIdx.x;
+  const float* r = logits + row * row_stride;
+  // chunks <= PICK_THREADS: one stretch per thread
+  const float cm = tid < chunks ? chunk_max[row * chunks + tid] : -INFINITY;
+  const float mx = block_max(cm, scratch);
+  weight[tid] = tid < chunks && cm > -INFINITY ? chunk_sum[row * chunks + tid] * expf((cm - mx) * inv_temperature) : 0.f;
+  __syncthreads();
+  if (tid == 0) {
+    float total = 0.f;
+    for (int c = 0; c < chunks; ++c) total += weight[c];
+    const float target = uniforms[row] * total;
+    float run = 0.f;
+    int c = 0;
+    for (; c < chunks - 1; ++c) {
+      if (run + weight[c] > target) break;
+      run += weight[c];
+    }
+    s_target = target;
+    s_before = run;
+    s_chunk = c;
+  }
+  __syncthreads();
+  const int per = (vocab + chunks - 1) / chunks;
+  const int i0 = min(vocab, s_chunk * per), i1 = min(vocab, i0 + per);
+  const int run_len = (per + PICK_THREADS - 1) / PICK_THREADS;
+  const int a = min(i1, i0 + tid * run_len), b = min(i1, a + run_len);
+  float mine = 0.f;
+  for (int i = a; i < b; ++i) mine += expf((r[i] - mx) * inv_temperature);
+  __syncthreads();                                         // the stretches' weights have been read
+  weight[tid] = mine;
+  __syncthreads();
+  if (tid == 0) {
+    float run = s_before;
+    int t = 0;
+    for (; t < PICK_THREADS - 1; ++t) {
+      if (run + weight[t] > s_target) break;
+      run += weight[t];
+    }
+    s_before = run;
+    s_thread = t;
+  }
+  __syncthreads();
+  if (tid != s_thread) return;
+  float run = s_before;
+  int pick = -1;
+  for (int i = a; i < b; ++i) {
+    run += expf((r[i] - mx) * inv_temperature);
+    if (run > s_target) { pick = i; break; }
+  }
+  if (pick < 0) {  // rounding left the target just beyond the sums: the last token with weight, from here down
+    pick = max((b > a ? b : i1) - 1, 0);
+    while (pick > 0 && !(expf((r[pick] - mx) * inv_temperature) > 0.f)) --pick;
+  }
+  out[row] = pick;
+}
+
 // scratch_v / scratch_i: room for n_rows * chunks entries each when chunks > 1
 DRYFT_API int dryft_argmax_rows(const float* logits, int n_rows, int vocab, int64_t row_stride, int* out, int chunks,
                                 float* scratch_v, int* scratch_i, hipStream_t stream) {
@@ -155,11 +251,23 @@ DRYFT_API int dryft_argmax_rows(const float* logits, int n_rows, int vocab, int6
   return DRYFT_LAUNCH_CHECK();
 }
 
+// chunk_max / chunk_sum: room for n_rows * chunks floats each when chunks > 1 (chunks <= 256)
 DRYFT_API int dryft_sample_rows(const float* logits, int n_rows, int vocab, int64_t row_stride, float temperature,
-                                const float* uniforms, int* out, hipStream_t stream) {
+                                const float* uniforms, int* out, int chunks, float* chunk_max, float* chunk_sum,
+                                hipStream_t stream) {
   if (n_rows <= 0) return 0;
-  if (!(temperature > 0.f)) return -1;
-  hipLaunchKernelGGL(sample_rows_kernel, dim3(n_rows), dim3(SAMPLE_THREADS), 0, stream, logits, vocab, row_stride,
-                     1.f / temperature, uniforms, out);
+  if (!(temperature > 0.f) || vocab <= 0) return -1;
+  if (chunks <= 1) {
+    hipLaunchKernelGGL(sample_rows_kernel, dim3(n_rows), dim3(SAMPLE_THREADS), 0, stream, logits, vocab, row_stride,
+                       1.f / temperature, uniforms, out);
+    return DRYFT_LAUNCH_CHECK();
+  }
+  if (chunks > PICK_THREADS || chunk_max == nullptr || chunk_sum == nullptr) return -1;
+  hipLaunchKernelGGL(sample_chunks_kernel, dim3(n_rows, chunks), dim3(256), 0, stream, logits, vocab, row_stride, chunks,
+                     1.f / temperature, chunk_max, chunk_sum);
+  int rc = DRYFT_LAUNCH_CHECK();
+  if (rc) return rc;
+  hipLaunchKernelGGL(sample_pick_kernel, dim3(n_rows), dim3(PICK_THREADS), 0, stream, logits, vocab, row_stride, chunks,
+                     1.f / temperature, chunk_max, chunk_sum, uniforms, out);
   return DRYFT_LAUNCH_CHECK();
 }

@@ -23,6 +23,7 @@ class Sampler:
         self.temperature = float(temperature)
         self._gen = torch.Generator(device="cpu")
         self._gen.manual_seed(int(seed))
+        self._staged: torch.Tensor | None = None
 
     @property
     def greedy(self) -> bool:
@@ -49,4 +50,9 @@ class Sampler:
             return ops.argmax_rows(logits, out)
         if uniforms is None:
             uniforms = self.draw(rows)
-        return ops.sample_rows(logits, self.temperature, uniforms.to(logits.device), out)
+        if uniforms.device != logits.device:
+            # through pinned memory, so that the copy is queued behind the step instead of the host waiting for it;
+            # the staging tensor is kept alive until the copy has surely run (the next draws replace it)
+            self._staged = uniforms.pin_memory()
+            uniforms = self._staged.to(logits.device, non_blocking=True)
+        return ops.sample_rows(logits, self.temperature, uniforms, out)
