@@ -209,7 +209,8 @@ __device__ __forceinline__ void page_update(RowBlock<KB>& st, f32x4 (&s)[4], con
 }
 
 // ---------------------------------------------------------------------------------------------------
-// Many rows per sequence. Grid: (pairs of 64-position query tiles, query heads / GP); 4 waves of 16 positions each.
+// Many rows per sequence. Grid: (pairs of 64-position query tiles, query heads / 2) with two heads per wave,
+// (query heads, tiles) with one; 4 waves of 16 positions each.
 // A wave serves GP query heads that share one kv head. The workgroup copies each page of keys and values
 // from the cache into LDS once (the next page's loads are in flight while the current one is used), every
 // wave reads its operands from there into registers once per page and uses them for each of its heads.
@@ -262,7 +263,7 @@ __device__ __forceinline__ void stage_load(PageStage<KB>& st, const bf16_t* __re
 }
 
 template <int KB>
-__device__ __forceinline__ void stage_store(const PageStage<KB>& st, bf16_t* k_lds, bf16_t* v_lds, int head_dim) {
+__device__ __forceinline__ void stage_store_k(const PageStage<KB>& st, bf16_t* k_lds, int head_dim) {
   const int pieces = 8 * head_dim;
 #pragma unroll
   for (int i = 0; i < KB; ++i) {
@@ -270,25 +271,43 @@ __device__ __forceinline__ void stage_store(const PageStage<KB>& st, bf16_t* k_l
     if (j < pieces) {
       const int e = 8 * j;                                   // element index within the page
       *(bf16x8*)(k_lds + (e / head_dim) * (head_dim + K_PAD) + e % head_dim) = st.k[i];
+    }
+  }
+}
+
+template <int KB>
+__device__ __forceinline__ void stage_store_v(const PageStage<KB>& st, bf16_t* v_lds, int head_dim) {
+  const int pieces = 8 * head_dim;
+#pragma unroll
+  for (int i = 0; i < KB; ++i) {
+    const int j = threadIdx.x + 256 * i;
+    if (j < pieces) {
+      const int e = 8 * j;
       *(bf16x8*)(v_lds + (e / PAGE_TOKENS) * (PAGE_TOKENS + V_PAD) + e % PAGE_TOKENS) = st.v[i];
     }
   }
 }
 
 template <int KB, bool FULL, int GP>
-__global__ __launch_bounds__(256, (GP * KB <= 8 && KB <= 4) ? 2 : 1) void attn_causal_kernel(
+__global__ __launch_bounds__(256, (GP * KB <= 8 && KB <= 4) ? (GP == 1 ? 3 : 2) : 1) void attn_causal_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
     const int* __restrict__ page_table, int max_pages, const int* __restrict__ seq_slot,
     const int* __restrict__ cu_rows, const int* __restrict__ tile_cu, const int* __restrict__ seq_start, int n_seqs,
     bf16_t* __restrict__ out, int n_heads, int n_kv, int head_dim, float scale, int window) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   const int n_tiles = tile_cu[n_seqs];
-  const int head0 = blockIdx.y * GP;
+  // Two heads per wave: a workgroup takes one tile from each end of the list (grid: pairs of tiles x heads / 2).
+  // One head per wave: one tile per workgroup, the ones with the most pages first, heads fastest (grid: heads x
+  // tiles), so that the short tiles fill the compute units that the long ones leave.
+  constexpr bool PAIRED = GP != 1;
+  const int head0 = (PAIRED ? blockIdx.y : blockIdx.x) * GP;
+  const int first_tile = PAIRED ? blockIdx.x : blockIdx.y;
   // A tile late in a sequence sees many keys, an early one few. Every workgroup takes one tile from each end
   // of the list, so all of them have about the same work.
   for (int half = 0; half < 2; ++half) {
-  const int tile = half == 0 ? n_tiles - 1 - (int)blockIdx.x : (int)blockIdx.x;
-  if (tile < 0 || tile >= n_tiles || (half == 1 && tile >= n_tiles - 1 - (int)blockIdx.x)) continue;
+  if (!PAIRED && half == 1) break;
+  const int tile = half == 0 ? n_tiles - 1 - first_tile : first_tile;
+  if (tile < 0 || tile >= n_tiles || (half == 1 && tile >= n_tiles - 1 - first_tile)) continue;
   int lo = 0, hi = n_seqs;  // the sequence whose tiles include `tile`
   while (hi - lo > 1) {
     const int mid = (lo + hi) >> 1;
@@ -332,23 +351,31 @@ __global__ __launch_bounds__(256, (GP * KB <= 8 && KB <= 4) ? 2 : 1) void attn_c
   for (int pg = pg_first; pg <= pg_last; ++pg) {
     const int buf = (pg - pg_first) & 1;
     bf16_t* const k_lds = smem + buf * k_elems;
-    bf16_t* const v_lds = smem + 2 * k_elems + buf * v_elems;
-    if (page >= 0) stage_store<KB>(stage, k_lds, v_lds, head_dim);
-    __syncthreads();   // the page is in LDS; and every wave is done with the buffer the next page will overwrite
+    // With one head per wave the values have one buffer only: three workgroups then fit a compute unit, and
+    // the third wave per SIMD covers more of the latency than the second barrier per page costs.
+    constexpr bool V_DOUBLE = GP != 1;
+    bf16_t* const v_lds = smem + 2 * k_elems + (V_DOUBLE ? buf * v_elems : 0);
+    if (page >= 0) {
+      stage_store_k<KB>(stage, k_lds, head_dim);
+      if (V_DOUBLE) stage_store_v<KB>(stage, v_lds, head_dim);
+    }
+    __syncthreads();   // the keys are in LDS; every wave is done with the page before (and the buffers it used)
+    if (!V_DOUBLE && page >= 0) stage_store_v<KB>(stage, v_lds, head_dim);
     const int page_now = page;
     page = pg < pg_last ? table[pg + 1] : -1;
     if (page >= 0)
       stage_load<KB>(stage, k_pages + ((int64_t)page * n_kv + kvh) * page_elems,
                      v_pages + ((int64_t)page * n_kv + kvh) * page_elems, head_dim);
     const int key0 = pg * PAGE_TOKENS;
-    if (page_now >= 0 && key0 <= hi_wave && key0 + PAGE_TOKENS > lo_wave) {   // some row of the wave sees some key
+    const bool sees = page_now >= 0 && key0 <= hi_wave && key0 + PAGE_TOKENS > lo_wave;   // some row sees some key
+    bf16x8 p[GP][2];
+    if (sees) {
       // every key of the page is seen by every row of the wave unless the page reaches past the wave's first row,
       // starts before a window's edge, or the wave has fewer than 16 rows
       const bool masked = key0 + PAGE_TOKENS - 1 > pos0 || rows < 16 ||
                           (window > 0 && key0 < pos0 + 15 - window + 1);
       // Every piece of a page is read from LDS once and used at once for each of the wave's heads, so that no
       // whole page of operands has to sit in registers.
-      bf16x8 p[GP][2];
       float alpha[GP];
       bool moved[GP];
       f32x4 s[GP][4];
@@ -374,6 +401,9 @@ __global__ __launch_bounds__(256, (GP * KB <= 8 && KB <= 4) ? 2 : 1) void attn_c
 #pragma unroll
           for (int dt = 0; dt < 2 * KB; ++dt) st[hh].o[dt] *= alpha[hh];
         }
+    }
+    if (!V_DOUBLE) __syncthreads();                          // the values are in LDS
+    if (sees) {
 #pragma unroll
       for (int dt = 0; dt < 2 * KB; ++dt)
 #pragma unroll
@@ -724,8 +754,10 @@ static int launch_causal(const void* q, const void* k_pages, const void* v_pages
                          int max_tiles, void* out, int n_heads, int n_kv, int head_dim, float scale, int window,
                          hipStream_t stream) {
   dim3 grid((max_tiles + 1) / 2, n_heads / GP), block(256);
-  // two pages of keys [64][D+8] and two of values [D][64+8]
-  const size_t lds = 2 * ((size_t)PAGE_TOKENS * (head_dim + K_PAD) + (size_t)head_dim * (PAGE_TOKENS + V_PAD)) * 2;
+  if (GP == 1) grid = dim3(n_heads, max_tiles);
+  if (grid.y > 65535) return -1;
+  // two pages of keys [64][D+8] and two of values [D][64+8] (one with one head per wave)
+  const size_t lds = (2 * (size_t)PAGE_TOKENS * (head_dim + K_PAD) + (GP == 1 ? 1 : 2) * (size_t)head_dim * (PAGE_TOKENS + V_PAD)) * 2;
 #define LAUNCH_CAUSAL(FULLV)                                                                                       \
   {                                                                                                                \
     auto kernel = attn_causal_kernel<KB, FULLV, GP>;                                                               \
