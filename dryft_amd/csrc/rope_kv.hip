@@ -173,16 +173,14 @@ __global__ __launch_bounds__(256) void qk_norm_rope_vec_kernel(const T* __restri
 // of its 8 features, which are the same for every head, and walks over the row's q and k heads four at a time,
 // so that it issues about a quarter of the loads per head of the kernel above. Value heads are not handled here.
 template <typename T, int LPH>   // lanes per head: head_dim / 8
-__global__ __launch_bounds__(256) void qk_norm_rope_row_kernel(const T* __restrict__ qkv, int64_t qkv_stride,
-                                                               const void* __restrict__ q_w, const void* __restrict__ k_w,
-                                                               int w_f32, int has_norm, float eps,
-                                                               const T* __restrict__ cos_t, const T* __restrict__ sin_t,
-                                                               const int* __restrict__ row_slot,
-                                                               const int* __restrict__ row_pos, T* __restrict__ q_out,
-                                                               T* __restrict__ k_pages, const int* __restrict__ page_table,
-                                                               int max_pages, int write_kv, int n_heads, int n_kv) {
+__device__ __forceinline__ void qk_norm_rope_row(int64_t row, const T* __restrict__ qkv, int64_t qkv_stride,
+                                                 const void* __restrict__ q_w, const void* __restrict__ k_w, int w_f32,
+                                                 int has_norm, float eps, const T* __restrict__ cos_t,
+                                                 const T* __restrict__ sin_t, const int* __restrict__ row_slot,
+                                                 const int* __restrict__ row_pos, T* __restrict__ q_out,
+                                                 T* __restrict__ k_pages, const int* __restrict__ page_table,
+                                                 int max_pages, int write_kv, int n_heads, int n_kv) {
   constexpr int D = 8 * LPH, PER = 256 / LPH;           // heads a workgroup handles side by side
-  const int64_t row = blockIdx.x;
   const int part = threadIdx.x % LPH, lane_head = threadIdx.x / LPH;
   const int slot = row_slot[row], pos = row_pos[row];
   if (slot < 0) {                                       // a dead row: its q is zero, nothing is cached
@@ -241,24 +239,6 @@ __global__ __launch_bounds__(256) void qk_norm_rope_row_kernel(const T* __restri
   }
 }
 
-template <typename T>
-static void launch_rope_rows(const void* qkv, int64_t qkv_stride, const void* q_w, const void* k_w, int w_f32, int has_norm,
-                             float eps, const void* cos_t, const void* sin_t, const int* row_slot, const int* row_pos,
-                             void* q_out, void* k_pages, const int* page_table, int max_pages, int write_kv, int n_rows,
-                             int n_heads, int n_kv, int head_dim, hipStream_t stream) {
-#define ROWS(LPHV)                                                                                                     \
-  hipLaunchKernelGGL((qk_norm_rope_row_kernel<T, LPHV>), dim3(n_rows), dim3(256), 0, stream, (const T*)qkv, qkv_stride, \
-                     q_w, k_w, w_f32, has_norm, eps, (const T*)cos_t, (const T*)sin_t, row_slot, row_pos, (T*)q_out,   \
-                     (T*)k_pages, page_table, max_pages, write_kv, n_heads, n_kv)
-  switch (head_dim) {
-    case 32: ROWS(4); break;
-    case 64: ROWS(8); break;
-    case 128: ROWS(16); break;
-    default: ROWS(32); break;
-  }
-#undef ROWS
-}
-
 // Values of a step with many rows: a workgroup takes 64 consecutive rows of one kv head and turns the tile in
 // LDS. Where 32 consecutive rows are one aligned block of 32 positions of one page (the usual case in a long
 // prompt), a thread writes 8 columns of a feature's row with one 16-byte store: they are two runs of four
@@ -266,18 +246,19 @@ static void launch_rope_rows(const void* qkv, int64_t qkv_stride, const void* q_
 // row's values 128 bytes apart.) head_dim must be a multiple of 8.
 #define V_TILE_ROWS 64
 #define V_TILE_LD (V_TILE_ROWS + 8)
+extern __shared__ __attribute__((aligned(16))) unsigned char v_tile_raw[];
+
 template <typename T>
-__global__ __launch_bounds__(256) void v_tile_write_kernel(const T* __restrict__ qkv, int64_t qkv_stride, int v_col0,
-                                                           const int* __restrict__ row_slot,
-                                                           const int* __restrict__ row_pos, T* __restrict__ v_pages,
-                                                           const int* __restrict__ page_table, int max_pages,
-                                                           int n_rows, int n_kv, int head_dim) {
-  extern __shared__ __attribute__((aligned(16))) unsigned char v_tile_raw[];
+__device__ __forceinline__ void v_tile_write(int tile_index, int kvh, const T* __restrict__ qkv, int64_t qkv_stride,
+                                             int v_col0, const int* __restrict__ row_slot,
+                                             const int* __restrict__ row_pos, T* __restrict__ v_pages,
+                                             const int* __restrict__ page_table, int max_pages, int n_rows, int n_kv,
+                                             int head_dim) {
   __shared__ int64_t base[V_TILE_ROWS];                     // start of the row's page for this kv head, or -1
   __shared__ int in_page[V_TILE_ROWS];                      // the row's position within its page
   __shared__ int block_ok[V_TILE_ROWS / 32];
   T* tile = (T*)v_tile_raw;                                 // [head_dim][V_TILE_LD]: already transposed
-  const int r0 = blockIdx.x * V_TILE_ROWS, kvh = blockIdx.y;
+  const int r0 = tile_index * V_TILE_ROWS;
   const int rows = min(V_TILE_ROWS, n_rows - r0);
   const int chunks = head_dim / 8;
   for (int e = threadIdx.x; e < V_TILE_ROWS * chunks; e += blockDim.x) {
@@ -331,6 +312,66 @@ __global__ __launch_bounds__(256) void v_tile_write_kernel(const T* __restrict__
   }
 }
 
+template <typename T>
+__global__ __launch_bounds__(256) void v_tile_write_kernel(const T* __restrict__ qkv, int64_t qkv_stride, int v_col0,
+                                                           const int* __restrict__ row_slot,
+                                                           const int* __restrict__ row_pos, T* __restrict__ v_pages,
+                                                           const int* __restrict__ page_table, int max_pages,
+                                                           int n_rows, int n_kv, int head_dim) {
+  v_tile_write<T>(blockIdx.x, blockIdx.y, qkv, qkv_stride, v_col0, row_slot, row_pos, v_pages, page_table, max_pages,
+                  n_rows, n_kv, head_dim);
+}
+
+// One launch for a step of many rows: the first workgroups turn the tiles of values (few, and waiting on memory
+// most of their time), the others take a row each for q and k; both read the same projection output.
+template <typename T, int LPH>
+__global__ __launch_bounds__(256) void rows_to_cache_kernel(const T* __restrict__ qkv, int64_t qkv_stride,
+                                                            const void* __restrict__ q_w, const void* __restrict__ k_w,
+                                                            int w_f32, int has_norm, float eps,
+                                                            const T* __restrict__ cos_t, const T* __restrict__ sin_t,
+                                                            const int* __restrict__ row_slot,
+                                                            const int* __restrict__ row_pos, T* __restrict__ q_out,
+                                                            T* __restrict__ k_pages, T* __restrict__ v_pages,
+                                                            const int* __restrict__ page_table, int max_pages,
+                                                            int write_kv, int n_rows, int n_heads, int n_kv, int v_tiles) {
+  const int v_blocks = v_tiles * n_kv;                      // none when nothing is cached
+  if ((int)blockIdx.x < v_blocks) {
+    v_tile_write<T>(blockIdx.x % v_tiles, blockIdx.x / v_tiles, qkv, qkv_stride, (n_heads + n_kv) * 8 * LPH, row_slot,
+                    row_pos, v_pages, page_table, max_pages, n_rows, n_kv, 8 * LPH);
+    return;
+  }
+  qk_norm_rope_row<T, LPH>((int64_t)blockIdx.x - v_blocks, qkv, qkv_stride, q_w, k_w, w_f32, has_norm, eps, cos_t, sin_t,
+                           row_slot, row_pos, q_out, k_pages, page_table, max_pages, write_kv, n_heads, n_kv);
+}
+
+template <typename T>
+static int launch_rows_to_cache(const void* qkv, int64_t qkv_stride, const void* q_w, const void* k_w, int w_f32,
+                                int has_norm, float eps, const void* cos_t, const void* sin_t, const int* row_slot,
+                                const int* row_pos, void* q_out, void* k_pages, void* v_pages, const int* page_table,
+                                int max_pages, int write_kv, int n_rows, int n_heads, int n_kv, int head_dim,
+                                hipStream_t stream) {
+  const int v_tiles = write_kv ? (n_rows + V_TILE_ROWS - 1) / V_TILE_ROWS : 0;
+  const size_t lds = (size_t)head_dim * V_TILE_LD * sizeof(T);
+#define ROWS(LPHV)                                                                                                     \
+  {                                                                                                                    \
+    auto kernel = rows_to_cache_kernel<T, LPHV>;                                                                       \
+    if (lds > 64 * 1024 &&                                                                                             \
+        hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)  \
+      return -2;                                                                                                       \
+    hipLaunchKernelGGL(kernel, dim3(v_tiles * n_kv + n_rows), dim3(256), lds, stream, (const T*)qkv, qkv_stride, q_w,  \
+                       k_w, w_f32, has_norm, eps, (const T*)cos_t, (const T*)sin_t, row_slot, row_pos, (T*)q_out,       \
+                       (T*)k_pages, (T*)v_pages, page_table, max_pages, write_kv, n_rows, n_heads, n_kv, v_tiles);      \
+  }
+  switch (head_dim) {
+    case 32: ROWS(4); break;
+    case 64: ROWS(8); break;
+    case 128: ROWS(16); break;
+    default: ROWS(32); break;
+  }
+#undef ROWS
+  return DRYFT_LAUNCH_CHECK();
+}
+
 DRYFT_API int dryft_qk_norm_rope_kv(const void* qkv, int64_t qkv_stride, const void* q_w, const void* k_w, int w_f32,
                                     int has_norm, float eps, const void* cos_t, const void* sin_t, int rot,
                                     const int* row_slot, const int* row_pos, void* q_out, void* k_pages,
@@ -343,15 +384,13 @@ DRYFT_API int dryft_qk_norm_rope_kv(const void* qkv, int64_t qkv_stride, const v
   // many rows: the values go through the tile kernel
   const int skip_v = (write_kv && n_rows >= 32 && head_dim % 8 == 0 && aligned) ? 1 : 0;
   const bool vec = aligned && rot == head_dim && (head_dim == 32 || head_dim == 64 || head_dim == 128 || head_dim == 256);
-  if (vec && skip_v && n_rows >= 64) {                  // many rows: a workgroup per row
-    if (is_f32)
-      launch_rope_rows<float>(qkv, qkv_stride, q_w, k_w, w_f32, has_norm, eps, cos_t, sin_t, row_slot, row_pos, q_out,
-                              k_pages, page_table, max_pages, write_kv, n_rows, n_heads, n_kv, head_dim, stream);
-    else
-      launch_rope_rows<bf16_t>(qkv, qkv_stride, q_w, k_w, w_f32, has_norm, eps, cos_t, sin_t, row_slot, row_pos, q_out,
-                               k_pages, page_table, max_pages, write_kv, n_rows, n_heads, n_kv, head_dim, stream);
-    int rc = DRYFT_LAUNCH_CHECK();
-    if (rc) return rc;
+  if (vec && skip_v && n_rows >= 64) {                  // many rows: a workgroup per row, and the values' tiles beside
+    return is_f32 ? launch_rows_to_cache<float>(qkv, qkv_stride, q_w, k_w, w_f32, has_norm, eps, cos_t, sin_t, row_slot,
+                                                row_pos, q_out, k_pages, v_pages, page_table, max_pages, write_kv, n_rows,
+                                                n_heads, n_kv, head_dim, stream)
+                  : launch_rows_to_cache<bf16_t>(qkv, qkv_stride, q_w, k_w, w_f32, has_norm, eps, cos_t, sin_t, row_slot,
+                                                 row_pos, q_out, k_pages, v_pages, page_table, max_pages, write_kv, n_rows,
+                                                 n_heads, n_kv, head_dim, stream);
   } else if (vec) {
     const int lph = head_dim / 8, per_block = 256 / lph;
     const int with_v = (write_kv && !skip_v) ? 1 : 0;
