@@ -132,7 +132,7 @@ DRYFT_API int dryft_add_rmsnorm(const void* res, const void* delta, int delta_ki
   if (delta_kind == 0) n_partials = 0;
   const bool aligned = (((uintptr_t)res | (uintptr_t)delta | (uintptr_t)res_out | (uintptr_t)y) & 15) == 0 &&
                        (partial_stride % 4) == 0;
-  if (width % 8 == 0 && width <= 8 * NORM_VEC_RUNS * 512 && aligned && n_rows <= 4096) {
+  if (width % 8 == 0 && width <= 8 * NORM_VEC_RUNS * 512 && aligned) {
     if (is_f32)
       launch_norm_vec<float, float>(res, delta, n_partials, partial_stride, w, w_f32, res_out, y, n_rows, width, eps, stream);
     else if (delta_kind == 2)
