@@ -308,6 +308,37 @@ def test_small_batch_unchanged_after_a_big_one(cases, dtype):
     assert list(engine.generate(small, 6)) == a, "state leaked from the larger batch"
 
 
+def test_library_tuning_keeps_results_and_slots(cases):
+    """`Engine.tune` runs stand-in steps of the given sizes while the vendor library times its candidate kernels:
+    afterwards every slot is free again, nothing more is timed, and whole prompts (whose products go through
+    the library) still match the plain implementation. A row count that does not fit is refused."""
+    import torch.cuda.tunable as tunable
+    from dryft_amd.engine.step import SeqStep
+    case = cases["B"]
+    engine = case.engine("bfloat16", max_batch=4, max_len=256, use_graph=True)
+    was_enabled = tunable.is_enabled()
+    try:
+        engine.tune([70, 200, 300])                         # 300 rows: spread over two sequences
+        assert engine.cache.slots.free_count == 4
+        assert not tunable.tuning_is_enabled()
+        with pytest.raises(ValueError):
+            engine.tune([4 * 256 + 1])
+        for rid in ("r70", "r200"):
+            tokens = case.requests[rid]
+            slots = engine.acquire(1)
+            try:
+                logits = engine.step([SeqStep(slots[0], tokens, list(range(len(tokens))))]).float().cpu()
+            finally:
+                engine.release(slots)
+            ref = case.plain_logits(rid)
+            err = float((logits - ref).abs().max()) / float(ref.abs().max())
+            assert err <= case.tolerance(rid, "bfloat16"), f"{rid}: {err}"
+    finally:
+        tunable.tuning_enable(False)
+        tunable.enable(was_enabled)
+    assert engine.cache.slots.free_count == 4
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_stop_tokens_and_more_requests_than_slots(cases, dtype):
     case = cases["A"]
