@@ -530,6 +530,137 @@ DRYFT_API int dryft_gemm_wide_swiglu_bf16(const void* x, int64_t x_stride, const
 #undef WS
 }
 
+// ------------------------------------------------------------------------------------------- block
+// Many rows: a workgroup owns a block of 128 rows by 128 outputs and walks K in steps of 64. Its 256 threads copy
+// the block's rows of x and of W for one step into LDS (whole cache lines per load; rows 32 bytes past a
+// multiple of 64 apart, the stride at which operand reads reach LDS's full rate), the next step's rows wait in
+// registers meanwhile; each of the four waves multiplies a quarter of the block, 64 by 64, with
+// v_mfma_f32_16x16x32_bf16 (four operands of x and four of W per 32 values of K feed 16 instructions). Rows beyond
+// M or N are read from a clamped, valid row and never stored; K is padded with zeros. The vendor library is
+// faster on the sizes it takes; this kernel takes the others (outputs that are no multiple of 8, results wanted
+// in float32 for many rows). With SWIGLU the 128 rows of W in a block are 64 gate rows and the 64 up rows of the
+// same outputs (W = [Wg; Wu]), and the epilogue stores T(T(silu(gate)) * up) (reference: kernels/silu_mul.py:29-32).
+#define BLOCK_M 128
+#define BLOCK_N 128
+#define BLOCK_STRIDE 160      // bytes between rows of a step in LDS: 128 of data
+
+template <bool SWIGLU, typename O>
+__global__ __launch_bounds__(256, 2) void gemm_block_kernel(const bf16_t* __restrict__ x, int64_t x_stride,
+                                                            const bf16_t* __restrict__ w, O* __restrict__ y, int M, int N,
+                                                            int K) {
+  __shared__ __align__(16) unsigned char lds[(BLOCK_M + BLOCK_N) * BLOCK_STRIDE];
+  unsigned char* const xs = lds;
+  unsigned char* const ws = lds + BLOCK_M * BLOCK_STRIDE;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE), lane = threadIdx.x % WAVE;
+  const int c = lane % 16, g = lane / 16;
+  const int wm = wave / 2, wn = wave % 2;                  // the wave's quarter
+  const int outs = SWIGLU ? BLOCK_N / 2 : BLOCK_N;         // outputs a block owns
+  const int m0 = blockIdx.y * BLOCK_M, n0 = blockIdx.x * outs;
+  // the rows this thread copies: row lr + 32 i of the block, 16-byte piece lp of the step
+  const int lr = threadIdx.x / 8, lp = threadIdx.x % 8;
+  const bf16_t* x_row[4];
+  const bf16_t* w_row[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = lr + 32 * i;
+    x_row[i] = x + (int64_t)min(m0 + r, M - 1) * x_stride;
+    int wr;                                                // row of W behind row r of the block
+    if (SWIGLU) wr = r < 64 ? min(n0 + r, N - 1) : N + min(n0 + r - 64, N - 1);
+    else wr = min(n0 + r, N - 1);
+    w_row[i] = w + (int64_t)wr * K;
+  }
+  f32x4 acc[4][4];                                         // [tile of 16 rows][tile of 16 outputs]
+#pragma unroll
+  for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt) acc[mt][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  bf16x8 xa[4], wa[4];
+  auto fetch = [&](int k0) {                               // nothing conditional: a piece beyond K is read from the
+    const int kk = min(k0 + 8 * lp, K - 8);                // row's last piece and replaced by zeros when it is stored
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      xa[i] = *(const bf16x8*)(x_row[i] + kk);
+      wa[i] = *(const bf16x8*)(w_row[i] + kk);
+    }
+  };
+  // rows of W behind the wave's four tiles of outputs, as rows of the block
+  int w_tile[4];
+#pragma unroll
+  for (int nt = 0; nt < 4; ++nt) w_tile[nt] = SWIGLU ? (nt < 2 ? 32 * wn + 16 * nt : 64 + 32 * wn + 16 * (nt - 2)) : 64 * wn + 16 * nt;
+  fetch(0);
+  for (int k0 = 0; k0 < K; k0 += 64) {
+    const bool in = k0 + 8 * lp < K;
+    __syncthreads();                                       // every wave is done with the step before
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int at = (lr + 32 * i) * BLOCK_STRIDE + 16 * lp;
+      *(bf16x8*)(xs + at) = in ? xa[i] : zero8g();
+      *(bf16x8*)(ws + at) = wa[i];
+    }
+    fetch(k0 + 64);
+    __syncthreads();
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      bf16x8 a[4], b[4];
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        a[t] = *(const bf16x8*)(ws + (w_tile[t] + c) * BLOCK_STRIDE + 64 * u + 16 * g);
+        b[t] = *(const bf16x8*)(xs + (64 * wm + 16 * t + c) * BLOCK_STRIDE + 64 * u + 16 * g);
+      }
+#pragma unroll
+      for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt) acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[nt], b[mt], acc[mt][nt], 0, 0, 0);
+    }
+  }
+  // acc[mt][nt][i] is output (tile nt) + 4g + i of row m0 + 64 wm + 16 mt + c
+#pragma unroll
+  for (int mt = 0; mt < 4; ++mt) {
+    const int m = m0 + 64 * wm + 16 * mt + c;
+    if (m >= M) continue;
+    if (SWIGLU) {
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int n = n0 + 32 * wn + 16 * nt + 4 * g + i;
+          if (n >= N) continue;
+          const float gv = rounded_as<bf16_t>(acc[mt][nt][i]), uv = rounded_as<bf16_t>(acc[mt][nt + 2][i]);
+          const float sv = rounded_as<bf16_t>(gv / (1.f + expf(-gv)));
+          store_from_float(y + (int64_t)m * N + n, sv * uv);
+        }
+    } else {
+#pragma unroll
+      for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int n = n0 + 64 * wn + 16 * nt + 4 * g + i;
+          if (n < N) store_from_float(y + (int64_t)m * N + n, acc[mt][nt][i]);
+        }
+    }
+  }
+}
+
+// Any M. y[M, N] = x . w^T (w of N rows), or with swiglu y[M, N] = T(T(silu(x . Wg^T)) * (x . Wu^T)) (w of 2N rows).
+DRYFT_API int dryft_gemm_block_bf16(const void* x, int64_t x_stride, const void* w, void* y, int M, int N, int K,
+                                    int swiglu, int out_f32, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (K <= 0 || K % 8 || x_stride % 8 || (swiglu && out_f32)) return -1;
+  const int outs = swiglu ? BLOCK_N / 2 : BLOCK_N;
+  dim3 grid((N + outs - 1) / outs, (M + BLOCK_M - 1) / BLOCK_M), block(256);
+  if (grid.y > 65535) return -1;
+  if (swiglu)
+    hipLaunchKernelGGL((gemm_block_kernel<true, bf16_t>), grid, block, 0, stream, (const bf16_t*)x, x_stride,
+                       (const bf16_t*)w, (bf16_t*)y, M, N, K);
+  else if (out_f32)
+    hipLaunchKernelGGL((gemm_block_kernel<false, float>), grid, block, 0, stream, (const bf16_t*)x, x_stride,
+                       (const bf16_t*)w, (float*)y, M, N, K);
+  else
+    hipLaunchKernelGGL((gemm_block_kernel<false, bf16_t>), grid, block, 0, stream, (const bf16_t*)x, x_stride,
+                       (const bf16_t*)w, (bf16_t*)y, M, N, K);
+  return DRYFT_LAUNCH_CHECK();
+}
+
 // y = T(sum_s partials[s]) in the order s = 0, 1, ...
 template <typename O>
 __global__ void sum_partials_kernel(const float* __restrict__ partials, O* __restrict__ y, int64_t n, int splits) {

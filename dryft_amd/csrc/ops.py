@@ -35,6 +35,7 @@ _SIGNATURES = {
              "dryft_gemm_stream_bf16": [_P, _L, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
              "dryft_gemm_stream_swiglu_bf16": [_P, _L, _P, _P, _I, _I, _I, _I, _I, _P],
              "dryft_gemm_wide_bf16": [_P, _L, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
+             "dryft_gemm_block_bf16": [_P, _L, _P, _P, _I, _I, _I, _I, _I, _P],
              "dryft_gemm_wide_swiglu_bf16": [_P, _L, _P, _P, _I, _I, _I, _I, _I, _P],
              "dryft_sum_partials": [_P, _P, _L, _I, _I, _P]},
     "sampling": {"dryft_argmax_rows": [_P, _I, _I, _L, _P, _I, _P, _P, _P],
@@ -437,6 +438,26 @@ def gemm_wide_swiglu_bf16(x, w_gate_up, out, group_blocks: int = 2, depth: int =
     _require(group_blocks in (1, 2) and depth in (1, 2, 3), "gemm_wide_swiglu: group_blocks in 1, 2 and depth in 1..3")
     _check(_fn("gemm", "dryft_gemm_wide_swiglu_bf16")(_ptr(x), x.stride(0), _ptr(w_gate_up), _ptr(out), m, two_n // 2, k,
                                                       int(group_blocks), int(depth), _stream()), "gemm_wide_swiglu_bf16")
+    return out
+
+
+def gemm_block_bf16(x, w, out, swiglu: bool = False) -> torch.Tensor:
+    """``x [M, K] @ w[N, K].T`` for any number of rows, by the kernel that owns blocks of 128 rows by 128 outputs;
+    ``out`` bfloat16 or float32. With ``swiglu``, ``w = [Wg; Wu]`` of ``2N`` rows and
+    ``out = silu(x @ Wg.T) * (x @ Wu.T)`` in bfloat16."""
+    _gpu(x, "x", torch.bfloat16)
+    _gpu(w, "w", torch.bfloat16)
+    _gpu(out, "out")
+    m, k = x.shape
+    n = w.shape[0] // 2 if swiglu else w.shape[0]
+    _require(w.dim() == 2 and w.shape[1] == k and w.is_contiguous() and x.stride(1) == 1 and (not swiglu or w.shape[0] % 2 == 0),
+             "gemm_block: x [M,K] row-major, w [N,K] (or [2N,K]) contiguous")
+    _require(k % 8 == 0 and x.stride(0) % 8 == 0, f"gemm_block: needs K % 8 == 0, got K={k}")
+    _require(x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0, "gemm_block: operands must be 16-byte aligned")
+    _require(out.shape == (m, n) and out.is_contiguous() and out.dtype in (torch.float32, torch.bfloat16) and
+             not (swiglu and out.dtype != torch.bfloat16), f"gemm_block: out must be contiguous [{m},{n}]")
+    _check(_fn("gemm", "dryft_gemm_block_bf16")(_ptr(x), x.stride(0), _ptr(w), _ptr(out), m, n, k, 1 if swiglu else 0,
+                                                1 if out.dtype == torch.float32 else 0, _stream()), "gemm_block_bf16")
     return out
 
 
