@@ -531,134 +531,152 @@ DRYFT_API int dryft_gemm_wide_swiglu_bf16(const void* x, int64_t x_stride, const
 }
 
 // ------------------------------------------------------------------------------------------- block
-// Many rows: a workgroup owns a block of 128 rows by 128 outputs and walks K in steps of 64. Its 256 threads copy
-// the block's rows of x and of W for one step into LDS (whole cache lines per load; rows 32 bytes past a
-// multiple of 64 apart, the stride at which operand reads reach LDS's full rate), the next step's rows wait in
-// registers meanwhile; each of the four waves multiplies a quarter of the block, 64 by 64, with
-// v_mfma_f32_16x16x32_bf16 (four operands of x and four of W per 32 values of K feed 16 instructions). Rows beyond
-// M or N are read from a clamped, valid row and never stored; K is padded with zeros. The vendor library is
-// faster on the sizes it takes; this kernel takes the others (outputs that are no multiple of 8, results wanted
-// in float32 for many rows). With SWIGLU the 128 rows of W in a block are 64 gate rows and the 64 up rows of the
-// same outputs (W = [Wg; Wu]), and the epilogue stores T(T(silu(gate)) * up) (reference: kernels/silu_mul.py:29-32).
-#define BLOCK_M 128
-#define BLOCK_N 128
+// Many rows: a workgroup owns a block of rows by outputs (128 x 128 with four waves, 256 x 256 with eight) and
+// walks K in steps of 64. Its threads copy the block's rows of x and of W for one step into LDS (whole cache
+// lines per load; rows 32 bytes past a multiple of 64 apart, the stride at which operand reads reach LDS's full
+// rate), the next step's rows wait in registers meanwhile; each wave multiplies its part of the block (64 x 64 or
+// 128 x 64) with v_mfma_f32_16x16x32_bf16. Rows beyond M or N are read from a clamped, valid row and never
+// stored; K is padded with zeros. What bounds it is the rate at which the caches deliver the blocks' rows (a
+// 128 x 128 block multiplies 64 flops per byte staged, a 256 x 256 block 128): 0.4-0.6 PFLOP/s at 2,048 rows,
+// 0.8-1.0 at 16,384. The vendor library is faster on the sizes it takes; this kernel takes the others (outputs
+// that are no multiple of 8, results wanted in float32 for many rows). With SWIGLU the rows of W in a block are
+// gate rows and the up rows of the same outputs (W = [Wg; Wu]), and the epilogue stores T(T(silu(gate)) * up)
+// (reference: kernels/silu_mul.py:29-32).
 #define BLOCK_STRIDE 160      // bytes between rows of a step in LDS: 128 of data
 
-template <bool SWIGLU, typename O>
-__global__ __launch_bounds__(256, 2) void gemm_block_kernel(const bf16_t* __restrict__ x, int64_t x_stride,
-                                                            const bf16_t* __restrict__ w, O* __restrict__ y, int M, int N,
-                                                            int K) {
-  __shared__ __align__(16) unsigned char lds[(BLOCK_M + BLOCK_N) * BLOCK_STRIDE];
-  unsigned char* const xs = lds;
-  unsigned char* const ws = lds + BLOCK_M * BLOCK_STRIDE;
+// WM x WN waves, each with MT x NT tiles of 16 x 16: a block of WM*MT*16 rows by WN*NT*16 rows of W
+template <int WM, int WN, int MT, int NT, bool SWIGLU, typename O>
+__global__ __launch_bounds__(64 * WM * WN, WM * WN <= 4 ? 2 : 1) void gemm_block_kernel(const bf16_t* __restrict__ x, int64_t x_stride,
+                                                                  const bf16_t* __restrict__ w, O* __restrict__ y, int M,
+                                                                  int N, int K) {
+  constexpr int THREADS = 64 * WM * WN, BM = WM * MT * 16, BN = WN * NT * 16;
+  constexpr int ROWS_PER_PASS = THREADS / 8, XP = BM / ROWS_PER_PASS, WP = BN / ROWS_PER_PASS;
+  static_assert(BM % ROWS_PER_PASS == 0 && BN % ROWS_PER_PASS == 0 && (!SWIGLU || NT % 2 == 0), "block shape");
+  extern __shared__ __align__(16) unsigned char block_lds[];
+  unsigned char* const xs = block_lds;
+  unsigned char* const ws = block_lds + BM * BLOCK_STRIDE;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE), lane = threadIdx.x % WAVE;
   const int c = lane % 16, g = lane / 16;
-  const int wm = wave / 2, wn = wave % 2;                  // the wave's quarter
-  const int outs = SWIGLU ? BLOCK_N / 2 : BLOCK_N;         // outputs a block owns
-  const int m0 = blockIdx.y * BLOCK_M, n0 = blockIdx.x * outs;
-  // the rows this thread copies: row lr + 32 i of the block, 16-byte piece lp of the step
+  const int wm = wave / WN, wn = wave % WN;                // the wave's part of the block
+  constexpr int OUTS = SWIGLU ? BN / 2 : BN;               // outputs a block owns
+  constexpr int WAVE_OUTS = OUTS / WN;
+  const int m0 = blockIdx.y * BM, n0 = blockIdx.x * OUTS;
+  // the rows this thread copies: row lr + ROWS_PER_PASS * i of the block, 16-byte piece lp of the step
   const int lr = threadIdx.x / 8, lp = threadIdx.x % 8;
-  const bf16_t* x_row[4];
-  const bf16_t* w_row[4];
+  const bf16_t* x_row[XP];
+  const bf16_t* w_row[WP];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int r = lr + 32 * i;
-    x_row[i] = x + (int64_t)min(m0 + r, M - 1) * x_stride;
+  for (int i = 0; i < XP; ++i) x_row[i] = x + (int64_t)min(m0 + lr + ROWS_PER_PASS * i, M - 1) * x_stride;
+#pragma unroll
+  for (int i = 0; i < WP; ++i) {
+    const int r = lr + ROWS_PER_PASS * i;
     int wr;                                                // row of W behind row r of the block
-    if (SWIGLU) wr = r < 64 ? min(n0 + r, N - 1) : N + min(n0 + r - 64, N - 1);
+    if (SWIGLU) wr = r < BN / 2 ? min(n0 + r, N - 1) : N + min(n0 + r - BN / 2, N - 1);
     else wr = min(n0 + r, N - 1);
     w_row[i] = w + (int64_t)wr * K;
   }
-  f32x4 acc[4][4];                                         // [tile of 16 rows][tile of 16 outputs]
+  f32x4 acc[MT][NT];                                       // [tile of 16 rows][tile of 16 outputs]
 #pragma unroll
-  for (int mt = 0; mt < 4; ++mt)
+  for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-    for (int nt = 0; nt < 4; ++nt) acc[mt][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
-  bf16x8 xa[4], wa[4];
+    for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  bf16x8 xa[XP], wa[WP];
   auto fetch = [&](int k0) {                               // nothing conditional: a piece beyond K is read from the
     const int kk = min(k0 + 8 * lp, K - 8);                // row's last piece and replaced by zeros when it is stored
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      xa[i] = *(const bf16x8*)(x_row[i] + kk);
-      wa[i] = *(const bf16x8*)(w_row[i] + kk);
-    }
-  };
-  // rows of W behind the wave's four tiles of outputs, as rows of the block
-  int w_tile[4];
+    for (int i = 0; i < XP; ++i) xa[i] = *(const bf16x8*)(x_row[i] + kk);
 #pragma unroll
-  for (int nt = 0; nt < 4; ++nt) w_tile[nt] = SWIGLU ? (nt < 2 ? 32 * wn + 16 * nt : 64 + 32 * wn + 16 * (nt - 2)) : 64 * wn + 16 * nt;
+    for (int i = 0; i < WP; ++i) wa[i] = *(const bf16x8*)(w_row[i] + kk);
+  };
+  // rows of W behind the wave's tiles of outputs, as rows of the block
+  int w_tile[NT];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt)
+    w_tile[nt] = SWIGLU ? (nt < NT / 2 ? WAVE_OUTS * wn + 16 * nt : BN / 2 + WAVE_OUTS * wn + 16 * (nt - NT / 2))
+                        : WAVE_OUTS * wn + 16 * nt;
   fetch(0);
   for (int k0 = 0; k0 < K; k0 += 64) {
     const bool in = k0 + 8 * lp < K;
     __syncthreads();                                       // every wave is done with the step before
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int at = (lr + 32 * i) * BLOCK_STRIDE + 16 * lp;
-      *(bf16x8*)(xs + at) = in ? xa[i] : zero8g();
-      *(bf16x8*)(ws + at) = wa[i];
-    }
+    for (int i = 0; i < XP; ++i) *(bf16x8*)(xs + (lr + ROWS_PER_PASS * i) * BLOCK_STRIDE + 16 * lp) = in ? xa[i] : zero8g();
+#pragma unroll
+    for (int i = 0; i < WP; ++i) *(bf16x8*)(ws + (lr + ROWS_PER_PASS * i) * BLOCK_STRIDE + 16 * lp) = wa[i];
     fetch(k0 + 64);
     __syncthreads();
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
-      bf16x8 a[4], b[4];
+      bf16x8 a[NT], b[MT];
 #pragma unroll
-      for (int t = 0; t < 4; ++t) {
-        a[t] = *(const bf16x8*)(ws + (w_tile[t] + c) * BLOCK_STRIDE + 64 * u + 16 * g);
-        b[t] = *(const bf16x8*)(xs + (64 * wm + 16 * t + c) * BLOCK_STRIDE + 64 * u + 16 * g);
-      }
+      for (int t = 0; t < NT; ++t) a[t] = *(const bf16x8*)(ws + (w_tile[t] + c) * BLOCK_STRIDE + 64 * u + 16 * g);
 #pragma unroll
-      for (int mt = 0; mt < 4; ++mt)
+      for (int t = 0; t < MT; ++t) b[t] = *(const bf16x8*)(xs + (MT * 16 * wm + 16 * t + c) * BLOCK_STRIDE + 64 * u + 16 * g);
 #pragma unroll
-        for (int nt = 0; nt < 4; ++nt) acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[nt], b[mt], acc[mt][nt], 0, 0, 0);
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[nt], b[mt], acc[mt][nt], 0, 0, 0);
     }
   }
-  // acc[mt][nt][i] is output (tile nt) + 4g + i of row m0 + 64 wm + 16 mt + c
+  // acc[mt][nt][i] is output (tile nt) + 4g + i of row m0 + MT*16*wm + 16 mt + c
 #pragma unroll
-  for (int mt = 0; mt < 4; ++mt) {
-    const int m = m0 + 64 * wm + 16 * mt + c;
+  for (int mt = 0; mt < MT; ++mt) {
+    const int m = m0 + MT * 16 * wm + 16 * mt + c;
     if (m >= M) continue;
     if (SWIGLU) {
 #pragma unroll
-      for (int nt = 0; nt < 2; ++nt)
+      for (int nt = 0; nt < NT / 2; ++nt)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          const int n = n0 + 32 * wn + 16 * nt + 4 * g + i;
+          const int n = n0 + WAVE_OUTS * wn + 16 * nt + 4 * g + i;
           if (n >= N) continue;
-          const float gv = rounded_as<bf16_t>(acc[mt][nt][i]), uv = rounded_as<bf16_t>(acc[mt][nt + 2][i]);
+          const float gv = rounded_as<bf16_t>(acc[mt][nt][i]), uv = rounded_as<bf16_t>(acc[mt][nt + NT / 2][i]);
           const float sv = rounded_as<bf16_t>(gv / (1.f + expf(-gv)));
           store_from_float(y + (int64_t)m * N + n, sv * uv);
         }
     } else {
 #pragma unroll
-      for (int nt = 0; nt < 4; ++nt)
+      for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          const int n = n0 + 64 * wn + 16 * nt + 4 * g + i;
+          const int n = n0 + WAVE_OUTS * wn + 16 * nt + 4 * g + i;
           if (n < N) store_from_float(y + (int64_t)m * N + n, acc[mt][nt][i]);
         }
     }
   }
 }
 
+template <int WM, int WN, int MT, int NT, bool SWIGLU, typename O>
+static int launch_block(const void* x, int64_t x_stride, const void* w, void* y, int M, int N, int K, hipStream_t stream) {
+  constexpr int BM = WM * MT * 16, BN = WN * NT * 16, OUTS = SWIGLU ? BN / 2 : BN;
+  constexpr int lds = (BM + BN) * BLOCK_STRIDE;
+  auto kernel = gemm_block_kernel<WM, WN, MT, NT, SWIGLU, O>;
+  static bool raised = false;                              // more dynamic LDS than the default limit allows
+  if (lds > 64 * 1024 && !raised) {
+    if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess) return -2;
+    raised = true;
+  }
+  dim3 grid((N + OUTS - 1) / OUTS, (M + BM - 1) / BM), block(64 * WM * WN);
+  if (grid.y > 65535) return -1;
+  hipLaunchKernelGGL(kernel, grid, block, lds, stream, (const bf16_t*)x, x_stride, (const bf16_t*)w, (O*)y, M, N, K);
+  return DRYFT_LAUNCH_CHECK();
+}
+
 // Any M. y[M, N] = x . w^T (w of N rows), or with swiglu y[M, N] = T(T(silu(x . Wg^T)) * (x . Wu^T)) (w of 2N rows).
+// shape: 0 = blocks of 128 x 128 (four waves), 1 = 256 x 256 (eight waves; twice the flops per byte staged)
 DRYFT_API int dryft_gemm_block_bf16(const void* x, int64_t x_stride, const void* w, void* y, int M, int N, int K,
-                                    int swiglu, int out_f32, hipStream_t stream) {
+                                    int swiglu, int out_f32, int shape, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (K <= 0 || K % 8 || x_stride % 8 || (swiglu && out_f32)) return -1;
-  const int outs = swiglu ? BLOCK_N / 2 : BLOCK_N;
-  dim3 grid((N + outs - 1) / outs, (M + BLOCK_M - 1) / BLOCK_M), block(256);
-  if (grid.y > 65535) return -1;
-  if (swiglu)
-    hipLaunchKernelGGL((gemm_block_kernel<true, bf16_t>), grid, block, 0, stream, (const bf16_t*)x, x_stride,
-                       (const bf16_t*)w, (bf16_t*)y, M, N, K);
-  else if (out_f32)
-    hipLaunchKernelGGL((gemm_block_kernel<false, float>), grid, block, 0, stream, (const bf16_t*)x, x_stride,
-                       (const bf16_t*)w, (float*)y, M, N, K);
-  else
-    hipLaunchKernelGGL((gemm_block_kernel<false, bf16_t>), grid, block, 0, stream, (const bf16_t*)x, x_stride,
-                       (const bf16_t*)w, (bf16_t*)y, M, N, K);
-  return DRYFT_LAUNCH_CHECK();
+#define BLK(WMV, WNV, MTV, NTV)                                                                                  \
+  return swiglu    ? launch_block<WMV, WNV, MTV, NTV, true, bf16_t>(x, x_stride, w, y, M, N, K, stream)          \
+         : out_f32 ? launch_block<WMV, WNV, MTV, NTV, false, float>(x, x_stride, w, y, M, N, K, stream)          \
+                   : launch_block<WMV, WNV, MTV, NTV, false, bf16_t>(x, x_stride, w, y, M, N, K, stream)
+  switch (shape) {
+    case 0: BLK(2, 2, 4, 4);
+    case 1: BLK(2, 4, 8, 4);
+    default: return -1;
+  }
+#undef BLK
 }
 
 // y = T(sum_s partials[s]) in the order s = 0, 1, ...

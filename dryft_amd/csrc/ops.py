@@ -35,7 +35,7 @@ _SIGNATURES = {
              "dryft_gemm_stream_bf16": [_P, _L, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
              "dryft_gemm_stream_swiglu_bf16": [_P, _L, _P, _P, _I, _I, _I, _I, _I, _P],
              "dryft_gemm_wide_bf16": [_P, _L, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
-             "dryft_gemm_block_bf16": [_P, _L, _P, _P, _I, _I, _I, _I, _I, _P],
+             "dryft_gemm_block_bf16": [_P, _L, _P, _P, _I, _I, _I, _I, _I, _I, _P],
              "dryft_gemm_wide_swiglu_bf16": [_P, _L, _P, _P, _I, _I, _I, _I, _I, _P],
              "dryft_sum_partials": [_P, _P, _L, _I, _I, _P]},
     "sampling": {"dryft_argmax_rows": [_P, _I, _I, _L, _P, _I, _P, _P, _P],
@@ -441,10 +441,11 @@ def gemm_wide_swiglu_bf16(x, w_gate_up, out, group_blocks: int = 2, depth: int =
     return out
 
 
-def gemm_block_bf16(x, w, out, swiglu: bool = False) -> torch.Tensor:
+def gemm_block_bf16(x, w, out, swiglu: bool = False, shape: int | None = None) -> torch.Tensor:
     """``x [M, K] @ w[N, K].T`` for any number of rows, by the kernel that owns blocks of 128 rows by 128 outputs;
     ``out`` bfloat16 or float32. With ``swiglu``, ``w = [Wg; Wu]`` of ``2N`` rows and
-    ``out = silu(x @ Wg.T) * (x @ Wu.T)`` in bfloat16."""
+    ``out = silu(x @ Wg.T) * (x @ Wu.T)`` in bfloat16. ``shape``: 0 = blocks of 128 x 128, 1 = 256 x 256; by default
+    the large blocks where there are enough of them to give every compute unit one."""
     _gpu(x, "x", torch.bfloat16)
     _gpu(w, "w", torch.bfloat16)
     _gpu(out, "out")
@@ -456,8 +457,11 @@ def gemm_block_bf16(x, w, out, swiglu: bool = False) -> torch.Tensor:
     _require(x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0, "gemm_block: operands must be 16-byte aligned")
     _require(out.shape == (m, n) and out.is_contiguous() and out.dtype in (torch.float32, torch.bfloat16) and
              not (swiglu and out.dtype != torch.bfloat16), f"gemm_block: out must be contiguous [{m},{n}]")
+    if shape is None:
+        shape = 1 if -(-m // 256) * -(-(2 * n if swiglu else n) // 256) >= 256 else 0
+    _require(shape in (0, 1), "gemm_block: shape 0 or 1")
     _check(_fn("gemm", "dryft_gemm_block_bf16")(_ptr(x), x.stride(0), _ptr(w), _ptr(out), m, n, k, 1 if swiglu else 0,
-                                                1 if out.dtype == torch.float32 else 0, _stream()), "gemm_block_bf16")
+                                                1 if out.dtype == torch.float32 else 0, int(shape), _stream()), "gemm_block_bf16")
     return out
 
 

@@ -14,8 +14,8 @@ engine/dryft_qwen3/model.py:153, 179-180, 237, 258-261). Here:
   for sizes the vendor library does not take;
 * bfloat16, otherwise (prompts, decoding at large batch): the vendor library through
   ``torch.mm``, as in the reference; float32 results of many rows and output sizes the
-  library does not take are this library's block kernel (128 rows by 128 outputs per
-  workgroup, about 0.6 of the library's speed), and what no matrix-core kernel takes goes
+  library does not take are this library's block kernel (128 x 128 or 256 x 256 outputs
+  per workgroup, about 0.6 of the library's speed), and what no matrix-core kernel takes goes
   to the plain kernel.
 """
 

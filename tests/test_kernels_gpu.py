@@ -470,14 +470,15 @@ def test_gemm_wide_swiglu(m, inter, k, group):
 
 @pytest.mark.parametrize("m,n,k", [(130, 331, 72), (1, 17, 8), (257, 128, 64), (300, 100, 1000), (128, 129, 136),
                                    (513, 2560, 2560), (64, 64, 9728)])
-def test_gemm_block(m, n, k):
+@pytest.mark.parametrize("shape", [0, 1])
+def test_gemm_block(m, n, k, shape):
     torch.manual_seed(m + n + k)
     x, w = torch.randn(m, k).to(torch.bfloat16), (torch.randn(n, k) / math.sqrt(k)).to(torch.bfloat16)
     want = x.double() @ w.double().T
     o = ops()
-    out = o.gemm_block_bf16(x.to(DEV), w.to(DEV), torch.full((m, n), float("nan"), dtype=torch.float32, device=DEV))
+    out = o.gemm_block_bf16(x.to(DEV), w.to(DEV), torch.full((m, n), float("nan"), dtype=torch.float32, device=DEV), shape=shape)
     close(out, want, torch.float32, what="block float32 out")
-    outb = o.gemm_block_bf16(x.to(DEV), w.to(DEV), torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=DEV))
+    outb = o.gemm_block_bf16(x.to(DEV), w.to(DEV), torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=DEV), shape=shape)
     close(outb, want, torch.bfloat16, ulps=1.0, what="block bfloat16 out")
     wide = torch.randn(m, k + 24).to(torch.bfloat16).to(DEV)               # rows that are not contiguous
     got = o.gemm_block_bf16(wide[:, :k], w.to(DEV), torch.empty(m, n, dtype=torch.float32, device=DEV))
@@ -485,13 +486,15 @@ def test_gemm_block(m, n, k):
 
 
 @pytest.mark.parametrize("m,inter,k", [(200, 224, 96), (129, 40, 64), (70, 37 * 8, 72), (300, 9728, 256)])
-def test_gemm_block_swiglu(m, inter, k):
+@pytest.mark.parametrize("shape", [0, 1])
+def test_gemm_block_swiglu(m, inter, k, shape):
     torch.manual_seed(m + inter)
     x = torch.randn(m, k).to(torch.bfloat16)
     w = (torch.randn(2 * inter, k) * 2 / math.sqrt(k)).to(torch.bfloat16)
     gu = (x.double() @ w.double().T).to(torch.bfloat16).float()            # the unfused path rounds the product first
     want = (torch.nn.functional.silu(gu[:, :inter]).to(torch.bfloat16).float() * gu[:, inter:]).to(torch.bfloat16)
-    out = ops().gemm_block_bf16(x.to(DEV), w.to(DEV), torch.empty(m, inter, dtype=torch.bfloat16, device=DEV), swiglu=True)
+    out = ops().gemm_block_bf16(x.to(DEV), w.to(DEV), torch.empty(m, inter, dtype=torch.bfloat16, device=DEV), swiglu=True,
+                                shape=shape)
     close(out, want, torch.bfloat16, what="block swiglu")
 
 
