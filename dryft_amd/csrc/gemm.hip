@@ -544,11 +544,38 @@ DRYFT_API int dryft_gemm_wide_swiglu_bf16(const void* x, int64_t x_stride, const
 // (reference: kernels/silu_mul.py:29-32).
 #define BLOCK_STRIDE 160      // bytes between rows of a step in LDS: 128 of data
 
-// WM x WN waves, each with MT x NT tiles of 16 x 16: a block of WM*MT*16 rows by WN*NT*16 rows of W
-template <int WM, int WN, int MT, int NT, bool SWIGLU, typename O>
-__global__ __launch_bounds__(64 * WM * WN, WM * WN <= 4 ? 2 : 1) void gemm_block_kernel(const bf16_t* __restrict__ x, int64_t x_stride,
-                                                                  const bf16_t* __restrict__ w, O* __restrict__ y, int M,
-                                                                  int N, int K) {
+// WM x WN waves, each with MT x NT tiles of 16 x 16: a block of WM*MT*16 rows by WN*NT*16 rows of W.
+// T = float: the same kernel on 32-bit values with v_mfma_f32_16x16x4_f32, which multiplies and adds in full
+// float precision (a step is then 32 values of K, and a lane's 16 bytes are 4 of them, one per instruction).
+template <typename T>
+struct BlockElem;
+template <>
+struct BlockElem<bf16_t> {
+  static constexpr int PER_PIECE = 8, STEP = 64;           // values per 16 bytes, values of K per step
+};
+template <>
+struct BlockElem<float> {
+  static constexpr int PER_PIECE = 4, STEP = 32;
+};
+
+template <typename T>
+__device__ __forceinline__ f32x4 block_mfma(f32x4 a, f32x4 b, f32x4 acc) {
+  if constexpr (sizeof(T) == 2) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), acc, 0, 0, 0);
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[i], b[i], acc, 0, 0, 0);
+    return acc;
+  }
+}
+
+template <typename T, int WM, int WN, int MT, int NT, bool SWIGLU, typename O>
+__global__ __launch_bounds__(64 * WM * WN, WM * WN <= 4 ? 2 : 1) void gemm_block_kernel(const T* __restrict__ x,
+                                                                                      int64_t x_stride,
+                                                                                      const T* __restrict__ w,
+                                                                                      O* __restrict__ y, int M, int N,
+                                                                                      int K) {
+  typedef BlockElem<T> E;
   constexpr int THREADS = 64 * WM * WN, BM = WM * MT * 16, BN = WN * NT * 16;
   constexpr int ROWS_PER_PASS = THREADS / 8, XP = BM / ROWS_PER_PASS, WP = BN / ROWS_PER_PASS;
   static_assert(BM % ROWS_PER_PASS == 0 && BN % ROWS_PER_PASS == 0 && (!SWIGLU || NT % 2 == 0), "block shape");
@@ -563,8 +590,8 @@ __global__ __launch_bounds__(64 * WM * WN, WM * WN <= 4 ? 2 : 1) void gemm_block
   const int m0 = blockIdx.y * BM, n0 = blockIdx.x * OUTS;
   // the rows this thread copies: row lr + ROWS_PER_PASS * i of the block, 16-byte piece lp of the step
   const int lr = threadIdx.x / 8, lp = threadIdx.x % 8;
-  const bf16_t* x_row[XP];
-  const bf16_t* w_row[WP];
+  const T* x_row[XP];
+  const T* w_row[WP];
 #pragma unroll
   for (int i = 0; i < XP; ++i) x_row[i] = x + (int64_t)min(m0 + lr + ROWS_PER_PASS * i, M - 1) * x_stride;
 #pragma unroll
@@ -580,13 +607,13 @@ __global__ __launch_bounds__(64 * WM * WN, WM * WN <= 4 ? 2 : 1) void gemm_block
   for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
-  bf16x8 xa[XP], wa[WP];
+  f32x4 xa[XP], wa[WP];                                    // 16 bytes each, whatever they hold
   auto fetch = [&](int k0) {                               // nothing conditional: a piece beyond K is read from the
-    const int kk = min(k0 + 8 * lp, K - 8);                // row's last piece and replaced by zeros when it is stored
+    const int kk = min(k0 + E::PER_PIECE * lp, K - E::PER_PIECE);   // row's last piece and stored as zeros
 #pragma unroll
-    for (int i = 0; i < XP; ++i) xa[i] = *(const bf16x8*)(x_row[i] + kk);
+    for (int i = 0; i < XP; ++i) xa[i] = *(const f32x4*)(x_row[i] + kk);
 #pragma unroll
-    for (int i = 0; i < WP; ++i) wa[i] = *(const bf16x8*)(w_row[i] + kk);
+    for (int i = 0; i < WP; ++i) wa[i] = *(const f32x4*)(w_row[i] + kk);
   };
   // rows of W behind the wave's tiles of outputs, as rows of the block
   int w_tile[NT];
@@ -595,26 +622,27 @@ __global__ __launch_bounds__(64 * WM * WN, WM * WN <= 4 ? 2 : 1) void gemm_block
     w_tile[nt] = SWIGLU ? (nt < NT / 2 ? WAVE_OUTS * wn + 16 * nt : BN / 2 + WAVE_OUTS * wn + 16 * (nt - NT / 2))
                         : WAVE_OUTS * wn + 16 * nt;
   fetch(0);
-  for (int k0 = 0; k0 < K; k0 += 64) {
-    const bool in = k0 + 8 * lp < K;
+  for (int k0 = 0; k0 < K; k0 += E::STEP) {
+    const bool in = k0 + E::PER_PIECE * lp < K;
     __syncthreads();                                       // every wave is done with the step before
 #pragma unroll
-    for (int i = 0; i < XP; ++i) *(bf16x8*)(xs + (lr + ROWS_PER_PASS * i) * BLOCK_STRIDE + 16 * lp) = in ? xa[i] : zero8g();
+    for (int i = 0; i < XP; ++i)
+      *(f32x4*)(xs + (lr + ROWS_PER_PASS * i) * BLOCK_STRIDE + 16 * lp) = in ? xa[i] : f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int i = 0; i < WP; ++i) *(bf16x8*)(ws + (lr + ROWS_PER_PASS * i) * BLOCK_STRIDE + 16 * lp) = wa[i];
-    fetch(k0 + 64);
+    for (int i = 0; i < WP; ++i) *(f32x4*)(ws + (lr + ROWS_PER_PASS * i) * BLOCK_STRIDE + 16 * lp) = wa[i];
+    fetch(k0 + E::STEP);
     __syncthreads();
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
-      bf16x8 a[NT], b[MT];
+      f32x4 a[NT], b[MT];
 #pragma unroll
-      for (int t = 0; t < NT; ++t) a[t] = *(const bf16x8*)(ws + (w_tile[t] + c) * BLOCK_STRIDE + 64 * u + 16 * g);
+      for (int t = 0; t < NT; ++t) a[t] = *(const f32x4*)(ws + (w_tile[t] + c) * BLOCK_STRIDE + 64 * u + 16 * g);
 #pragma unroll
-      for (int t = 0; t < MT; ++t) b[t] = *(const bf16x8*)(xs + (MT * 16 * wm + 16 * t + c) * BLOCK_STRIDE + 64 * u + 16 * g);
+      for (int t = 0; t < MT; ++t) b[t] = *(const f32x4*)(xs + (MT * 16 * wm + 16 * t + c) * BLOCK_STRIDE + 64 * u + 16 * g);
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[nt], b[mt], acc[mt][nt], 0, 0, 0);
+        for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = block_mfma<T>(a[nt], b[mt], acc[mt][nt]);
     }
   }
   // acc[mt][nt][i] is output (tile nt) + 4g + i of row m0 + MT*16*wm + 16 mt + c
@@ -629,8 +657,8 @@ __global__ __launch_bounds__(64 * WM * WN, WM * WN <= 4 ? 2 : 1) void gemm_block
         for (int i = 0; i < 4; ++i) {
           const int n = n0 + WAVE_OUTS * wn + 16 * nt + 4 * g + i;
           if (n >= N) continue;
-          const float gv = rounded_as<bf16_t>(acc[mt][nt][i]), uv = rounded_as<bf16_t>(acc[mt][nt + NT / 2][i]);
-          const float sv = rounded_as<bf16_t>(gv / (1.f + expf(-gv)));
+          const float gv = rounded_as<T>(acc[mt][nt][i]), uv = rounded_as<T>(acc[mt][nt + NT / 2][i]);
+          const float sv = rounded_as<T>(gv / (1.f + expf(-gv)));
           store_from_float(y + (int64_t)m * N + n, sv * uv);
         }
     } else {
@@ -645,11 +673,11 @@ __global__ __launch_bounds__(64 * WM * WN, WM * WN <= 4 ? 2 : 1) void gemm_block
   }
 }
 
-template <int WM, int WN, int MT, int NT, bool SWIGLU, typename O>
+template <typename T, int WM, int WN, int MT, int NT, bool SWIGLU, typename O>
 static int launch_block(const void* x, int64_t x_stride, const void* w, void* y, int M, int N, int K, hipStream_t stream) {
   constexpr int BM = WM * MT * 16, BN = WN * NT * 16, OUTS = SWIGLU ? BN / 2 : BN;
   constexpr int lds = (BM + BN) * BLOCK_STRIDE;
-  auto kernel = gemm_block_kernel<WM, WN, MT, NT, SWIGLU, O>;
+  auto kernel = gemm_block_kernel<T, WM, WN, MT, NT, SWIGLU, O>;
   static bool raised = false;                              // more dynamic LDS than the default limit allows
   if (lds > 64 * 1024 && !raised) {
     if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess) return -2;
@@ -657,7 +685,7 @@ static int launch_block(const void* x, int64_t x_stride, const void* w, void* y,
   }
   dim3 grid((N + OUTS - 1) / OUTS, (M + BM - 1) / BM), block(64 * WM * WN);
   if (grid.y > 65535) return -1;
-  hipLaunchKernelGGL(kernel, grid, block, lds, stream, (const bf16_t*)x, x_stride, (const bf16_t*)w, (O*)y, M, N, K);
+  hipLaunchKernelGGL(kernel, grid, block, lds, stream, (const T*)x, x_stride, (const T*)w, (O*)y, M, N, K);
   return DRYFT_LAUNCH_CHECK();
 }
 
@@ -667,16 +695,113 @@ DRYFT_API int dryft_gemm_block_bf16(const void* x, int64_t x_stride, const void*
                                     int swiglu, int out_f32, int shape, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (K <= 0 || K % 8 || x_stride % 8 || (swiglu && out_f32)) return -1;
-#define BLK(WMV, WNV, MTV, NTV)                                                                                  \
-  return swiglu    ? launch_block<WMV, WNV, MTV, NTV, true, bf16_t>(x, x_stride, w, y, M, N, K, stream)          \
-         : out_f32 ? launch_block<WMV, WNV, MTV, NTV, false, float>(x, x_stride, w, y, M, N, K, stream)          \
-                   : launch_block<WMV, WNV, MTV, NTV, false, bf16_t>(x, x_stride, w, y, M, N, K, stream)
+#define BLK(WMV, WNV, MTV, NTV)                                                                                        \
+  return swiglu    ? launch_block<bf16_t, WMV, WNV, MTV, NTV, true, bf16_t>(x, x_stride, w, y, M, N, K, stream)        \
+         : out_f32 ? launch_block<bf16_t, WMV, WNV, MTV, NTV, false, float>(x, x_stride, w, y, M, N, K, stream)        \
+                   : launch_block<bf16_t, WMV, WNV, MTV, NTV, false, bf16_t>(x, x_stride, w, y, M, N, K, stream)
   switch (shape) {
     case 0: BLK(2, 2, 4, 4);
     case 1: BLK(2, 4, 8, 4);
     default: return -1;
   }
 #undef BLK
+}
+
+// The same on 32-bit values: y[M, N] = x . w^T in full float precision. K and x_stride multiples of 4.
+DRYFT_API int dryft_gemm_block_f32(const void* x, int64_t x_stride, const void* w, void* y, int M, int N, int K, int shape,
+                                   hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (K <= 0 || K % 4 || x_stride % 4) return -1;
+  switch (shape) {
+    case 0: return launch_block<float, 2, 2, 4, 4, false, float>(x, x_stride, w, y, M, N, K, stream);
+    case 1: return launch_block<float, 2, 4, 8, 4, false, float>(x, x_stride, w, y, M, N, K, stream);
+    default: return -1;
+  }
+}
+
+// ------------------------------------------------------------------------------------------- rows of 32-bit values
+// At most 16 rows of 32-bit values (decoding in the float32 path): bound by reading W once. A workgroup owns 8
+// weight rows, two per wave, and walks K in chunks of 256: the rows of x for a chunk are staged in LDS once for all
+// four waves (double-buffered, one barrier per chunk), a lane takes four consecutive values of each of its weight
+// rows (16-byte loads, a wave reads 1 KB of a row per instruction; the next chunk's are in flight while this one is
+// multiplied) and the matching four of every row of x, and multiplies with plain fused multiply-adds. At the end
+// the 64 lanes' sums are added. K must be a multiple of 4; rows beyond N are read from a clamped row, never stored.
+#define ROWS_CHUNK 256
+template <int MR>
+__global__ __launch_bounds__(256) void gemm_rows_f32_kernel(const float* __restrict__ x, int64_t x_stride,
+                                                            const float* __restrict__ w, float* __restrict__ y, int M,
+                                                            int N, int K) {
+  __shared__ __align__(16) float xs[2][MR][ROWS_CHUNK + 4];
+  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+  const int n0 = blockIdx.x * 8 + 2 * wave;
+  const float* w_row[2] = {w + (int64_t)min(n0, N - 1) * K, w + (int64_t)min(n0 + 1, N - 1) * K};
+  float acc[2][MR];
+#pragma unroll
+  for (int r = 0; r < 2; ++r)
+#pragma unroll
+    for (int m = 0; m < MR; ++m) acc[r][m] = 0.f;
+  float xr[MR];                                            // thread t brings value k0 + t of every row of x
+  auto fetch_x = [&](int k0) {                             // beyond K or M: a valid address, stored as zero
+    const int k = min(k0 + (int)threadIdx.x, K - 1);
+#pragma unroll
+    for (int m = 0; m < MR; ++m) xr[m] = x[(int64_t)min(m, M - 1) * x_stride + k];
+  };
+  auto store_x = [&](int buf, int k0) {
+    const bool in = k0 + (int)threadIdx.x < K;
+#pragma unroll
+    for (int m = 0; m < MR; ++m) xs[buf][m][threadIdx.x] = (in && m < M) ? xr[m] : 0.f;
+  };
+  f32x4 wv[2], wn[2];
+  auto fetch = [&](f32x4 (&v)[2], int k0) {                // beyond K: the row's last four values, multiplied by zeros
+    const int kk = min(k0 + 4 * lane, K - 4);
+    v[0] = *(const f32x4*)(w_row[0] + kk);
+    v[1] = *(const f32x4*)(w_row[1] + kk);
+  };
+  fetch_x(0);
+  fetch(wv, 0);
+  store_x(0, 0);
+  int buf = 0;
+  for (int k0 = 0; k0 < K; k0 += ROWS_CHUNK, buf ^= 1) {
+    __syncthreads();                                       // the chunk is staged; the other buffer is free again
+    fetch_x(k0 + ROWS_CHUNK);                              // the next chunk's loads are in flight during the products
+    fetch(wn, k0 + ROWS_CHUNK);
+#pragma unroll
+    for (int m = 0; m < MR; ++m) {
+      const f32x4 xv = *(const f32x4*)&xs[buf][m][4 * lane];   // zeros beyond K
+#pragma unroll
+      for (int r = 0; r < 2; ++r)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[r][m] = fmaf(wv[r][i], xv[i], acc[r][m]);
+    }
+    store_x(buf ^ 1, k0 + ROWS_CHUNK);
+    wv[0] = wn[0];
+    wv[1] = wn[1];
+  }
+#pragma unroll
+  for (int r = 0; r < 2; ++r)
+#pragma unroll
+    for (int m = 0; m < MR; ++m) {
+      const float s = wave_sum(acc[r][m]);
+      if (lane == 0 && m < M && n0 + r < N) y[(int64_t)m * N + n0 + r] = s;
+    }
+}
+
+// M <= 16, K % 4 == 0
+DRYFT_API int dryft_gemm_rows_f32(const void* x, int64_t x_stride, const void* w, void* y, int M, int N, int K,
+                                  hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (M > 16 || K <= 0 || K % 4) return -1;
+  dim3 grid((N + 7) / 8), block(256);
+#define RW(MRV)                                                                                                \
+  hipLaunchKernelGGL(gemm_rows_f32_kernel<MRV>, grid, block, 0, stream, (const float*)x, x_stride, (const float*)w, \
+                     (float*)y, M, N, K)
+  if (M <= 1) RW(1);
+  else if (M <= 2) RW(2);
+  else if (M <= 4) RW(4);
+  else if (M <= 8) RW(8);
+  else RW(16);
+#undef RW
+  return DRYFT_LAUNCH_CHECK();
 }
 
 // y = T(sum_s partials[s]) in the order s = 0, 1, ...

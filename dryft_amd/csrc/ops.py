@@ -36,6 +36,8 @@ _SIGNATURES = {
              "dryft_gemm_stream_swiglu_bf16": [_P, _L, _P, _P, _I, _I, _I, _I, _I, _P],
              "dryft_gemm_wide_bf16": [_P, _L, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
              "dryft_gemm_block_bf16": [_P, _L, _P, _P, _I, _I, _I, _I, _I, _I, _P],
+             "dryft_gemm_block_f32": [_P, _L, _P, _P, _I, _I, _I, _I, _P],
+             "dryft_gemm_rows_f32": [_P, _L, _P, _P, _I, _I, _I, _P],
              "dryft_gemm_wide_swiglu_bf16": [_P, _L, _P, _P, _I, _I, _I, _I, _I, _P],
              "dryft_sum_partials": [_P, _P, _L, _I, _I, _P]},
     "sampling": {"dryft_argmax_rows": [_P, _I, _I, _L, _P, _I, _P, _P, _P],
@@ -462,6 +464,41 @@ def gemm_block_bf16(x, w, out, swiglu: bool = False, shape: int | None = None) -
     _require(shape in (0, 1), "gemm_block: shape 0 or 1")
     _check(_fn("gemm", "dryft_gemm_block_bf16")(_ptr(x), x.stride(0), _ptr(w), _ptr(out), m, n, k, 1 if swiglu else 0,
                                                 1 if out.dtype == torch.float32 else 0, int(shape), _stream()), "gemm_block_bf16")
+    return out
+
+
+def gemm_block_f32(x, w, out, shape: int | None = None) -> torch.Tensor:
+    """``x [M, K] @ w[N, K].T`` on float32 values with the matrix cores' full-precision instruction
+    (``v_mfma_f32_16x16x4_f32``); ``K`` a multiple of 4, operands 16-byte aligned."""
+    _gpu(x, "x", torch.float32)
+    _gpu(w, "w", torch.float32)
+    _gpu(out, "out", torch.float32)
+    m, k = x.shape
+    n = w.shape[0]
+    _require(w.shape == (n, k) and w.is_contiguous() and x.stride(1) == 1, "gemm_block_f32: x [M,K] row-major, w [N,K] contiguous")
+    _require(k % 4 == 0 and x.stride(0) % 4 == 0, f"gemm_block_f32: needs K % 4 == 0, got K={k}")
+    _require(x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0, "gemm_block_f32: operands must be 16-byte aligned")
+    _require(out.shape == (m, n) and out.is_contiguous(), f"gemm_block_f32: out must be contiguous [{m},{n}]")
+    if shape is None:
+        shape = 1 if -(-m // 256) * -(-n // 256) >= 256 else 0
+    _require(shape in (0, 1), "gemm_block_f32: shape 0 or 1")
+    _check(_fn("gemm", "dryft_gemm_block_f32")(_ptr(x), x.stride(0), _ptr(w), _ptr(out), m, n, k, int(shape), _stream()),
+           "gemm_block_f32")
+    return out
+
+
+def gemm_rows_f32(x, w, out) -> torch.Tensor:
+    """``x [M<=16, K] @ w[N, K].T`` on float32 values by plain multiply-adds, every weight read once; ``K`` a
+    multiple of 4 and ``w`` 16-byte aligned."""
+    _gpu(x, "x", torch.float32)
+    _gpu(w, "w", torch.float32)
+    _gpu(out, "out", torch.float32)
+    m, k = x.shape
+    n = w.shape[0]
+    _require(w.shape == (n, k) and w.is_contiguous() and x.stride(1) == 1, "gemm_rows_f32: x [M,K] row-major, w [N,K] contiguous")
+    _require(m <= 16 and k % 4 == 0 and w.data_ptr() % 16 == 0, f"gemm_rows_f32: needs M <= 16, K % 4 == 0, aligned w; got M={m} K={k}")
+    _require(out.shape == (m, n) and out.is_contiguous(), f"gemm_rows_f32: out must be contiguous [{m},{n}]")
+    _check(_fn("gemm", "dryft_gemm_rows_f32")(_ptr(x), x.stride(0), _ptr(w), _ptr(out), m, n, k, _stream()), "gemm_rows_f32")
     return out
 
 

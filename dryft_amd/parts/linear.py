@@ -3,8 +3,10 @@
 The reference hands every projection to a vendor library (F.linear,
 engine/dryft_qwen3/model.py:153, 179-180, 237, 258-261). Here:
 
-* float32: this library's own kernel, plain multiply-adds, so the 32-bit path has no
-  reduced-precision matrix mode anywhere;
+* float32: this library's own kernels, so the 32-bit path has no reduced-precision matrix
+  mode anywhere: plain multiply-adds that read every weight once for at most 16 rows, the
+  matrix cores' full-precision instruction (``v_mfma_f32_16x16x4_f32``) in blocks of
+  128 x 128 for more, and a plain tiled kernel for sizes those do not take;
 * bfloat16, at most 16 rows (decoding at small batch): this library's weight-streaming
   matrix-core kernel, which stages whole cache lines through LDS and can leave its result
   as float32 partial sums over K for the consumer to add;
@@ -74,7 +76,13 @@ def linear(x: torch.Tensor, w: torch.Tensor, *, out_dtype: torch.dtype | None = 
     n = w.shape[0]
     out_dtype = out_dtype or x.dtype
     if x.dtype == torch.float32:
-        return ops.gemm_tiled(x, w, torch.empty((m, n), dtype=torch.float32, device=x.device))
+        out = torch.empty((m, n), dtype=torch.float32, device=x.device)
+        if k % 4 == 0 and w.data_ptr() % 16 == 0:
+            if m <= STREAM_ROWS:
+                return ops.gemm_rows_f32(x, w, out)
+            if x.stride(0) % 4 == 0 and x.data_ptr() % 16 == 0:
+                return ops.gemm_block_f32(x, w, out, shape=0)
+        return ops.gemm_tiled(x, w, out)
     few_ok = few_rows_ok(x, w)
     library_ok = k % 8 == 0 and n % 8 == 0 and x.is_contiguous() and out_dtype == x.dtype
     if m <= STREAM_ROWS and few_ok:

@@ -498,6 +498,31 @@ def test_gemm_block_swiglu(m, inter, k, shape):
     close(out, want, torch.bfloat16, what="block swiglu")
 
 
+@pytest.mark.parametrize("m,n,k", [(130, 331, 72), (1, 17, 4), (257, 128, 64), (300, 100, 1000), (128, 129, 136),
+                                   (513, 700, 2560)])
+@pytest.mark.parametrize("shape", [0, 1])
+def test_gemm_block_f32(m, n, k, shape):
+    torch.manual_seed(m + n + k)
+    x, w = torch.randn(m, k), torch.randn(n, k) / math.sqrt(k)
+    out = ops().gemm_block_f32(x.to(DEV), w.to(DEV), torch.full((m, n), float("nan"), device=DEV), shape=shape)
+    close(out, x.double() @ w.double().T, torch.float32, what="block float32")
+    wide = torch.randn(m, k + 12).to(DEV)                                  # rows that are not contiguous
+    got = ops().gemm_block_f32(wide[:, :k], w.to(DEV), torch.empty(m, n, device=DEV), shape=shape)
+    close(got, wide[:, :k].cpu().double() @ w.double().T, torch.float32, what="block float32 strided rows")
+
+
+@pytest.mark.parametrize("m", [1, 2, 3, 5, 8, 11, 16])
+@pytest.mark.parametrize("n,k", [(17, 4), (331, 72), (100, 1000), (129, 260), (64, 2560), (2560, 256)])
+def test_gemm_rows_f32(m, n, k):
+    torch.manual_seed(m + n + k)
+    x, w = torch.randn(m, k), torch.randn(n, k) / math.sqrt(k)
+    out = ops().gemm_rows_f32(x.to(DEV), w.to(DEV), torch.full((m, n), float("nan"), device=DEV))
+    close(out, x.double() @ w.double().T, torch.float32, what="rows float32")
+    wide = torch.randn(m, k + 3).to(DEV)                                   # rows of a wider matrix, not even aligned
+    got = ops().gemm_rows_f32(wide[:, :k], w.to(DEV), torch.empty(m, n, device=DEV))
+    close(got, wide[:, :k].cpu().double() @ w.double().T, torch.float32, what="rows float32 strided rows")
+
+
 def test_linear_dispatch_matches_everywhere():
     """The same product through every route the linear helper can take."""
     from dryft_amd.parts.linear import linear
