@@ -422,6 +422,48 @@ def test_graph_replay_equals_eager(cases, dtype):
 
 
 # --------------------------------------------------------------------------------- the program
+def test_layer_sizes_of_a_real_model_bfloat16_agrees_with_float32():
+    """Two layers with Qwen3-4B's sizes (head size 128, four query heads to a kv head, widths 2560 / 9728, the
+    151,936-token head), the sizes at which the matrix-core kernels take their fast paths: the bfloat16 engine
+    against the float32 engine, which shares no matrix kernel with it. Prompts of unequal length in one step (one
+    long enough for two heads per wave in the prompt attention, which starts at 4,096 positions of 32 heads),
+    then decoding through captured graphs at 3 sequences, and 40 sequences for the products of 17 to 64 rows."""
+    from dryft_amd import Engine
+    from dryft_amd.engine.step import SeqStep
+    from dryft_amd.models.qwen3 import load_preset
+    raw = dict(load_preset("qwen3-4b"))
+    raw["num_hidden_layers"] = 2
+    vocab = raw["vocab_size"]
+    engines = {dt: Engine(config=raw, seed=5, dtype=dt, max_batch=40, max_len=4608, max_tokens=40 * 320 + 3 * 4608)
+               for dt in ("float32", "bfloat16")}
+    prompts = [random_tokens(n, vocab, seed=7 + n) for n in (4200, 70, 300)]
+    follow = [random_tokens(6, vocab, seed=50 + i) for i in range(3)]
+    many = [random_tokens(100 + i, vocab, seed=200 + i) for i in range(40)]
+    got = {}
+    for dt, eng in engines.items():
+        slots = eng.acquire(3)
+        rows = [eng.step([SeqStep(s, p, [len(p) - 1]) for s, p in zip(slots, prompts)]).float().cpu()]
+        for t in range(6):                                      # given tokens, so both engines see the same ones
+            rows.append(eng.step([SeqStep(s, [f[t]], [0]) for s, f in zip(slots, follow)]).float().cpu())
+        eng.release(slots)
+        slots = eng.acquire(40)
+        rows.append(eng.step([SeqStep(s, p, [len(p) - 1]) for s, p in zip(slots, many)]).float().cpu())
+        rows.append(eng.step([SeqStep(s, [p[0]], [0]) for s, p in zip(slots, many)]).float().cpu())
+        eng.release(slots)
+        got[dt] = torch.cat(rows)
+        del eng
+    ref, low = got["float32"], got["bfloat16"]
+    assert torch.isfinite(ref).all() and torch.isfinite(low).all()
+    err = float((low - ref).abs().max()) / float(ref.abs().max())
+    assert err <= TOL["bfloat16"], err
+    # and through the generation loop with captured graphs: the same greedy tokens where float32 leaves no doubt
+    greedy = {dt: engines[dt].generate_all([p[:200] for p in prompts], 5) for dt in engines}
+    margin_ok = 0
+    for a, b in zip(greedy["float32"], greedy["bfloat16"]):
+        margin_ok += a[0] == b[0]
+    assert margin_ok >= 2
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_trace_run_program(cases, dtype, tmp_path):
     case = cases["B"]
