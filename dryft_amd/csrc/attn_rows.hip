@@ -17,7 +17,7 @@ template <typename T>
 __global__ void attn_rows_kernel(const T* __restrict__ q, const T* __restrict__ k_pages, const T* __restrict__ v_pages,
                                  const int* __restrict__ page_table, int max_pages, const int* __restrict__ row_slot,
                                  const int* __restrict__ row_pos, T* __restrict__ out, int n_heads, int n_kv,
-                                 int head_dim, float scale, int window) {
+                                 int head_dim, float scale, int window, int vec) {
   __shared__ float qs[ROWS_MAX_HEAD_DIM];
   __shared__ float ps[ROWS_THREADS];
   __shared__ int pages[ROWS_THREADS / PAGE_TOKENS];
@@ -49,7 +49,16 @@ __global__ void attn_rows_kernel(const T* __restrict__ q, const T* __restrict__ 
     if (seen) {
       const T* kp = k_pages + (((int64_t)page * n_kv + kvh) * PAGE_TOKENS + j % PAGE_TOKENS) * head_dim;
       float d = 0.f;
-      for (int i = 0; i < head_dim; ++i) d += qs[i] * load_as_float(kp + i);
+      if (vec) {                                           // head_dim % 8 == 0, 16-byte aligned: 8 values a load
+        for (int i = 0; i < head_dim; i += 8) {
+          float kv[8];
+          load8_as_float(kp + i, kv);
+#pragma unroll
+          for (int u = 0; u < 8; ++u) d += qs[i + u] * kv[u];
+        }
+      } else {
+        for (int i = 0; i < head_dim; ++i) d += qs[i] * load_as_float(kp + i);
+      }
       s = d * scale;
     }
     const float m_new = fmaxf(m, block_max(s, scratch));  // finite: every chunk holds a key the row sees
@@ -61,11 +70,31 @@ __global__ void attn_rows_kernel(const T* __restrict__ q, const T* __restrict__ 
     if (tid < head_dim) {
       acc *= alpha;
       const int n = min(ROWS_THREADS, pos - c + 1);
-      for (int jj = 0; jj < n; ++jj) {
-        const int pg = pages[jj / PAGE_TOKENS];
-        if (pg < 0) continue;
-        const T* vp = v_pages + (((int64_t)pg * n_kv + kvh) * head_dim + tid) * PAGE_TOKENS + value_column(jj % PAGE_TOKENS);
-        acc += ps[jj] * load_as_float(vp);
+      if (vec) {
+        // a feature's 64 values of a page in the order they are stored, 8 a load: columns 8g..8g+3 of a block of
+        // 32 are positions 4g..4g+3, columns 8g+4..8g+7 positions 16+4g.. (value_column); keys the row does not
+        // see have weight 0 and their values, whatever was stored there before, are finite
+        for (int pi = 0; pi * PAGE_TOKENS < n; ++pi) {
+          const int pg = pages[pi];
+          if (pg < 0) continue;
+          const T* vrow = v_pages + (((int64_t)pg * n_kv + kvh) * head_dim + tid) * PAGE_TOKENS;
+          const float* pw = ps + pi * PAGE_TOKENS;
+#pragma unroll
+          for (int c8 = 0; c8 < PAGE_TOKENS / 8; ++c8) {
+            float vv[8];
+            load8_as_float(vrow + 8 * c8, vv);
+            const int at = 32 * (c8 / 4) + 4 * (c8 % 4);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc += pw[at + i] * vv[i] + pw[at + 16 + i] * vv[4 + i];
+          }
+        }
+      } else {
+        for (int jj = 0; jj < n; ++jj) {
+          const int pg = pages[jj / PAGE_TOKENS];
+          if (pg < 0) continue;
+          const T* vp = v_pages + (((int64_t)pg * n_kv + kvh) * head_dim + tid) * PAGE_TOKENS + value_column(jj % PAGE_TOKENS);
+          acc += ps[jj] * load_as_float(vp);
+        }
       }
     }
     m = m_new;
@@ -80,13 +109,14 @@ DRYFT_API int dryft_attn_rows(const void* q, const void* k_pages, const void* v_
   if (n_rows <= 0) return 0;
   if (head_dim > ROWS_MAX_HEAD_DIM || n_kv <= 0 || n_heads % n_kv) return -1;
   dim3 grid(n_rows, n_heads), block(ROWS_THREADS);
+  const int vec = head_dim % 8 == 0 && (((uintptr_t)k_pages | (uintptr_t)v_pages) & 15) == 0;
   if (is_f32)
     hipLaunchKernelGGL(attn_rows_kernel<float>, grid, block, 0, stream, (const float*)q, (const float*)k_pages,
                        (const float*)v_pages, page_table, max_pages, row_slot, row_pos, (float*)out, n_heads, n_kv,
-                       head_dim, scale, window);
+                       head_dim, scale, window, vec);
   else
     hipLaunchKernelGGL(attn_rows_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)q, (const bf16_t*)k_pages,
                        (const bf16_t*)v_pages, page_table, max_pages, row_slot, row_pos, (bf16_t*)out, n_heads, n_kv,
-                       head_dim, scale, window);
+                       head_dim, scale, window, vec);
   return DRYFT_LAUNCH_CHECK();
 }
