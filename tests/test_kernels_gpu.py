@@ -247,7 +247,7 @@ CASES = [  # n_heads, n_kv, D, lengths (cached tokens incl. the rows'), q rows p
 ]
 
 
-def run_attention_case(kind, dtype, n_heads, n_kv, D, lengths, tq, window=None, seed=0):
+def run_attention_case(kind, dtype, n_heads, n_kv, D, lengths, tq, window=None, seed=0, misaligned=False):
     torch.manual_seed(seed + D + len(lengths))
     B, L = len(lengths), max(lengths)
     n_slots, n_pages = B + 2, sum((n + 63) // 64 for n in lengths) + 3
@@ -277,7 +277,14 @@ def run_attention_case(kind, dtype, n_heads, n_kv, D, lengths, tq, window=None, 
     o = ops()
     w = window or 0
     if kind == "rows":
-        o.attn_rows(d(q_packed), d(k_pages), d(v_pages), d(table), d(row_slot), d(row_pos), out, n_heads, n_kv, D, scale, w)
+        kp, vp = d(k_pages), d(v_pages)
+        if misaligned:                                       # pages that start one value past a 16-byte boundary
+            def shifted(t):
+                view = torch.empty(t.numel() + 1, dtype=t.dtype, device=DEV)[1:].view(t.shape)
+                view.copy_(t)
+                return view
+            kp, vp = shifted(kp), shifted(vp)
+        o.attn_rows(d(q_packed), kp, vp, d(table), d(row_slot), d(row_pos), out, n_heads, n_kv, D, scale, w)
     elif kind == "causal":
         o.attn_causal_bf16(d(q_packed), d(k_pages), d(v_pages), d(table), d(torch.tensor(slots, dtype=torch.int32)),
                            d(torch.from_numpy(cu)), d(torch.from_numpy(tiles)),
@@ -297,6 +304,13 @@ def run_attention_case(kind, dtype, n_heads, n_kv, D, lengths, tq, window=None, 
 @pytest.mark.parametrize("case", CASES)
 def test_attn_rows(dtype, case):
     run_attention_case("rows", dtype, *case)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_attn_rows_takes_pages_at_any_address(dtype):
+    """Pages that are not 16-byte aligned go value by value instead of eight a load."""
+    run_attention_case("rows", dtype, 6, 3, 48, [200, 70, 130], 33, misaligned=True)
+    run_attention_case("rows", dtype, 8, 2, 32, [200, 70, 130], 200, window=70, misaligned=True)
 
 
 @pytest.mark.parametrize("case", CASES)
