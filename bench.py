@@ -143,10 +143,13 @@ def main() -> int:
         pf_tok_s, pf_ms = prefill_rate()
         peak = PEAK_FLOPS["bf16" if args.dtype == "bfloat16" else "fp32"]
         pf_frac = prefill_flops(cfg, layers, PROMPT) / (pf_ms * 1e-3) / peak
-    points = {}
+    points, points_frac = {}, {}
     if not args.no_points and args.phase == "all":
         for b in (1, 64):
-            points[f"decode_b{b}"] = round(decode_rate(b, max(16, args.steps // 2), max(4, args.warmup // 2))[0], 1)
+            rate, ms, ctx = decode_rate(b, max(16, args.steps // 2), max(4, args.warmup // 2))
+            points[f"decode_b{b}"] = round(rate, 1)
+            # the same roofline as the main batch: bytes the step has to read / its time / the HBM peak
+            points_frac[f"decode_b{b}"] = round(decode_bytes(cfg, layers, b, ctx, elem) / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
     line = {
         "metric": f"decode tok/s ({args.preset} layer sizes, 2,048-token prompts, 4,096-token slots)",
         "value": round(tok_s, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -165,6 +168,7 @@ def main() -> int:
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4)},
         "points": points,
+        "points_frac": points_frac,
     }
     print(json.dumps(line))
     return 0
