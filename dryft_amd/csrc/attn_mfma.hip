@@ -288,57 +288,91 @@ __device__ __forceinline__ void stage_store_v(const PageStage<KB>& st, bf16_t* v
   }
 }
 
-template <int KB, bool FULL, int GP>
-__global__ __launch_bounds__(256, (GP * KB <= 8 && KB <= 4) ? (GP == 1 ? 3 : 2) : 1) void attn_causal_kernel(
+// A wave serves U = GP * RP units: GP query heads of one kv group, each over RP tiles of 16 consecutive rows. Every
+// piece of a page that a wave reads from LDS is used for all its units, so two units halve the LDS reads per
+// matrix instruction. A workgroup's tile is 64 * RP rows.
+template <int KB, bool FULL, int GP, int RP>
+__global__ __launch_bounds__(256, (GP * RP * KB <= 8 && KB <= 4) ? (GP * RP == 1 ? 3 : 2) : 1) void attn_causal_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
     const int* __restrict__ page_table, int max_pages, const int* __restrict__ seq_slot,
     const int* __restrict__ cu_rows, const int* __restrict__ tile_cu, const int* __restrict__ seq_start, int n_seqs,
     bf16_t* __restrict__ out, int n_heads, int n_kv, int head_dim, float scale, int window) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
-  const int n_tiles = tile_cu[n_seqs];
+  constexpr int U = GP * RP, TILE_ROWS = 64 * RP, WAVE_ROWS = 16 * RP;
   // Two heads per wave: a workgroup takes one tile from each end of the list (grid: pairs of tiles x heads / 2).
-  // One head per wave: one tile per workgroup, the ones with the most pages first, heads fastest (grid: heads x
-  // tiles), so that the short tiles fill the compute units that the long ones leave.
+  // Otherwise: one tile per workgroup, the ones with the most pages first, heads fastest (grid: heads x tiles),
+  // so that the short tiles fill the compute units that the long ones leave.
   constexpr bool PAIRED = GP != 1;
   const int head0 = (PAIRED ? blockIdx.y : blockIdx.x) * GP;
   const int first_tile = PAIRED ? blockIdx.x : blockIdx.y;
-  // A tile late in a sequence sees many keys, an early one few. Every workgroup takes one tile from each end
-  // of the list, so all of them have about the same work.
+  int n_tiles;                                                // tiles of TILE_ROWS rows over all sequences
+  if (RP == 1) {
+    n_tiles = tile_cu[n_seqs];
+  } else {
+    n_tiles = 0;
+    for (int sq = 0; sq < n_seqs; ++sq) n_tiles += (cu_rows[sq + 1] - cu_rows[sq] + TILE_ROWS - 1) / TILE_ROWS;
+  }
+  // A tile late in a sequence sees many keys, an early one few. With pairs every workgroup takes one tile from
+  // each end of the list, so all of them have about the same work.
   for (int half = 0; half < 2; ++half) {
   if (!PAIRED && half == 1) break;
   const int tile = half == 0 ? n_tiles - 1 - first_tile : first_tile;
   if (tile < 0 || tile >= n_tiles || (half == 1 && tile >= n_tiles - 1 - first_tile)) continue;
-  int lo = 0, hi = n_seqs;  // the sequence whose tiles include `tile`
-  while (hi - lo > 1) {
-    const int mid = (lo + hi) >> 1;
-    if (tile_cu[mid] <= tile) lo = mid; else hi = mid;
+  int seq, tile_in_seq;                                       // the sequence whose tiles include `tile`
+  if (RP == 1) {
+    int lo = 0, hi = n_seqs;
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) >> 1;
+      if (tile_cu[mid] <= tile) lo = mid; else hi = mid;
+    }
+    while (lo + 1 < n_seqs && tile_cu[lo + 1] <= tile) ++lo;
+    seq = lo;
+    tile_in_seq = tile - tile_cu[seq];
+  } else {
+    seq = 0;
+    tile_in_seq = tile;
+    for (;;) {
+      const int cnt = (cu_rows[seq + 1] - cu_rows[seq] + TILE_ROWS - 1) / TILE_ROWS;
+      if (tile_in_seq < cnt || seq + 1 >= n_seqs) break;
+      tile_in_seq -= cnt;
+      ++seq;
+    }
   }
-  while (lo + 1 < n_seqs && tile_cu[lo + 1] <= tile) ++lo;
-  const int seq = lo, slot = seq_slot[seq];
+  const int slot = seq_slot[seq];
   if (slot < 0) continue;                                     // the whole workgroup skips the tile together
   __syncthreads();                                            // the previous tile's pages are no longer read
   const int k_elems = PAGE_TOKENS * (head_dim + K_PAD), v_elems = head_dim * (PAGE_TOKENS + V_PAD);
   bf16_t* const smem = (bf16_t*)lds_raw;    // [2][64][D+8] keys, then [2][D][64+8] values
   const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE, c = lane % 16, g = lane / 16;
   const int q_len = cu_rows[seq + 1] - cu_rows[seq];
-  const int tile_first = (tile - tile_cu[seq]) * 64;          // first row of the tile within the sequence
-  const int first = tile_first + 16 * wave;                   // first of the wave's rows
-  const int rows = max(0, min(16, q_len - first));            // a wave past the sequence's end has none
-  const bool row_valid = c < rows;
-  const int64_t row = (int64_t)cu_rows[seq] + first + c;
-  const int kvh = head0 / (n_heads / n_kv);
-  RowBlock<KB> st[GP];
-#pragma unroll
-  for (int hh = 0; hh < GP; ++hh)
-    init_rows<KB>(st[hh], q + (row * n_heads + head0 + hh) * head_dim, row_valid, head_dim);
+  const int tile_first = tile_in_seq * TILE_ROWS;             // first row of the tile within the sequence
+  const int wave_first = tile_first + WAVE_ROWS * wave;       // first of the wave's rows
+  const int wave_rows = max(0, min(WAVE_ROWS, q_len - wave_first));   // a wave past the sequence's end has none
   const int pos_tile = seq_start[seq] + tile_first;           // position of the tile's first row
-  const int pos0 = pos_tile + 16 * wave;
-  const int pos_row = row_valid ? pos0 + c : -1;              // an absent row sees nothing
-  const int lo_row = window > 0 ? max(0, pos_row - window + 1) : 0;
-  const int lo_wave = window > 0 ? max(0, pos0 - window + 1) : 0;
-  const int hi_wave = pos0 + rows - 1;                        // below lo_wave for a wave without rows
+  const int pos_wave = pos_tile + WAVE_ROWS * wave;
+  // per tile of 16 rows
+  int rows[RP], pos0[RP], pos_row[RP], lo_row[RP];
+  bool row_valid[RP];
+  int64_t row[RP];
+#pragma unroll
+  for (int rt = 0; rt < RP; ++rt) {
+    const int first = wave_first + 16 * rt;
+    rows[rt] = max(0, min(16, q_len - first));
+    row_valid[rt] = c < rows[rt];
+    row[rt] = (int64_t)cu_rows[seq] + first + c;
+    pos0[rt] = pos_wave + 16 * rt;
+    pos_row[rt] = row_valid[rt] ? pos0[rt] + c : -1;          // an absent row sees nothing
+    lo_row[rt] = window > 0 ? max(0, pos_row[rt] - window + 1) : 0;
+  }
+  const int kvh = head0 / (n_heads / n_kv);
+  RowBlock<KB> st[U];                                         // unit u: head u % GP, rows of tile u / GP
+#pragma unroll
+  for (int u = 0; u < U; ++u)
+    init_rows<KB>(st[u], q + (row[u / GP] * n_heads + head0 + u % GP) * head_dim, row_valid[u / GP], head_dim);
+  const int lo_wave = window > 0 ? max(0, pos_wave - window + 1) : 0;
+  const int hi_wave = pos_wave + wave_rows - 1;               // below lo_wave for a wave without rows
   const int lo_tile = window > 0 ? max(0, pos_tile - window + 1) : 0;
-  const int hi_tile = pos_tile + min(64, q_len - tile_first) - 1;
+  const int hi_tile = pos_tile + min(TILE_ROWS, q_len - tile_first) - 1;
   const float scale_log2 = scale * 1.44269504088896340736f;
   const int64_t page_elems = (int64_t)PAGE_TOKENS * head_dim;
   const int* table = page_table + (int64_t)slot * max_pages;
@@ -351,9 +385,9 @@ __global__ __launch_bounds__(256, (GP * KB <= 8 && KB <= 4) ? (GP == 1 ? 3 : 2) 
   for (int pg = pg_first; pg <= pg_last; ++pg) {
     const int buf = (pg - pg_first) & 1;
     bf16_t* const k_lds = smem + buf * k_elems;
-    // With one head per wave the values have one buffer only: three workgroups then fit a compute unit, and
+    // With one unit per wave the values have one buffer only: three workgroups then fit a compute unit, and
     // the third wave per SIMD covers more of the latency than the second barrier per page costs.
-    constexpr bool V_DOUBLE = GP != 1;
+    constexpr bool V_DOUBLE = U != 1;
     bf16_t* const v_lds = smem + 2 * k_elems + (V_DOUBLE ? buf * v_elems : 0);
     if (page >= 0) {
       stage_store_k<KB>(stage, k_lds, head_dim);
@@ -368,38 +402,40 @@ __global__ __launch_bounds__(256, (GP * KB <= 8 && KB <= 4) ? (GP == 1 ? 3 : 2) 
                      v_pages + ((int64_t)page * n_kv + kvh) * page_elems, head_dim);
     const int key0 = pg * PAGE_TOKENS;
     const bool sees = page_now >= 0 && key0 <= hi_wave && key0 + PAGE_TOKENS > lo_wave;   // some row sees some key
-    bf16x8 p[GP][2];
+    bf16x8 p[U][2];
     if (sees) {
-      // every key of the page is seen by every row of the wave unless the page reaches past the wave's first row,
-      // starts before a window's edge, or the wave has fewer than 16 rows
-      const bool masked = key0 + PAGE_TOKENS - 1 > pos0 || rows < 16 ||
-                          (window > 0 && key0 < pos0 + 15 - window + 1);
-      // Every piece of a page is read from LDS once and used at once for each of the wave's heads, so that no
+      // Every piece of a page is read from LDS once and used at once for each of the wave's units, so that no
       // whole page of operands has to sit in registers.
-      float alpha[GP];
-      bool moved[GP];
-      f32x4 s[GP][4];
+      float alpha[U];
+      bool moved[U];
+      f32x4 s[U][4];
 #pragma unroll
       for (int t = 0; t < 4; ++t) {
 #pragma unroll
-        for (int hh = 0; hh < GP; ++hh) s[hh][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int u = 0; u < U; ++u) s[u][t] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int kb = 0; kb < KB; ++kb) {
           const int d = FULL ? 32 * kb + 8 * g : min(32 * kb + 8 * g, head_dim - 8);
           const bf16x8 a = load8(k_lds + (16 * t + c) * (head_dim + K_PAD) + d);
 #pragma unroll
-          for (int hh = 0; hh < GP; ++hh) s[hh][t] = MFMA16(a, st[hh].q[kb], s[hh][t]);
+          for (int u = 0; u < U; ++u) s[u][t] = MFMA16(a, st[u].q[kb], s[u][t]);
         }
       }
 #pragma unroll
-      for (int hh = 0; hh < GP; ++hh)
-        alpha[hh] = masked ? page_softmax<KB, true>(st[hh], s[hh], p[hh], scale_log2, key0, lo_row, pos_row, moved[hh])
-                           : page_softmax<KB, false>(st[hh], s[hh], p[hh], scale_log2, key0, lo_row, pos_row, moved[hh]);
+      for (int u = 0; u < U; ++u) {
+        const int rt = u / GP;
+        // every key of the page is seen by every row of the tile unless the page reaches past the tile's first
+        // row, starts before a window's edge, or the tile has fewer than 16 rows
+        const bool masked = key0 + PAGE_TOKENS - 1 > pos0[rt] || rows[rt] < 16 ||
+                            (window > 0 && key0 < pos0[rt] + 15 - window + 1);
+        alpha[u] = masked ? page_softmax<KB, true>(st[u], s[u], p[u], scale_log2, key0, lo_row[rt], pos_row[rt], moved[u])
+                          : page_softmax<KB, false>(st[u], s[u], p[u], scale_log2, key0, lo_row[rt], pos_row[rt], moved[u]);
+      }
 #pragma unroll
-      for (int hh = 0; hh < GP; ++hh)
-        if (moved[hh]) {                                      // rare once the maxima have settled
+      for (int u = 0; u < U; ++u)
+        if (moved[u]) {                                       // rare once the maxima have settled
 #pragma unroll
-          for (int dt = 0; dt < 2 * KB; ++dt) st[hh].o[dt] *= alpha[hh];
+          for (int dt = 0; dt < 2 * KB; ++dt) st[u].o[dt] *= alpha[u];
         }
     }
     if (!V_DOUBLE) __syncthreads();                          // the values are in LDS
@@ -411,24 +447,23 @@ __global__ __launch_bounds__(256, (GP * KB <= 8 && KB <= 4) ? (GP == 1 ? 3 : 2) 
           const int d = FULL ? 16 * dt + c : min(16 * dt + c, head_dim - 1);
           const bf16x8 a = load8(v_lds + d * (PAGE_TOKENS + V_PAD) + 32 * h + 8 * g);
 #pragma unroll
-          for (int hh = 0; hh < GP; ++hh) st[hh].o[dt] = MFMA16(a, p[hh][h], st[hh].o[dt]);
+          for (int u = 0; u < U; ++u) st[u].o[dt] = MFMA16(a, p[u][h], st[u].o[dt]);
         }
     }
   }
-  float row_l[GP];
+  float row_l[U];
 #pragma unroll
-  for (int hh = 0; hh < GP; ++hh) row_l[hh] = row_sum<KB>(st[hh]);
-  if (row_valid) {
+  for (int u = 0; u < U; ++u) row_l[u] = row_sum<KB>(st[u]);
 #pragma unroll
-    for (int hh = 0; hh < GP; ++hh) {
-      const float inv = 1.f / row_l[hh];
-      bf16_t* o = out + (row * n_heads + head0 + hh) * head_dim;
+  for (int u = 0; u < U; ++u) {
+    if (!row_valid[u / GP]) continue;
+    const float inv = 1.f / row_l[u];
+    bf16_t* o = out + (row[u / GP] * n_heads + head0 + u % GP) * head_dim;
 #pragma unroll
-      for (int dt = 0; dt < 2 * KB; ++dt) {
-        if (FULL || 16 * dt < head_dim) {
+    for (int dt = 0; dt < 2 * KB; ++dt) {
+      if (FULL || 16 * dt < head_dim) {
 #pragma unroll
-          for (int i = 0; i < 4; ++i) o[16 * dt + 4 * g + i] = float_to_bf16(st[hh].o[dt][i] * inv);
-        }
+        for (int i = 0; i < 4; ++i) o[16 * dt + 4 * g + i] = float_to_bf16(st[u].o[dt][i] * inv);
       }
     }
   }
@@ -748,19 +783,20 @@ static int head_shape_ok(int n_heads, int n_kv, int head_dim) {
   return head_dim > 0 && head_dim % 16 == 0 && head_dim <= 256 && n_kv > 0 && n_heads % n_kv == 0;
 }
 
-template <int GP>
+template <int GP, int RP>
 static int launch_causal(const void* q, const void* k_pages, const void* v_pages, const int* page_table, int max_pages,
                          const int* seq_slot, const int* cu_rows, const int* tile_cu, const int* seq_start, int n_seqs,
                          int max_tiles, void* out, int n_heads, int n_kv, int head_dim, float scale, int window,
                          hipStream_t stream) {
   dim3 grid((max_tiles + 1) / 2, n_heads / GP), block(256);
-  if (GP == 1) grid = dim3(n_heads, max_tiles);
+  // tiles of 64 * RP rows: at most one more than half the 64-row tiles for every sequence
+  if (GP == 1) grid = dim3(n_heads, RP == 1 ? max_tiles : (max_tiles + n_seqs + 1) / 2);
   if (grid.y > 65535) return -1;
-  // two pages of keys [64][D+8] and two of values [D][64+8] (one with one head per wave)
-  const size_t lds = (2 * (size_t)PAGE_TOKENS * (head_dim + K_PAD) + (GP == 1 ? 1 : 2) * (size_t)head_dim * (PAGE_TOKENS + V_PAD)) * 2;
+  // two pages of keys [64][D+8] and two of values [D][64+8] (one with one unit per wave)
+  const size_t lds = (2 * (size_t)PAGE_TOKENS * (head_dim + K_PAD) + (GP * RP == 1 ? 1 : 2) * (size_t)head_dim * (PAGE_TOKENS + V_PAD)) * 2;
 #define LAUNCH_CAUSAL(FULLV)                                                                                       \
   {                                                                                                                \
-    auto kernel = attn_causal_kernel<KB, FULLV, GP>;                                                               \
+    auto kernel = attn_causal_kernel<KB, FULLV, GP, RP>;                                                           \
     if (lds > 64 * 1024 &&                                                                                          \
         hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) \
       return -1;                                                                                                   \
@@ -777,23 +813,32 @@ static int launch_causal(const void* q, const void* k_pages, const void* v_pages
   return DRYFT_LAUNCH_CHECK();
 }
 
+// mode: 0 = chosen here; 1 = one head and 16 rows per wave; 2 = two heads of a kv group per wave (even groups,
+// head_dim <= 128); 3 = one head and 32 rows per wave (head_dim <= 128)
 DRYFT_API int dryft_attn_causal_bf16(const void* q, const void* k_pages, const void* v_pages, const int* page_table,
                                      int max_pages, const int* seq_slot, const int* cu_rows, const int* tile_cu,
                                      const int* seq_start, int n_seqs, int max_tiles, void* out, int n_heads,
-                                     int n_kv, int head_dim, float scale, int window, hipStream_t stream) {
+                                     int n_kv, int head_dim, float scale, int window, int mode, hipStream_t stream) {
   if (n_seqs <= 0 || max_tiles <= 0) return 0;
   if (!head_shape_ok(n_heads, n_kv, head_dim)) return -1;
   const int group = n_heads / n_kv;
-  // Two heads of one kv group can be served by one wave: every piece of a page is then read from LDS once for
-  // both, and LDS reads are what the kernel waits for most. It halves the number of workgroups, so it pays once
-  // there are still two for every compute unit (measured: 0.64 against 0.47 PFLOP/s at 4,096 positions of
-  // Qwen3-4B's heads, 0.81 against 0.62 at 30,000; at 2,048 positions one head per wave is faster).
-  const int pairs = (max_tiles + 1) / 2;
-  if (group % 2 == 0 && head_dim <= 128 && (int64_t)pairs * (n_heads / 2) >= 512)
-    return launch_causal<2>(q, k_pages, v_pages, page_table, max_pages, seq_slot, cu_rows, tile_cu, seq_start, n_seqs,
-                            max_tiles, out, n_heads, n_kv, head_dim, scale, window, stream);
-  return launch_causal<1>(q, k_pages, v_pages, page_table, max_pages, seq_slot, cu_rows, tile_cu, seq_start, n_seqs,
-                          max_tiles, out, n_heads, n_kv, head_dim, scale, window, stream);
+  if (mode < 0 || mode > 3 || (mode == 2 && (group % 2 || head_dim > 128)) || (mode == 3 && head_dim > 128)) return -1;
+  if (mode == 0) {
+    // Two units per wave (twice the rows of one head, or two heads of a kv group) use every piece of a page that
+    // is read from LDS twice, and LDS reads are what the kernel waits for most; they also halve the number of
+    // workgroups, so they pay once there are still four for every compute unit. Measured on Qwen3-4B's heads,
+    // one sequence, PFLOP/s with 16 rows / 32 rows / two heads per wave: 0.46 / 0.40 / 0.34 at 2,048 positions,
+    // 0.55 / 0.53 / 0.45 at 3,000, 0.59 / 0.72 / 0.62 at 4,096, 0.63 / 0.77 / 0.69 at 8,192, 0.71 / 0.92 / 0.78 at
+    // 30,000. (Two heads per wave stay available as mode 2; nothing chooses them.)
+    mode = head_dim <= 128 && (int64_t)((max_tiles + 1) / 2) * n_heads >= 1024 ? 3 : 1;
+  }
+#define CAUSAL(GPV, RPV)                                                                                          \
+  return launch_causal<GPV, RPV>(q, k_pages, v_pages, page_table, max_pages, seq_slot, cu_rows, tile_cu, seq_start, \
+                                 n_seqs, max_tiles, out, n_heads, n_kv, head_dim, scale, window, stream)
+  if (mode == 2) CAUSAL(2, 1);
+  if (mode == 3) CAUSAL(1, 2);
+  CAUSAL(1, 1);
+#undef CAUSAL
 }
 
 static int launch_split(const void* q, const void* k_pages, const void* v_pages, const int* page_table, int max_pages,

@@ -26,7 +26,7 @@ _SIGNATURES = {
     "rope_kv": {"dryft_qk_norm_rope_kv": [_P, _L, _P, _P, _I, _I, _F, _P, _P, _I, _P, _P, _P, _P, _P, _P, _I, _I,
                                           _I, _I, _I, _I, _I, _P]},
     "attn_rows": {"dryft_attn_rows": [_P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _F, _I, _I, _P]},
-    "attn_mfma": {"dryft_attn_causal_bf16": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _P, _I, _I, _I, _F, _I, _P],
+    "attn_mfma": {"dryft_attn_causal_bf16": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _P, _I, _I, _I, _F, _I, _I, _P],
                   "dryft_attn_split_bf16": [_P, _P, _P, _P, _I, _P, _P, _P, _I, _P, _P, _I, _P, _I, _I, _I, _F, _I,
                                             _P],
                   "dryft_attn_decode_fused_bf16": [_P, _L, _P, _P, _I, _I, _F, _P, _P, _I, _I, _P, _P, _P, _I, _P, _P,
@@ -250,7 +250,10 @@ def attn_rows(q, k_pages, v_pages, page_table, row_slot, row_pos, out, n_heads: 
 
 
 def attn_causal_bf16(q, k_pages, v_pages, page_table, seq_slot, cu_rows, tile_cu, seq_start, n_seqs: int,
-                     max_tiles: int, out, n_heads: int, n_kv: int, head_dim: int, scale: float, window: int) -> None:
+                     max_tiles: int, out, n_heads: int, n_kv: int, head_dim: int, scale: float, window: int,
+                     mode: int = 0) -> None:
+    """Causal attention of steps with many rows per sequence. ``mode``: 0 lets the library choose how much a wave
+    takes; 1 = one head and 16 rows, 2 = two heads of a kv group, 3 = one head and 32 rows."""
     _gpu(q, "q", torch.bfloat16)
     _gpu(out, "out", torch.bfloat16)
     _require(q.is_contiguous() and out.is_contiguous() and out.numel() == q.numel(), "attn_causal: q and out contiguous")
@@ -263,7 +266,7 @@ def attn_causal_bf16(q, k_pages, v_pages, page_table, seq_slot, cu_rows, tile_cu
     _check(_fn("attn_mfma", "dryft_attn_causal_bf16")(
         _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(page_table), page_table.shape[1], _ptr(seq_slot), _ptr(cu_rows),
         _ptr(tile_cu), _ptr(seq_start), n_seqs, max_tiles, _ptr(out), n_heads, n_kv, head_dim, float(scale),
-        int(window), _stream()), "attn_causal_bf16")
+        int(window), int(mode), _stream()), "attn_causal_bf16")
 
 
 def attn_split_bf16(q, k_pages, v_pages, page_table, seq_slot, cu_rows, kv_len, n_seqs: int, part_o, part_ml,

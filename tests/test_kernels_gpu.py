@@ -285,11 +285,11 @@ def run_attention_case(kind, dtype, n_heads, n_kv, D, lengths, tq, window=None, 
                 return view
             kp, vp = shifted(kp), shifted(vp)
         o.attn_rows(d(q_packed), kp, vp, d(table), d(row_slot), d(row_pos), out, n_heads, n_kv, D, scale, w)
-    elif kind == "causal":
+    elif str(kind).startswith("causal"):                     # "causal2": with the kernel's mode 2
         o.attn_causal_bf16(d(q_packed), d(k_pages), d(v_pages), d(table), d(torch.tensor(slots, dtype=torch.int32)),
                            d(torch.from_numpy(cu)), d(torch.from_numpy(tiles)),
                            d(torch.tensor([n - ql for n, ql in zip(lengths, q_lens)], dtype=torch.int32)), B,
-                           int(tiles[-1]) + 1, out, n_heads, n_kv, D, scale, w)
+                           int(tiles[-1]) + 1, out, n_heads, n_kv, D, scale, w, int(str(kind)[6:] or 0))
     else:
         splits = kind
         part_o = torch.empty(B * n_heads * splits * D, dtype=torch.float32, device=DEV)
@@ -313,9 +313,20 @@ def test_attn_rows_takes_pages_at_any_address(dtype):
     run_attention_case("rows", dtype, 8, 2, 32, [200, 70, 130], 200, window=70, misaligned=True)
 
 
-@pytest.mark.parametrize("case", CASES)
-def test_attn_causal_bf16(case):
-    run_attention_case("causal", torch.bfloat16, *case)
+CAUSAL_CASES = CASES + [      # many rows: several tiles per sequence, sequences that end inside a tile
+    (8, 2, 64, [300, 129, 70, 500], 500),
+    (32, 8, 128, [260], 260),
+    (32, 8, 128, [700, 330], 290),      # rows that continue after 410 and 40 cached tokens
+    (9, 3, 32, [200, 150, 1, 65], 200),   # three heads to a kv head: no pairs of heads
+]
+
+
+@pytest.mark.parametrize("mode", [0, 1, 2, 3])      # chosen by the kernel; 16 rows; two heads; 32 rows a wave
+@pytest.mark.parametrize("case", CAUSAL_CASES)
+def test_attn_causal_bf16(case, mode):
+    if mode == 2 and (case[0] // case[1]) % 2:
+        pytest.skip("two heads per wave need an even number of heads per kv head")
+    run_attention_case(f"causal{mode}", torch.bfloat16, *case)
 
 
 @pytest.mark.parametrize("splits", [1, 2, 5, 32])
@@ -374,7 +385,7 @@ def test_attn_decode_fused_equals_the_two_kernels(n_heads, n_kv, D, splits, wind
     assert torch.equal(k3, k1) and torch.equal(v3, v1) and torch.equal(out3, out2)
 
 
-@pytest.mark.parametrize("kind", ["rows", "causal", 3])
+@pytest.mark.parametrize("kind", ["rows", "causal1", "causal2", "causal3", 3])
 def test_attention_window(kind):
     tq = 1 if kind == 3 else 90
     run_attention_case(kind, torch.bfloat16, 8, 2, 32, [200, 70, 130], tq, window=70)
