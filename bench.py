@@ -28,27 +28,14 @@ PEAK_FLOPS = {"bf16": 2.5e15, "fp16": 2.5e15, "fp8": 5.0e15, "fp32": 157.3e12}
 PROMPT, SLOT = 2048, 4096
 
 
-def matmul_params(cfg) -> tuple[int, int]:
-    """(weights of one layer's matrix products, weights of the output head)."""
-    per_layer = (cfg.q_dim + 2 * cfg.kv_dim) * cfg.hidden_size + cfg.hidden_size * cfg.q_dim \
-        + 3 * cfg.intermediate_size * cfg.hidden_size
-    return per_layer, cfg.vocab_size * cfg.hidden_size
-
-
-def decode_bytes(cfg, layers: int, batch: int, context: float, elem: int = 2) -> float:
+def decode_bytes(engine, batch: int, context: float) -> float:
     """What a decode step has to read: every weight it uses once, and the cache of the live requests."""
-    per_layer, head = matmul_params(cfg)
-    norms = layers * (2 * cfg.hidden_size + 2 * cfg.head_dim) + cfg.hidden_size
-    weights = (layers * per_layer + head + norms) * elem
-    kv = batch * context * layers * 2 * cfg.kv_dim * elem
-    return weights + kv
+    return engine.model.streamed_weight_bytes() + batch * engine.cache.bytes_read(context)
 
 
-def prefill_flops(cfg, layers: int, tokens: int) -> float:
-    per_layer, head = matmul_params(cfg)
-    linear = 2.0 * tokens * layers * per_layer + 2.0 * head          # the head runs on the last row only
-    attention = layers * 2.0 * tokens * tokens * cfg.q_dim            # QK^T and PV, causal half of each
-    return linear + attention
+def prefill_flops(engine, tokens: int) -> float:
+    """One prompt of `tokens` tokens whose logits are wanted at its last position."""
+    return engine.model.step_flops([(0, tokens)], 1)
 
 
 def main() -> int:
@@ -75,29 +62,30 @@ def main() -> int:
     import numpy as np
     import torch
 
+    from dataclasses import asdict
+
     from dryft_amd import Engine
-    from dryft_amd.models.qwen3 import load_preset
+    from dryft_amd.models import load_preset
 
     raw = dict(load_preset(args.preset))
     full_layers = raw["num_hidden_layers"]
     if args.layers:
         raw["num_hidden_layers"] = args.layers
-    layers = raw["num_hidden_layers"]
     max_batch = args.batch if args.no_points else max(args.batch, 64)
     engine = Engine(config=raw, seed=args.seed, dtype=args.dtype, max_batch=max_batch, max_len=SLOT,
                     use_graph=not args.no_graph, verbose=True)
     cfg = engine.config
+    vocab = engine.model.plan.vocab_size
     if not args.no_tune and args.dtype == "bfloat16":
         t0 = time.perf_counter()
         rows = sorted({PROMPT, args.batch, args.batch * PROMPT} | (set() if args.no_points else {64}))
         engine.tune(rows)                                               # outside every timed region
         print(f"[bench] vendor library tuned for steps of {rows} rows in {time.perf_counter() - t0:.1f}s",
               file=sys.stderr, flush=True)
-    elem = 2 if args.dtype == "bfloat16" else 4
     rng = np.random.default_rng(args.seed)
 
     def prompts(b):
-        return [[int(t) for t in rng.integers(0, cfg.vocab_size, size=PROMPT)] for _ in range(b)]
+        return [[int(t) for t in rng.integers(0, vocab, size=PROMPT)] for _ in range(b)]
 
     def sync():
         torch.cuda.synchronize()
@@ -137,32 +125,30 @@ def main() -> int:
     tok_s = ms_step = achieved = pf_tok_s = pf_ms = pf_frac = 0.0
     if args.phase in ("all", "decode"):
         tok_s, ms_step, context = decode_rate(args.batch, args.steps, args.warmup)
-        need = decode_bytes(cfg, layers, args.batch, context, elem)
+        need = decode_bytes(engine, args.batch, context)
         achieved = need / (ms_step * 1e-3) / 1e9
     if args.phase in ("all", "prefill"):
         pf_tok_s, pf_ms = prefill_rate()
         peak = PEAK_FLOPS["bf16" if args.dtype == "bfloat16" else "fp32"]
-        pf_frac = prefill_flops(cfg, layers, PROMPT) / (pf_ms * 1e-3) / peak
+        pf_frac = prefill_flops(engine, PROMPT) / (pf_ms * 1e-3) / peak
     points, points_frac = {}, {}
     if not args.no_points and args.phase == "all":
         for b in (1, 64):
             rate, ms, ctx = decode_rate(b, max(16, args.steps // 2), max(4, args.warmup // 2))
             points[f"decode_b{b}"] = round(rate, 1)
             # the same roofline as the main batch: bytes the step has to read / its time / the HBM peak
-            points_frac[f"decode_b{b}"] = round(decode_bytes(cfg, layers, b, ctx, elem) / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
+            points_frac[f"decode_b{b}"] = round(decode_bytes(engine, b, ctx) / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
     line = {
         "metric": f"decode tok/s ({args.preset} layer sizes, 2,048-token prompts, 4,096-token slots)",
         "value": round(tok_s, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic (random weights, uniform random token ids)",
+        # every size of the typed configuration under its config.json name (the layers are those that ran), flat
         "config": {
             "model": args.preset, "global_batch": args.batch, "seq_len": SLOT, "prompt_len": PROMPT,
-            "parallelism": "none", "layers": layers, "layers_of_model": full_layers, "hidden_size": cfg.hidden_size,
-            "num_attention_heads": cfg.num_attention_heads, "num_key_value_heads": cfg.num_key_value_heads,
-            "head_dim": cfg.head_dim, "intermediate_size": cfg.intermediate_size, "vocab_size": cfg.vocab_size,
-            "rope_theta": cfg.rope_theta, "rms_norm_eps": cfg.rms_norm_eps,
-            "tie_word_embeddings": cfg.tie_word_embeddings, "graph": not args.no_graph,
+            "parallelism": "none", "layers_of_model": full_layers, "graph": not args.no_graph,
             "library_tuned": not args.no_tune,
+            **{k: v for k, v in asdict(cfg).items() if isinstance(v, (bool, int, float, str))},
         },
         "prefill": {"value": round(pf_tok_s, 1), "tokens": PROMPT, "ms": round(pf_ms, 3), "frac": round(pf_frac, 4)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",

@@ -190,5 +190,16 @@ class CacheStore:
     def bytes(self) -> int:
         return sum(g.bytes() for g in self.kv_groups) + sum(g.bytes() for g in self.state_groups)
 
+    def bytes_read(self, context: float) -> float:
+        """What one more token of a sequence ``context`` tokens long reads from the cache: the keys and values it
+        sees on every line, and its fixed-size state."""
+        total = 0.0
+        for g in self.kv_groups:
+            seen = min(context, g.need.window) if g.need.window else context
+            total += 2.0 * len(g.lines) * g.need.num_kv_heads * g.need.head_dim * g.k.element_size() * seen
+        for g in self.state_groups:
+            total += g.bytes() / self.n_slots
+        return total
+
     def lengths_host(self) -> np.ndarray:
         return self.slots.lengths.copy()

@@ -10,6 +10,7 @@ agent/bench.py:180-192).
     python -m dryft_amd bench --preset qwen3-4b --workload b8,8,2048,64
     python -m dryft_amd profile --preset qwen3-4b --batch 8 --prompt-len 2048 --steps 8
     python -m dryft_amd replay --model DIR --dtype float32 --out DIR --max-tokens 4096 < steps.jsonl
+    python -m dryft_amd build [names...]
 """
 
 from __future__ import annotations
@@ -30,14 +31,16 @@ def _add_model_options(ap: argparse.ArgumentParser) -> None:
     ap.add_argument("--tiny", action="store_true", help="same as --preset tiny-a")
     ap.add_argument("--weight-seed", type=int, default=0, help="seed of the random weights")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32", "bfloat16", "float32"])
-    ap.add_argument("--max-len", type=int, default=4096, help="longest sequence a cache slot can hold")
+    ap.add_argument("--max-len", type=int, default=None,
+                    help="longest sequence a cache slot can hold (default: what the command needs, or 8,192 where it "
+                         "cannot know, bounded by what the model allows)")
     ap.add_argument("--max-batch", type=int, default=None, help="cache slots (default: the number of prompts)")
     ap.add_argument("--no-graph", action="store_true", help="run decoding steps without graph capture")
 
 
 def _engine(args, max_batch: int, max_tokens: int | None = None):
     from . import Engine
-    from .models.qwen3 import load_preset
+    from .models import load_preset
 
     kw = dict(dtype=args.dtype, max_batch=args.max_batch or max_batch, max_len=args.max_len, max_tokens=max_tokens,
               use_graph=not args.no_graph, verbose=True)
@@ -64,7 +67,7 @@ def _prompts(args, vocab: int) -> list[list[int]]:
 def cmd_generate(args) -> int:
     n = len(args.prompt_ids.split(";")) if args.prompt_ids else (len(args.random_prompts.split(",")) if args.random_prompts else 8)
     engine = _engine(args, max(1, n))
-    prompts = _prompts(args, engine.config.vocab_size)
+    prompts = _prompts(args, engine.model.plan.vocab_size)
     stops = [int(t) for t in args.stop_ids.split(",")] if args.stop_ids else []
     columns: list[list[int]] = [[] for _ in prompts]
     for step in engine.generate(prompts, args.max_new_tokens, temperature=args.temperature,
@@ -85,7 +88,7 @@ def cmd_make_model(args) -> int:
 
     from .engine.model import DecoderModel
     from .models import resolve_architecture
-    from .models.qwen3 import load_preset
+    from .models import load_preset
     from .weights import random_tensors, write_model_dir
 
     if args.config:
@@ -101,6 +104,16 @@ def cmd_make_model(args) -> int:
     return 0
 
 
+def cmd_build(args) -> int:
+    """Compile the kernel libraries for gfx950 (all of them, or the named ones) without running anything."""
+    from .csrc import build
+
+    names = args.names or list(build.MODULES)
+    for name, path in sorted(build.build(names, force=args.force).items()):
+        print(f"{name}: {path}")
+    return 0
+
+
 def cmd_bench(args) -> int:
     """Per workload: one untimed warm-up call, then ``--samples`` timed calls with fresh random prompts
     (agent/bench.py:96-126); reports median tokens/s, time to first token and time per output token."""
@@ -108,13 +121,13 @@ def cmd_bench(args) -> int:
 
     workloads = [w.split(",") for w in (args.workload or ["b1,1,512,32", "b4,4,2048,32", "b16,16,512,128"])]
     workloads = [(n, int(b), int(i), int(o)) for n, b, i, o in workloads]
-    args.max_len = max(args.max_len, max(i + o for _, _, i, o in workloads))
+    args.max_len = max(args.max_len or 0, max(i + o for _, _, i, o in workloads))
     # the cache holds the largest workload, not the largest batch times the longest sequence
     engine = _engine(args, max(b for _, b, _, _ in workloads), max(b * (-(-(i + o) // 64) * 64) for _, b, i, o in workloads))
     if args.tune:
         engine.tune(sorted({b for _, b, _, _ in workloads} | {b * inp for _, b, inp, _ in workloads}))
     rng = random.Random(args.seed)
-    vocab = engine.config.vocab_size
+    vocab = engine.model.plan.vocab_size
     for name, b, inp, out in workloads:
         totals, firsts = [], []
         for sample in range(args.samples + 1):
@@ -147,10 +160,10 @@ def cmd_profile(args) -> int:
     from .engine.step import SeqStep
 
     args.no_graph = True
-    args.max_len = max(args.max_len, args.prompt_len + args.steps + 8)
+    args.max_len = max(args.max_len or 0, args.prompt_len + args.steps + 8)
     engine = _engine(args, args.batch)
     rng = random.Random(args.seed)
-    vocab = engine.config.vocab_size
+    vocab = engine.model.plan.vocab_size
     prompts = [[rng.randrange(vocab) for _ in range(args.prompt_len)] for _ in range(args.batch)]
     slots = engine.acquire(args.batch)
     try:
@@ -190,9 +203,8 @@ def cmd_profile(args) -> int:
     for name, (count, us) in sorted(rows.items(), key=lambda kv: -kv[1][1])[: args.rows]:
         print(f"{name[:72]:72s} {count / steps:10.1f} {us / steps:10.1f} {100 * us / max(total, 1e-9):5.1f}%")
     if not args.prefill and total > 0:
-        cfg = engine.config
-        weights = engine.model.weight_bytes() - (0 if cfg.tie_word_embeddings else cfg.vocab_size * cfg.hidden_size * 2)
-        cache = args.batch * (args.prompt_len + 2 + args.steps / 2) * cfg.num_hidden_layers * 2 * cfg.kv_dim * 2
+        weights = engine.model.streamed_weight_bytes()
+        cache = args.batch * engine.cache.bytes_read(args.prompt_len + 2 + args.steps / 2)
         print(f"implied bandwidth: {(weights + cache) / (total / steps * 1e-6) / 1e9:.0f} GB/s "
               f"(weights read once, cache of the live sequences)")
     return 0
@@ -245,6 +257,11 @@ def main(argv=None) -> int:
     pr.add_argument("--rows", type=int, default=20, help="kernels to list")
     pr.add_argument("--seed", type=int, default=0)
     pr.set_defaults(fn=cmd_profile)
+
+    bd = sub.add_parser("build", help="compile the HIP kernel libraries (needs hipcc, no GPU)")
+    bd.add_argument("names", nargs="*", help="libraries to build (default: all)")
+    bd.add_argument("--force", action="store_true", help="also rebuild what is up to date")
+    bd.set_defaults(fn=cmd_build)
 
     r = sub.add_parser("replay", help="trace replay (same as bin/trace_run)", add_help=False)
     r.set_defaults(fn=None)

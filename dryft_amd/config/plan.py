@@ -55,6 +55,10 @@ class ModelPlan:
     final_norm: PartSpec
     head: PartSpec
     positions: dict[str, PartSpec] = field(default_factory=dict)
+    # Tensors a checkpoint may hold although the model reads them under another name: each maps to the name of
+    # the tensor it has to equal when present (a tied head's copy of the embedding).
+    optional_tensors: dict[str, str] = field(default_factory=dict)
+    max_positions: int | None = None      # longest sequence the architecture allows; None: no bound of its own
 
     def validate(self) -> None:
         problems = []

@@ -15,6 +15,7 @@ from __future__ import annotations
 from dataclasses import asdict, dataclass
 from typing import Any
 
+from ..limits import MAX_HEAD_DIM
 from .base import KeyReader
 
 
@@ -80,6 +81,8 @@ class Qwen3Config:
                     f"num_attention_heads ({heads}) is not a multiple of num_key_value_heads ({kv_heads})")
         if cfg.head_dim:
             r.check(cfg.head_dim % 2 == 0, f"head_dim: must be even for rotary pairs, got {cfg.head_dim}")
+            r.check(cfg.head_dim <= MAX_HEAD_DIM,
+                    f"head_dim: the attention kernels take at most {MAX_HEAD_DIM}, got {cfg.head_dim}")
         r.finish("unsupported or malformed Qwen3 config.json")
         return cfg
 

@@ -306,11 +306,13 @@ __global__ __launch_bounds__(256, (GP * RP * KB <= 8 && KB <= 4) ? (GP * RP == 1
   const int head0 = (PAIRED ? blockIdx.y : blockIdx.x) * GP;
   const int first_tile = PAIRED ? blockIdx.x : blockIdx.y;
   int n_tiles;                                                // tiles of TILE_ROWS rows over all sequences
+  // A sequence that sits out (slot < 0) keeps its rows in cu_rows but has no tiles, here as in tile_cu.
   if (RP == 1) {
     n_tiles = tile_cu[n_seqs];
   } else {
     n_tiles = 0;
-    for (int sq = 0; sq < n_seqs; ++sq) n_tiles += (cu_rows[sq + 1] - cu_rows[sq] + TILE_ROWS - 1) / TILE_ROWS;
+    for (int sq = 0; sq < n_seqs; ++sq)
+      if (seq_slot[sq] >= 0) n_tiles += (cu_rows[sq + 1] - cu_rows[sq] + TILE_ROWS - 1) / TILE_ROWS;
   }
   // A tile late in a sequence sees many keys, an early one few. With pairs every workgroup takes one tile from
   // each end of the list, so all of them have about the same work.
@@ -332,7 +334,7 @@ __global__ __launch_bounds__(256, (GP * RP * KB <= 8 && KB <= 4) ? (GP * RP == 1
     seq = 0;
     tile_in_seq = tile;
     for (;;) {
-      const int cnt = (cu_rows[seq + 1] - cu_rows[seq] + TILE_ROWS - 1) / TILE_ROWS;
+      const int cnt = seq_slot[seq] >= 0 ? (cu_rows[seq + 1] - cu_rows[seq] + TILE_ROWS - 1) / TILE_ROWS : 0;
       if (tile_in_seq < cnt || seq + 1 >= n_seqs) break;
       tile_in_seq -= cnt;
       ++seq;
@@ -557,12 +559,14 @@ struct FusedQKV {
 #define SPLIT_MAX_D 256
 
 template <int KB, bool FULL>
+// The fused form appends the row's key and value through k_pages_w / v_pages_w, which are the same buffers as
+// k_pages / v_pages: none of the four is declared restrict.
 __global__ __launch_bounds__(64 * SPLIT_WAVES, 2) void attn_split_kernel(
-    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
+    const bf16_t* __restrict__ q, const bf16_t* k_pages, const bf16_t* v_pages,
     const int* __restrict__ page_table, int max_pages, const int* __restrict__ seq_slot,
     const int* __restrict__ cu_rows, const int* __restrict__ kv_len, float* __restrict__ part_o,
     float* __restrict__ part_ml, int n_heads, int n_kv, int head_dim, float scale, int window, int n_splits,
-    FusedQKV fused, bf16_t* __restrict__ k_pages_w, bf16_t* __restrict__ v_pages_w, bf16_t* __restrict__ out) {
+    FusedQKV fused, bf16_t* k_pages_w, bf16_t* v_pages_w, bf16_t* __restrict__ out) {
   __shared__ float merge_o[SPLIT_WAVES][16][32 * KB + 1];
   __shared__ float merge_ml[SPLIT_WAVES][16][2];
   __shared__ __attribute__((aligned(16))) bf16_t q_lds[16][32 * KB];
@@ -789,7 +793,8 @@ static int launch_causal(const void* q, const void* k_pages, const void* v_pages
                          int max_tiles, void* out, int n_heads, int n_kv, int head_dim, float scale, int window,
                          hipStream_t stream) {
   dim3 grid((max_tiles + 1) / 2, n_heads / GP), block(256);
-  // tiles of 64 * RP rows: at most one more than half the 64-row tiles for every sequence
+  // max_tiles bounds the 64-row tiles of the sequences that take part. Tiles of 128 rows: a sequence with t
+  // 64-row tiles has (t + 1) / 2 of them, so all together at most (max_tiles + n_seqs) / 2.
   if (GP == 1) grid = dim3(n_heads, RP == 1 ? max_tiles : (max_tiles + n_seqs + 1) / 2);
   if (grid.y > 65535) return -1;
   // two pages of keys [64][D+8] and two of values [D][64+8] (one with one unit per wave)

@@ -6,10 +6,10 @@
 
 // One block. Inputs: seq_slot[B] (-1 = not taking part), q_len[B] (new tokens of
 // each sequence), lengths[slots] (cached tokens per slot). Outputs: cu_rows[B+1],
-// tile_cu[B+1] (prefix sums of rows and of 64-row query tiles), kv_len[B] (cached
+// tile_cu[B+1] (prefix sums of rows and of tiles of `tile_rows` rows), kv_len[B] (cached
 // tokens after this step), row_seq/row_slot/row_pos[n_rows]. Advances lengths.
 __global__ void prepare_batch_kernel(const int* __restrict__ seq_slot, const int* __restrict__ q_len,
-                                     int* __restrict__ lengths, int n_seqs, int n_rows,
+                                     int* __restrict__ lengths, int n_seqs, int n_rows, int tile_rows,
                                      int* __restrict__ cu_rows, int* __restrict__ tile_cu,
                                      int* __restrict__ kv_len, int* __restrict__ seq_start,
                                      int* __restrict__ row_seq, int* __restrict__ row_slot,
@@ -25,7 +25,7 @@ __global__ void prepare_batch_kernel(const int* __restrict__ seq_slot, const int
       seq_start[s] = past;
       kv_len[s] = past + q;
       rows += q_len[s];                         // rows of a sequence that sits out still occupy their places
-      tiles += (q + 63) / 64;
+      tiles += (q + tile_rows - 1) / tile_rows;
       if (slot >= 0) lengths[slot] = past + q;
     }
     cu_rows[n_seqs] = rows;
@@ -48,9 +48,10 @@ __global__ void prepare_batch_kernel(const int* __restrict__ seq_slot, const int
 }
 
 DRYFT_API int dryft_prepare_batch(const int* seq_slot, const int* q_len, int* lengths, int n_seqs, int n_rows,
-                                  int* cu_rows, int* tile_cu, int* kv_len, int* seq_start, int* row_seq,
+                                  int tile_rows, int* cu_rows, int* tile_cu, int* kv_len, int* seq_start, int* row_seq,
                                   int* row_slot, int* row_pos, hipStream_t stream) {
+  if (tile_rows <= 0) return -1;
   hipLaunchKernelGGL(prepare_batch_kernel, dim3(1), dim3(256), 0, stream, seq_slot, q_len, lengths, n_seqs, n_rows,
-                     cu_rows, tile_cu, kv_len, seq_start, row_seq, row_slot, row_pos);
+                     tile_rows, cu_rows, tile_cu, kv_len, seq_start, row_seq, row_slot, row_pos);
   return DRYFT_LAUNCH_CHECK();
 }

@@ -97,8 +97,9 @@ def hipcc_path() -> str | None:
 def _compile(name: str, out_dir: str) -> str:
     hipcc = hipcc_path()
     if hipcc is None:
-        raise ExtensionError(f"kernel library {name!r} is not built and hipcc was not found; "
-                             f"run `python -c 'import __graft_entry__ as g; g.build()'` where ROCm is installed")
+        raise ExtensionError(f"kernel library {name!r} is not built and hipcc was not found; build it where ROCm is "
+                             f"installed with `python -m dryft_amd build` (hipcc {' '.join(HIPCC_FLAGS)} "
+                             f"{name}.hip -o {_lib_name(name)})")
     so = os.path.join(out_dir, _lib_name(name))
     tmp = so + f".tmp{os.getpid()}"
     cmd = [hipcc] + HIPCC_FLAGS + [os.path.join(_HERE, name + ".hip"), "-o", tmp]

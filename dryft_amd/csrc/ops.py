@@ -18,7 +18,7 @@ from . import build
 
 _P, _I, _L, _F = c_void_p, c_int, c_int64, c_float
 _SIGNATURES = {
-    "batch": {"dryft_prepare_batch": [_P, _P, _P, _I, _I, _P, _P, _P, _P, _P, _P, _P, _P]},
+    "batch": {"dryft_prepare_batch": [_P, _P, _P, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _P]},
     "embed": {"dryft_embed_rows": [_P, _P, _P, _I, _I, _I, _I, _P]},
     "norm": {"dryft_add_rmsnorm": [_P, _P, _I, _I, _L, _P, _I, _P, _P, _I, _I, _F, _I, _P],
              "dryft_add_rows": [_P, _P, _P, _L, _I, _P]},
@@ -97,6 +97,14 @@ def _ptr(t) -> int:
 
 
 # ------------------------------------------------------------------------------------------- batch
+ROW_TILE = 64      # rows of a sequence that one workgroup of the prompt-attention kernel takes (its smallest tile)
+
+
+def row_tiles(q_len: int) -> int:
+    """Tiles of ``ROW_TILE`` rows that a sequence bringing ``q_len`` rows occupies."""
+    return (q_len + ROW_TILE - 1) // ROW_TILE
+
+
 def prepare_batch(seq_slot, q_len, lengths, n_seqs: int, n_rows: int, cu_rows, tile_cu, kv_len, seq_start,
                   row_seq, row_slot, row_pos) -> None:
     for name, t, n in (("seq_slot", seq_slot, n_seqs), ("q_len", q_len, n_seqs), ("cu_rows", cu_rows, n_seqs + 1),
@@ -106,7 +114,7 @@ def prepare_batch(seq_slot, q_len, lengths, n_seqs: int, n_rows: int, cu_rows, t
         _gpu(t, name, torch.int32)
         _require(t.is_contiguous() and t.numel() >= n, f"{name}: needs {n} contiguous entries, has {t.numel()}")
     _check(_fn("batch", "dryft_prepare_batch")(
-        _ptr(seq_slot), _ptr(q_len), _ptr(lengths), n_seqs, n_rows, _ptr(cu_rows), _ptr(tile_cu), _ptr(kv_len),
+        _ptr(seq_slot), _ptr(q_len), _ptr(lengths), n_seqs, n_rows, ROW_TILE, _ptr(cu_rows), _ptr(tile_cu), _ptr(kv_len),
         _ptr(seq_start), _ptr(row_seq), _ptr(row_slot), _ptr(row_pos), _stream()), "prepare_batch")
 
 

@@ -18,6 +18,7 @@ from typing import Any, Iterator, Sequence
 
 import torch
 
+from ..cache.spec import PAGE_TOKENS, pages_for
 from ..cache.store import CacheStore
 from ..config.base import read_config_json
 from ..models import resolve_architecture
@@ -29,6 +30,7 @@ from .graph import DecodeGraph
 from .model import DecoderModel
 from .step import SeqStep, Stepper
 
+DEFAULT_MAX_LEN = 8192
 DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32}
 
 
@@ -57,7 +59,7 @@ class PendingStep:
 class Engine:
     def __init__(self, model_path: str | None = None, *, config: dict[str, Any] | None = None,
                  seed: int | None = None, norm_std: float = 0.0, dtype: str = "bfloat16", max_batch: int = 32,
-                 max_len: int = 8192, max_tokens: int | None = None, use_graph: bool = True,
+                 max_len: int | None = None, max_tokens: int | None = None, use_graph: bool = True,
                  device: str = "cuda:0", verbose: bool = False):
         t0 = time.time()
         self.device = require_gpu(device)
@@ -80,8 +82,15 @@ class Engine:
             tensors = random_tensors(specs, seed, self.dtype, norm_std=norm_std, device=self.device)
         self.model.load(tensors)
         del tensors
+        # The longest sequence a slot holds: what is asked for, bounded by what the architecture allows (the reference
+        # reads max_position_embeddings as that bound, engine/dryft_qwen3/config.py:154). Asking for more is an error.
+        limit = self.model.plan.max_positions
+        if max_len is None:
+            max_len = min(DEFAULT_MAX_LEN, limit) if limit else DEFAULT_MAX_LEN
+        if limit and max_len > limit:
+            raise ValueError(f"max_len {max_len} exceeds the {limit} positions this model allows")
         self.max_batch, self.max_len = int(max_batch), int(max_len)
-        per_seq = -(-self.max_len // 64) * 64
+        per_seq = pages_for(self.max_len) * PAGE_TOKENS
         self.max_tokens = int(max_tokens) if max_tokens is not None else self.max_batch * per_seq
         self.cache = CacheStore(self.model.cache_needs(), max_tokens=self.max_tokens, n_slots=self.max_batch,
                                 max_len=self.max_len, dtype=self.dtype, device=self.device)
@@ -110,7 +119,7 @@ class Engine:
             for rows in row_counts:
                 rows = int(rows)
                 n_seqs = max(1, -(-rows // self.max_len))
-                if rows <= 0 or n_seqs > self.max_batch or -(-rows // 64) * 64 + 64 * n_seqs > self.max_tokens:
+                if rows <= 0 or n_seqs > self.max_batch or (pages_for(rows) + n_seqs) * PAGE_TOKENS > self.max_tokens:
                     raise ValueError(f"a step of {rows} rows does not fit this engine "
                                      f"({self.max_batch} sequences of {self.max_len}, {self.max_tokens} tokens)")
                 lengths = [rows // n_seqs + (i < rows % n_seqs) for i in range(n_seqs)]
@@ -207,18 +216,14 @@ class Engine:
     # ------------------------------------------------------------------ generation
     def generate(self, input_ids: Sequence[Sequence[int]], max_new_tokens: int, *, temperature: float = 0.0,
                  sample_seed: int = 0, stop_token_ids: Sequence[int] = ()) -> Iterator[list[int]]:
-        """Yields one list of ``len(input_ids)`` token ids per step; ``-1`` marks an ended sequence."""
+        """Yields one list of ``len(input_ids)`` token ids per step as the steps are computed; ``-1`` stands where
+        a sequence has nothing in that step: it has ended, or, when there are more prompts than ``max_batch``, its
+        batch is not the one running (batches run one after another, each yielding its own steps)."""
         prompts = [list(map(int, p)) for p in input_ids]
         if not prompts or max_new_tokens <= 0:
             return
         self._sampler = Sampler(temperature, sample_seed)
-        if len(prompts) <= self.max_batch:
-            yield from loop.generate_batch(self, prompts, max_new_tokens, stop_token_ids)
-            return
-        # more requests than one batch holds: batches run one after another, then the steps are handed out
-        per_request = loop.generate_all(self, prompts, max_new_tokens, stop_token_ids)
-        for t in range(max(len(r) for r in per_request)):
-            yield [r[t] if t < len(r) else loop.FILL for r in per_request]
+        yield from loop.generate_steps(self, prompts, max_new_tokens, stop_token_ids)
 
     def generate_all(self, input_ids: Sequence[Sequence[int]], max_new_tokens: int, *, temperature: float = 0.0,
                      sample_seed: int = 0, stop_token_ids: Sequence[int] = ()) -> list[list[int]]:

@@ -123,14 +123,29 @@ def plan_batches(n_requests: int, max_batch: int) -> list[range]:
     return [range(i, min(n_requests, i + max_batch)) for i in range(0, n_requests, max_batch)]
 
 
+def generate_steps(backend: StepBackend, prompts: list[list[int]], max_new_tokens: int,
+                   stop_token_ids: Sequence[int] = ()) -> Iterator[list[int]]:
+    """Any number of requests, step by step: every yielded list has one place per request; the places of requests
+    whose batch is not the one running hold ``FILL``. With one batch this is ``generate_batch``."""
+    n = len(prompts)
+    for batch in plan_batches(n, backend.max_batch):
+        idx = list(batch)
+        for step in generate_batch(backend, [prompts[i] for i in idx], max_new_tokens, stop_token_ids):
+            if len(idx) == n:
+                yield step
+                continue
+            out = [FILL] * n
+            for i, t in zip(idx, step):
+                out[i] = t
+            yield out
+
+
 def generate_all(backend: StepBackend, prompts: list[list[int]], max_new_tokens: int,
                  stop_token_ids: Sequence[int] = ()) -> list[list[int]]:
     """Any number of requests: per request the tokens it generated (stop token included)."""
     results: list[list[int]] = [[] for _ in prompts]
-    for batch in plan_batches(len(prompts), backend.max_batch):
-        idx = list(batch)
-        for step in generate_batch(backend, [prompts[i] for i in idx], max_new_tokens, stop_token_ids):
-            for i, t in zip(idx, step):
-                if t != FILL:
-                    results[i].append(t)
+    for step in generate_steps(backend, prompts, max_new_tokens, stop_token_ids):
+        for i, t in enumerate(step):
+            if t != FILL:
+                results[i].append(t)
     return results

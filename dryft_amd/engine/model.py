@@ -60,19 +60,17 @@ class DecoderModel:
         return list(specs.values())
 
     def optional_names(self) -> set[str]:
-        """Tensors a checkpoint may hold without the model reading them (a tied head's copy)."""
-        return {"lm_head.weight"} if getattr(self.head, "tied", False) else set()
+        """Tensors a checkpoint may hold without the model reading them (the plan lists them)."""
+        return set(self.plan.optional_tensors)
 
     def load(self, tensors: dict[str, torch.Tensor]) -> None:
+        """Hands every part its tensors. Parts whose plans name the same checkpoint tensor share it."""
+        for extra, same_as in self.plan.optional_tensors.items():
+            if extra in tensors and not torch.equal(tensors[extra], tensors[same_as]):
+                # the reference's check of a tied head's copy (engine/dryft_qwen3/weights.py:86-87)
+                raise ValueError(f"{extra} is present and differs from {same_as}, which the model reads in its place")
         for part, names in self._bindings:
             part.load({logical: tensors[names[logical]] for logical in part.tensor_specs()})
-        if getattr(self.head, "tied", False):
-            extra = tensors.get("lm_head.weight")
-            if extra is not None and not torch.equal(extra, self.embedding.weight):
-                # the reference's check (engine/dryft_qwen3/weights.py:86-87)
-                raise ValueError("lm_head.weight is present and differs from the embedding although "
-                                 "tie_word_embeddings is set")
-            self.head.tie(self.embedding.weight)
 
     def kernel_modules(self) -> list[str]:
         mods = {"batch", "embed"}
@@ -87,6 +85,28 @@ class DecoderModel:
                 if isinstance(v, torch.Tensor) and v.data_ptr() not in seen:
                     seen.add(v.data_ptr())
                     total += v.numel() * v.element_size()
+        return total
+
+    def streamed_weight_bytes(self) -> int:
+        """Bytes of the tensors that every step reads whole, each counted once (the decode roofline's weights)."""
+        seen, total = set(), 0
+        for part, _ in self._bindings:
+            if not part.reads_whole():
+                continue
+            for v in vars(part).values():
+                if isinstance(v, torch.Tensor) and v.data_ptr() not in seen:
+                    seen.add(v.data_ptr())
+                    total += v.numel() * v.element_size()
+        return total
+
+    def step_flops(self, spans: list[tuple[int, int]], logit_rows: int) -> float:
+        """Floating-point operations of a step whose sequences bring ``q`` rows after ``start`` cached ones
+        (``spans`` of ``(start, q)``) and whose logits are wanted at ``logit_rows`` rows."""
+        rows = sum(q for _, q in spans)
+        total = self.head.flops(logit_rows, spans)
+        for run in self.plan.schedule:
+            for part in self.blocks[run.layer].parts().values():
+                total += part.flops(rows, spans)
         return total
 
     # ---- what the model wants from the cache

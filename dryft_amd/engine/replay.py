@@ -29,7 +29,7 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--dtype", required=True, choices=["bfloat16", "float32"])
     ap.add_argument("--out", required=True, help="folder for <step>.f32 files")
     ap.add_argument("--max-tokens", type=int, required=True,
-                    help="most tokens live requests hold at any time, each request rounded up to 64")
+                    help="most tokens live requests hold at any time, each request rounded up to a whole cache page")
     return ap
 
 
@@ -59,12 +59,20 @@ class Replayer:
 
 def main(argv=None) -> int:
     args = build_parser().parse_args(argv)
+    from ..cache.spec import PAGE_TOKENS, pages_for
+    from ..config.base import read_config_json
+    from ..models import resolve_architecture
     from .engine import Engine
 
     os.makedirs(args.out, exist_ok=True)
-    pages = max(1, -(-args.max_tokens // 64))
-    engine = Engine(args.model, dtype=args.dtype, max_batch=min(pages, 4096), max_len=pages * 64,
-                    max_tokens=pages * 64, use_graph=False)
+    # the budget in whole pages; one request may take all of it, up to what the model allows
+    pages = max(1, pages_for(args.max_tokens))
+    raw = read_config_json(args.model)
+    arch = resolve_architecture(raw)
+    limit = arch.plan(arch.config_class.from_dict(raw)).max_positions
+    max_len = min(pages * PAGE_TOKENS, limit) if limit else pages * PAGE_TOKENS
+    engine = Engine(args.model, dtype=args.dtype, max_batch=min(pages, 4096), max_len=max_len,
+                    max_tokens=pages * PAGE_TOKENS, use_graph=False)
     replayer = Replayer(engine)
     for line in sys.stdin:
         line = line.strip()

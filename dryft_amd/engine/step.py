@@ -4,9 +4,11 @@ The reference has two entry points, ``prefill`` for prompts of one length and
 ``decode_step`` for one token per row (engine/dryft_qwen3/model.py:122-128, 190-198), and
 runs unequal prompts as one call per length (engine/engine.py:172-186). Here one function
 serves both: the sequences of a step either all start (their prompts, of any lengths,
-packed into one batch of rows) or all go on by one token. Only the tokens given are
-run; everything earlier comes from the cache. Tokens are always given by the caller,
-never fed back from the model's own choice.
+packed into one batch of rows) or all go on by one token; that is what the generation
+loop and the replay program ask of it. The function itself takes any mixture: a sequence
+may bring a further portion of its prompt, of any length, while others bring one token.
+Only the tokens given are run; everything earlier comes from the cache. Tokens are always
+given by the caller, never fed back from the model's own choice.
 """
 
 from __future__ import annotations
@@ -75,7 +77,7 @@ def stage_batch(cache: CacheStore, buf: BatchBuffers, slots: list[int], q_lens: 
     buf.seq_slot[:n_seqs].copy_(stage[n_rows:n_rows + n_seqs])
     buf.q_len[:n_seqs].copy_(stage[n_rows + n_seqs:])
     ctx = make_context(buf, n_rows, n_seqs, dtype, max_q_len=max(q_lens),
-                       max_tiles=sum((q + 63) // 64 for q in live_q),
+                       max_tiles=sum(ops.row_tiles(q) for q in live_q),
                        max_kv_len=max([st + q for st, q in zip(starts_live, live_q)], default=0),
                        host=HostBatch(list(slots), list(q_lens), starts))
     derive_rows(cache, buf, ctx)

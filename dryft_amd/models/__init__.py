@@ -7,6 +7,8 @@ here it is the only place where a model is chosen.
 
 from __future__ import annotations
 
+import json
+import os
 from dataclasses import dataclass
 from typing import Any, Callable
 
@@ -50,6 +52,23 @@ def resolve_architecture(raw_config: dict[str, Any]) -> Architecture:
         raise ConfigError("config.json", [
             f"architectures: {names[0]!r} is not registered; known: {known_architectures()}"])
     return arch
+
+
+_PRESET_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "presets")
+
+
+def preset_names() -> list[str]:
+    return sorted(f[:-5] for f in os.listdir(_PRESET_DIR) if f.endswith(".json"))
+
+
+def load_preset(name: str) -> dict:
+    """A named ``config.json`` shipped as data: sizes live in the file, not in code, and the file's own
+    ``architectures`` entry says which registered model it is for."""
+    path = os.path.join(_PRESET_DIR, name + ".json")
+    if not os.path.isfile(path):
+        raise KeyError(f"unknown preset {name!r}; known: {preset_names()}")
+    with open(path, "r", encoding="utf-8") as f:
+        return json.load(f)
 
 
 from . import qwen3 as _qwen3  # noqa: E402,F401  (registers Qwen3ForCausalLM)

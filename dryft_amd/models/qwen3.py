@@ -11,9 +11,6 @@ Checkpoint tensor names are those the reference loads (weights.py:81-114).
 
 from __future__ import annotations
 
-import json
-import os
-
 from ..config.plan import LayerSpec, ModelPlan, PartSpec, Run
 from ..config.qwen3 import Qwen3Config
 from . import register_architecture
@@ -47,34 +44,24 @@ def qwen3_plan(cfg: Qwen3Config) -> ModelPlan:
                                  {"weight": p + "post_attention_layernorm.weight"}),
             "ffn": feed_forward,
         }))
-    head_tensors = {} if cfg.tie_word_embeddings else {"weight": "lm_head.weight"}
+    embedding_name, head_name = "model.embed_tokens.weight", "lm_head.weight"
+    tied = cfg.tie_word_embeddings          # the head then reads the embedding's tensor (weights.py:47-49)
     return ModelPlan(
         vocab_size=cfg.vocab_size,
         hidden_size=cfg.hidden_size,
         embedding=PartSpec("token_embedding", dict(vocab_size=cfg.vocab_size, hidden_size=cfg.hidden_size),
-                           {"weight": "model.embed_tokens.weight"}),
+                           {"weight": embedding_name}),
         layers=tuple(layers),
         schedule=tuple(Run(i, i) for i in range(cfg.num_hidden_layers)),
         final_norm=PartSpec("rmsnorm", dict(size=cfg.hidden_size, **norm_args), {"weight": "model.norm.weight"}),
-        head=PartSpec("lm_head", dict(vocab_size=cfg.vocab_size, hidden_size=cfg.hidden_size,
-                                      tied=cfg.tie_word_embeddings), head_tensors),
+        head=PartSpec("lm_head", dict(vocab_size=cfg.vocab_size, hidden_size=cfg.hidden_size),
+                      {"weight": embedding_name if tied else head_name}),
         positions={"rotary": PartSpec("rotary", dict(dim=cfg.head_dim, theta=cfg.rope_theta))},
+        # a tied checkpoint may still carry a copy of the embedding under the head's name; it must equal it
+        # (weights.py:82-88)
+        optional_tensors={head_name: embedding_name} if tied else {},
+        max_positions=cfg.max_position_embeddings,
     )
 
 
 register_architecture(Qwen3Config.architecture, Qwen3Config, qwen3_plan, model_type="qwen3")
-
-_PRESET_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "presets")
-
-
-def preset_names() -> list[str]:
-    return sorted(f[:-5] for f in os.listdir(_PRESET_DIR) if f.endswith(".json"))
-
-
-def load_preset(name: str) -> dict:
-    """A named ``config.json`` shipped as data (sizes live in the file, not in code)."""
-    path = os.path.join(_PRESET_DIR, name + ".json")
-    if not os.path.isfile(path):
-        raise KeyError(f"unknown preset {name!r}; known: {preset_names()}")
-    with open(path, "r", encoding="utf-8") as f:
-        return json.load(f)

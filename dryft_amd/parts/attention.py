@@ -21,6 +21,7 @@ import torch
 from ..cache.spec import KVNeed
 from ..cache.store import KVLine
 from ..csrc import ops
+from ..limits import MATRIX_CORE_HEAD_STEP, MAX_HEAD_DIM
 from ..weights.spec import VECTOR
 from . import register_part
 from .base import Mixer, StepContext, matrix
@@ -36,12 +37,14 @@ class GQAAttention(Mixer):
                  window: int | None = None, scale: float | None = None):
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} query heads cannot share {num_kv_heads} kv heads evenly")
-        if head_dim % 16 or head_dim > 256:
-            raise ValueError(f"head_dim must be a multiple of 16 up to 256, got {head_dim}")
+        if not 0 < head_dim <= MAX_HEAD_DIM:
+            raise ValueError(f"head_dim must lie in 1..{MAX_HEAD_DIM}, got {head_dim}")
         self.hidden, self.n_heads, self.n_kv, self.head_dim = int(hidden_size), int(num_heads), int(num_kv_heads), int(head_dim)
         self.qk_norm_eps = qk_norm_eps
         self.positions = positions
         self.rotary_dim = int(rotary_dim if rotary_dim is not None else head_dim) if positions else 0
+        if self.rotary_dim % 2 or self.rotary_dim > head_dim:
+            raise ValueError(f"the rotated width must be even and at most head_dim ({head_dim}), got {self.rotary_dim}")
         self.window = int(window) if window else None
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(head_dim)   # model.py:65
         self.q_dim, self.kv_dim = self.n_heads * self.head_dim, self.n_kv * self.head_dim
@@ -79,8 +82,14 @@ class GQAAttention(Mixer):
             if ctx.max_kv_len > table.n_positions:
                 raise ValueError(f"position tables cover {table.n_positions} positions, the step reaches {ctx.max_kv_len}")
         window = self.window or 0
-        out = torch.empty((rows, self.n_heads, self.head_dim), dtype=h.dtype, device=h.device)
-        decoding = h.dtype == torch.bfloat16 and ctx.max_q_len == 1
+        # Every kernel leaves the rows of sequences that sit out at zero; the tiled prompt kernel never visits them,
+        # so for it they are cleared beforehand.
+        sitting_out = ctx.host is not None and any(s < 0 for s in ctx.host.slots)
+        make = torch.zeros if sitting_out and ctx.max_q_len > 1 else torch.empty
+        out = make((rows, self.n_heads, self.head_dim), dtype=h.dtype, device=h.device)
+        # bfloat16 on the matrix cores where they take the head size; float32 and the other head sizes on the plain kernel
+        matrix_cores = h.dtype == torch.bfloat16 and self.head_dim % MATRIX_CORE_HEAD_STEP == 0
+        decoding = matrix_cores and ctx.max_q_len == 1
         if decoding:
             splits = self.decode_splits(ctx.n_seqs, ctx.max_kv_len)
             part_o = torch.empty((ctx.n_seqs, self.n_heads, splits, self.head_dim), dtype=torch.float32, device=h.device)
@@ -100,7 +109,7 @@ class GQAAttention(Mixer):
             ops.attn_split_bf16(q, line.k, line.v, line.page_table, ctx.seq_slot, ctx.cu_rows, ctx.kv_len,
                                 ctx.n_seqs, part_o, part_ml, splits, out, self.n_heads, self.n_kv, self.head_dim,
                                 self.scale, window)
-        elif h.dtype == torch.bfloat16:
+        elif matrix_cores:
             ops.attn_causal_bf16(q, line.k, line.v, line.page_table, ctx.seq_slot, ctx.cu_rows, ctx.tile_cu,
                                  ctx.seq_start, ctx.n_seqs, ctx.max_tiles, out, self.n_heads, self.n_kv,
                                  self.head_dim, self.scale, window)
@@ -108,6 +117,18 @@ class GQAAttention(Mixer):
             ops.attn_rows(q, line.k, line.v, line.page_table, ctx.row_slot, ctx.row_pos, out, self.n_heads, self.n_kv,
                           self.head_dim, self.scale, window)
         return linear(out.view(rows, self.q_dim), self.w_o, allow_partials=True)
+
+    def flops(self, rows, spans):
+        """The projections, and both attention products over the keys each row sees."""
+        seen = 0
+        for start, q in spans:
+            first, last = start + 1, start + q                  # keys that the span's first and last row see
+            if self.window:
+                full = max(0, min(last, self.window) - first + 1)          # rows that still see every key
+                seen += (2 * first + full - 1) * full // 2 + (q - full) * self.window
+            else:
+                seen += (first + last) * q // 2
+        return super().flops(rows, spans) + 4.0 * self.q_dim * seen
 
     def decode_splits(self, n_seqs: int, max_kv_len: int) -> int:
         """How many ways each sequence's keys are split: as many as run at the same time, and no more.

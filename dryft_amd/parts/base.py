@@ -32,8 +32,9 @@ class StepContext:
     Rows are the step's tokens, packed sequence after sequence. Row ``r`` belongs to
     sequence ``row_seq[r]`` in cache slot ``row_slot[r]`` (-1: takes no part) at
     position ``row_pos[r]``. ``cu_rows``/``tile_cu`` are prefix sums over sequences of
-    rows and of 64-row tiles; ``kv_len`` is each sequence's cached length after this
-    step, ``seq_start`` before it.
+    rows and of row tiles (``csrc.ops.ROW_TILE`` rows, for kernels that walk a step tile
+    by tile); ``kv_len`` is each sequence's cached length after this step, ``seq_start``
+    before it.
     """
 
     n_rows: int
@@ -50,7 +51,7 @@ class StepContext:
     kv_len: torch.Tensor
     seq_start: torch.Tensor
     max_q_len: int                      # host bound on rows per sequence; 1 means a decoding step
-    max_tiles: int                      # host bound on 64-row tiles in the step
+    max_tiles: int                      # host bound on row tiles in the step
     max_kv_len: int                     # host bound on any sequence's cached length after the step
     host: HostBatch | None = None
     positions: dict[str, Any] = field(default_factory=dict)   # name -> position encoding, tables ready
@@ -83,6 +84,19 @@ class Part:
         """The kernel libraries this part will call, so they can be compiled together up front."""
         return ()
 
+    # ---- what a step costs, for measurement (rooflines); nothing on the compute path reads these
+    def reads_whole(self) -> bool:
+        """Does a step read all of this part's tensors (a matrix product does; a row gather does not)?"""
+        return True
+
+    def flops(self, rows: int, spans: list[tuple[int, int]]) -> float:
+        """Floating-point operations of one step of ``rows`` rows, whose sequences each bring ``q`` rows after
+        ``start`` cached ones (``spans`` holds ``(start, q)``): by default two per row and matrix element."""
+        if not self.reads_whole():
+            return 0.0
+        elements = sum(_numel(shape) for shape, role, _ in self.tensor_specs().values() if role == MATRIX)
+        return 2.0 * rows * elements
+
 
 class Norm(Part):
     def forward(self, x: torch.Tensor) -> torch.Tensor:
@@ -113,6 +127,13 @@ class FeedForward(Part):
 class PositionEncoding(Part):
     def prepare(self, n_positions: int, dtype: torch.dtype, device) -> None:
         """Build whatever tables are needed for positions ``0..n_positions-1``."""
+
+
+def _numel(shape) -> int:
+    n = 1
+    for d in shape:
+        n *= int(d)
+    return n
 
 
 def matrix(shape) -> tuple[tuple[int, ...], str, str]:

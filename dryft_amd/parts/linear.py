@@ -130,7 +130,3 @@ def library_tuning():
         yield
     finally:
         tunable.tuning_enable(False)
-
-
-def linear_modules(dtype: torch.dtype) -> tuple[str, ...]:
-    return ("gemm",)

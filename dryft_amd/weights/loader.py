@@ -1,9 +1,10 @@
 """Reading a checkpoint by tensor name.
 
-Shard discovery is the reference's (engine/dryft_qwen3/weights.py:52-61): the
-files named by ``model.safetensors.index.json``, else every ``*.safetensors``
-in the folder. Unlike the reference, which stops at the first bad tensor
-(weights.py:73-75) and only warns about leftovers (weights.py:115-116), all
+Which files hold the checkpoint is decided as in the reference
+(engine/dryft_qwen3/weights.py:52-61): ``model.safetensors.index.json`` if there
+is one, else every ``*.safetensors`` in the folder; here the index is also what
+says in which shard a tensor lives, so no shard is opened for its names.
+Unlike the reference, which stops at the first bad tensor (weights.py:73-75) and only warns about leftovers (weights.py:115-116), all
 missing names, unexpected names and wrong shapes are gathered into one
 ``WeightError``; tensors are fetched one at a time rather than staged whole.
 
@@ -49,16 +50,54 @@ class WeightError(RuntimeError):
         super().__init__("\n".join(lines))
 
 
-def shard_files(model_dir: str) -> list[str]:
-    index = os.path.join(model_dir, "model.safetensors.index.json")
-    if os.path.exists(index):
-        with open(index, "r", encoding="utf-8") as f:
-            weight_map = json.load(f)["weight_map"]
-        return sorted({os.path.join(model_dir, v) for v in weight_map.values()})
-    files = sorted(glob.glob(os.path.join(model_dir, "*.safetensors")))
-    if not files:
-        raise FileNotFoundError(f"no .safetensors file in {model_dir}")
-    return files
+class ShardSet:
+    """Where each tensor of a checkpoint lives, and the open files it has been read from so far.
+
+    With an index file the map from tensor name to shard is taken from it as it stands, and a shard is
+    opened only when one of its tensors is asked for; without one every ``*.safetensors`` file of the
+    folder is opened once to learn its names.
+    """
+
+    INDEX = "model.safetensors.index.json"
+
+    def __init__(self, model_dir: str):
+        self.model_dir = model_dir
+        self.where: dict[str, str] = {}
+        self._open: dict[str, object] = {}
+        index_path = os.path.join(model_dir, self.INDEX)
+        if os.path.isfile(index_path):
+            with open(index_path, "r", encoding="utf-8") as f:
+                for tensor_name, file_name in json.load(f)["weight_map"].items():
+                    self.where[tensor_name] = os.path.join(model_dir, file_name)
+            return
+        paths = sorted(glob.glob(os.path.join(model_dir, "*.safetensors")))
+        if not paths:
+            raise FileNotFoundError(f"no .safetensors file in {model_dir}")
+        for path in paths:
+            for tensor_name in self._handle(path).keys():
+                self.where[tensor_name] = path
+
+    def _handle(self, path: str):
+        h = self._open.get(path)
+        if h is None:
+            h = self._open[path] = safe_open(path, framework="pt", device="cpu")
+        return h
+
+    def files(self) -> list[str]:
+        return sorted(set(self.where.values()))
+
+    def shape(self, name: str) -> tuple[int, ...] | None:
+        """The stored shape, or None when the shard the index names does not hold the tensor."""
+        h = self._handle(self.where[name])
+        if name not in h.keys():
+            return None
+        return tuple(h.get_slice(name).get_shape())
+
+    def tensor(self, name: str) -> torch.Tensor:
+        return self._handle(self.where[name]).get_tensor(name)
+
+    def close(self) -> None:
+        self._open.clear()
 
 
 def stored_dtype_to_held(stored: torch.dtype, role: str, compute_dtype: torch.dtype) -> torch.dtype:
@@ -82,30 +121,24 @@ def load_tensors(model_dir: str, specs: Iterable[TensorSpec], compute_dtype: tor
     specs = list(specs)
     by_name = {s.name: s for s in specs}
     ignore = set(ignore)
-    where: dict[str, str] = {}
-    handles = {}
+    shards = ShardSet(model_dir)
     try:
-        for path in shard_files(model_dir):
-            h = safe_open(path, framework="pt", device="cpu")
-            handles[path] = h
-            for name in h.keys():
-                where[name] = path
+        where = shards.where
         missing = [s.name for s in specs if s.name not in where]
         unexpected = sorted(n for n in where if n not in by_name and n not in ignore)
         wrong = []
-        other = []
         for s in specs:
-            if s.name not in where:
-                continue
-            sl = handles[where[s.name]].get_slice(s.name)
-            got = tuple(sl.get_shape())
-            if got != tuple(s.shape):
-                wrong.append((s.name, tuple(s.shape), got))
+            if s.name in where:
+                got = shards.shape(s.name)
+                if got is None:                       # the index names a shard that does not hold it
+                    missing.append(s.name)
+                elif got != tuple(s.shape):
+                    wrong.append((s.name, tuple(s.shape), got))
         if missing or unexpected or wrong:
-            raise WeightError(model_dir, missing, unexpected, wrong, other)
+            raise WeightError(model_dir, missing, unexpected, wrong)
         out: dict[str, torch.Tensor] = {}
         for name in list(by_name) + sorted(n for n in ignore if n in where):
-            t = handles[where[name]].get_tensor(name)
+            t = shards.tensor(name)
             role = by_name[name].role if name in by_name else MATRIX
             if role == INT_TABLE:
                 if t.is_floating_point():
@@ -116,4 +149,4 @@ def load_tensors(model_dir: str, specs: Iterable[TensorSpec], compute_dtype: tor
             out[name] = t.to(device=device, dtype=held).contiguous()
         return out
     finally:
-        handles.clear()
+        shards.close()

@@ -6,7 +6,8 @@ import pytest
 
 from dryft_amd.config import ConfigError, Qwen3Config, Run, read_config_json
 from dryft_amd.models import known_architectures, register_architecture, resolve_architecture
-from dryft_amd.models.qwen3 import load_preset, preset_names, qwen3_plan
+from dryft_amd.models import load_preset, preset_names
+from dryft_amd.models.qwen3 import qwen3_plan
 from helpers import TINY_A, TINY_B
 
 
@@ -16,6 +17,18 @@ def test_reads_every_size_from_the_file():
     assert (cfg.head_dim, cfg.intermediate_size, cfg.vocab_size) == (32, 224, 384)
     assert cfg.rope_theta == 1e6 and cfg.rms_norm_eps == 1e-5 and cfg.tie_word_embeddings is False
     assert (cfg.q_dim, cfg.kv_dim, cfg.group) == (256, 64, 4)          # q width differs from hidden
+
+
+def test_head_sizes_are_checked_with_everything_else():
+    """Any even head size up to 256 is a valid configuration (float32 and bfloat16 both run it); an odd or too
+    wide one is one more line of the one error."""
+    assert Qwen3Config.from_dict(dict(TINY_A, head_dim=40)).head_dim == 40
+    assert Qwen3Config.from_dict(dict(TINY_A, head_dim=72)).q_dim == 4 * 72
+    with pytest.raises(ConfigError) as e:
+        Qwen3Config.from_dict(dict(TINY_A, head_dim=258, hidden_act="gelu"))
+    assert len(e.value.problems) == 2 and any("head_dim" in p and "256" in p for p in e.value.problems)
+    with pytest.raises(ConfigError, match="even"):
+        Qwen3Config.from_dict(dict(TINY_A, head_dim=33))
 
 
 def test_head_dim_defaults_to_hidden_over_heads():
@@ -95,7 +108,10 @@ def test_plan_is_data_chosen_layer_by_layer():
     assert mixer.kind == "gqa_attention" and mixer.args["head_dim"] == 32 and mixer.args["qk_norm_eps"] == 1e-5
     assert mixer.tensors["q_norm"] == "model.layers.1.self_attn.q_norm.weight"
     assert plan.head.tensors == {"weight": "lm_head.weight"}
-    assert qwen3_plan(Qwen3Config.from_dict(TINY_A)).head.tensors == {}   # tied: the head has no tensor of its own
+    assert plan.optional_tensors == {} and plan.max_positions == 4096
+    tied = qwen3_plan(Qwen3Config.from_dict(TINY_A))                    # tied: the head reads the embedding's tensor
+    assert tied.head.tensors == tied.embedding.tensors == {"weight": "model.embed_tokens.weight"}
+    assert tied.optional_tensors == {"lm_head.weight": "model.embed_tokens.weight"}
 
 
 def test_plan_validation_catches_bad_schedules():

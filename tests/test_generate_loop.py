@@ -2,7 +2,8 @@
 
 import pytest
 
-from dryft_amd.engine.generate import FILL, check_request, generate_all, generate_batch, plan_batches
+from dryft_amd.engine.generate import (FILL, check_request, generate_all, generate_batch, generate_steps,
+                                       plan_batches)
 
 
 class Scripted:
@@ -113,6 +114,26 @@ def test_batches_one_after_another():
     acquires = [e for e in be.log if e[0] == "acquire"]
     assert [len(a[1]) for a in acquires] == [3, 3, 1]
     assert acquires[1][1] == acquires[0][1]                    # the second batch uses the first one's slots again
+
+
+def test_more_requests_than_slots_are_yielded_step_by_step():
+    """Batches run one after another and every step is handed out as it is computed: seven requests on three slots
+    give the first batch's steps, then the second's, with FILL where a request's batch is not the one running."""
+    be = Scripted(max_batch=3)
+    prompts = [[10 * i] for i in range(7)]
+    gen = generate_steps(be, prompts, 3, stop_token_ids=[32])
+    first = next(gen)
+    assert first == [1, 11, 21, FILL, FILL, FILL, FILL]
+    assert [e[0] for e in be.log].count("acquire") == 1        # nothing of the second batch has run yet
+    rest = list(gen)
+    assert [first] + rest == [
+        [1, 11, 21, FILL, FILL, FILL, FILL], [2, 12, 22, FILL, FILL, FILL, FILL], [3, 13, 23, FILL, FILL, FILL, FILL],
+        [FILL, FILL, FILL, 31, 41, 51, FILL], [FILL, FILL, FILL, 32, 42, 52, FILL], [FILL, FILL, FILL, FILL, 43, 53, FILL],
+        [FILL, FILL, FILL, FILL, FILL, FILL, 61], [FILL, FILL, FILL, FILL, FILL, FILL, 62],
+        [FILL, FILL, FILL, FILL, FILL, FILL, 63]]
+    assert sorted(be.free) == [0, 1, 2]
+    # one batch: exactly what generate_batch yields
+    assert list(generate_steps(Scripted(), prompts[:3], 3)) == list(generate_batch(Scripted(), prompts[:3], 3))
 
 
 class Chained(Scripted):

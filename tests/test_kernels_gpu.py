@@ -247,7 +247,9 @@ CASES = [  # n_heads, n_kv, D, lengths (cached tokens incl. the rows'), q rows p
 ]
 
 
-def run_attention_case(kind, dtype, n_heads, n_kv, D, lengths, tq, window=None, seed=0, misaligned=False):
+def run_attention_case(kind, dtype, n_heads, n_kv, D, lengths, tq, window=None, seed=0, misaligned=False, dead=()):
+    """``dead``: sequences that sit the step out (slot -1). They keep their rows, which every kernel leaves at
+    zero (the tiled prompt kernel by never visiting them), and have no tiles."""
     torch.manual_seed(seed + D + len(lengths))
     B, L = len(lengths), max(lengths)
     n_slots, n_pages = B + 2, sum((n + 63) // 64 for n in lengths) + 3
@@ -263,15 +265,18 @@ def run_attention_case(kind, dtype, n_heads, n_kv, D, lengths, tq, window=None, 
         far = 0 if window is None else max(0, n - window)
         k[b, far, :, :] = (4.0 * q[b, q_lens[b] - 1].float().view(n_kv, -1, D).mean(1)).to(dtype)
     scale = 1.0 / math.sqrt(D)
+    for b in dead:
+        q_pos[b] = -1                                            # the reference leaves these rows at zero
     want = attention_ref(q.float(), k.float(), v.float(), lengths, q_pos, scale, window)
     k_pages, v_pages, table, slots = build_pages(k, v, lengths, n_pages, n_slots, seed=seed, poison=1e4)
+    slots = [-1 if b in dead else s for b, s in enumerate(slots)]
     rows = sum(q_lens)
     q_packed = torch.cat([q[b, :ql] for b, ql in enumerate(q_lens)]).contiguous()
     want_packed = torch.cat([want[b, :ql] for b, ql in enumerate(q_lens)])
     row_slot = torch.tensor([slots[b] for b, ql in enumerate(q_lens) for _ in range(ql)], dtype=torch.int32)
     row_pos = torch.tensor([int(p) for b, ql in enumerate(q_lens) for p in q_pos[b, :ql]], dtype=torch.int32)
     cu = np.concatenate([[0], np.cumsum(q_lens)]).astype(np.int32)
-    tiles = np.concatenate([[0], np.cumsum([(ql + 63) // 64 for ql in q_lens])]).astype(np.int32)
+    tiles = np.concatenate([[0], np.cumsum([0 if b in dead else (ql + 63) // 64 for b, ql in enumerate(q_lens)])]).astype(np.int32)
     d = lambda t: t.to(DEV)
     out = torch.zeros(rows, n_heads, D, dtype=dtype, device=DEV)
     o = ops()
@@ -298,6 +303,8 @@ def run_attention_case(kind, dtype, n_heads, n_kv, D, lengths, tq, window=None, 
                           d(torch.from_numpy(cu)), d(torch.tensor(lengths, dtype=torch.int32)), B, part_o, part_ml,
                           splits, out, n_heads, n_kv, D, scale, w)
     close(out, want_packed, dtype, ulps=4.0, floor=1e-3, what=f"attention {kind} {n_heads}/{n_kv}/{D} {lengths} tq={tq}")
+    for b in dead:
+        assert not out[int(cu[b]):int(cu[b + 1])].any(), f"rows of sequence {b}, which sits out, were written"
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -329,10 +336,41 @@ def test_attn_causal_bf16(case, mode):
     run_attention_case(f"causal{mode}", torch.bfloat16, *case)
 
 
+# Sequences that sit out, of one row and of several hundred, before and between the ones that take part. The
+# second case has enough rows (33 tiles of 64 heads) for the kernel to choose 32 rows a wave by itself.
+DEAD_CASES = [((8, 2, 32, [1, 200, 330, 150, 70], 330), (0, 2)),
+              ((64, 16, 32, [1, 1000, 300, 1030, 64], 1030), (0, 2)),
+              ((32, 8, 128, [300, 260, 1, 129], 300), (0, 2, 3))]
+
+
+@pytest.mark.parametrize("mode", [0, 1, 2, 3])
+@pytest.mark.parametrize("case,dead", DEAD_CASES)
+def test_attn_causal_bf16_with_sequences_that_sit_out(case, dead, mode):
+    run_attention_case(f"causal{mode}", torch.bfloat16, *case, dead=dead)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_attn_rows_with_sequences_that_sit_out(dtype):
+    run_attention_case("rows", dtype, *DEAD_CASES[0][0], dead=DEAD_CASES[0][1])
+
+
 @pytest.mark.parametrize("splits", [1, 2, 5, 32])
 @pytest.mark.parametrize("case", [c for c in CASES if c[4] == 1])
 def test_attn_split_bf16(case, splits):
     run_attention_case(splits, torch.bfloat16, *case)
+
+
+# The reference's own lengths for its split-KV kernel (kernels/attn_decode.py:204-215) at Qwen3-4B's heads: a
+# split here walks up to 128 pages, four waves taking them in turn.
+LONG_DECODE = [(32, 8, 128, [2047], 1), (32, 8, 128, [8191, 4096], 1), (32, 8, 128, list(range(3, 3 + 16 * 31, 31)), 1)]
+
+
+@pytest.mark.parametrize("splits", [1, 8, 32])
+@pytest.mark.parametrize("case", LONG_DECODE)
+def test_attn_split_bf16_long_sequences(case, splits):
+    run_attention_case(splits, torch.bfloat16, *case)
+    if splits == 8:
+        run_attention_case(splits, torch.bfloat16, *case, dead=(0,) if len(case[3]) > 1 else ())
 
 
 @pytest.mark.parametrize("n_heads,n_kv,D,splits,window", [(32, 8, 128, 3, 0), (6, 3, 48, 1, 0), (4, 2, 16, 2, 0),

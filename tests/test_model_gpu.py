@@ -31,26 +31,27 @@ LENGTHS = [1, 5, 9, 17, 33, 64, 65, 70, 128, 129, 131, 200]     # 64-token cache
 class Case:
     """A tiny model folder, its plain logits and engines on it."""
 
-    def __init__(self, name, tmp, sharp=False):
-        raw, kw = TINY[name]
+    def __init__(self, name, tmp, sharp=False, raw=None, kw=None, lengths=LENGTHS, sharpness=4.0):
+        if raw is None:
+            raw, kw = TINY[name]
         self.name = name
         self.dir = make_model_dir(os.path.join(tmp, name + ("_sharp" if sharp else "")), raw, **kw)
         if sharp:
-            self._sharpen()
+            self._sharpen(sharpness)
         self.raw, self.weights = read_model_dir(self.dir)
         self.vocab = raw["vocab_size"]
-        self.requests = {f"r{n}": random_tokens(n, self.vocab, seed=1000 + n) for n in LENGTHS}
+        self.requests = {f"r{n}": random_tokens(n, self.vocab, seed=1000 + n) for n in lengths}
         self._plain = {}
         self._engines = {}
 
-    def _sharpen(self):
+    def _sharpen(self, factor):
         """Scale every q_norm weight so that attention is peaked and a lost or misplaced key shows."""
         from safetensors.torch import load_file, save_file
         path = os.path.join(self.dir, "model.safetensors")
         t = load_file(path)
         for k in t:
             if k.endswith("q_norm.weight"):
-                t[k] = (t[k].float() * 4.0).to(t[k].dtype)
+                t[k] = (t[k].float() * factor).to(t[k].dtype)
         save_file(t, path)
 
     def plain_logits(self, rid):
@@ -87,10 +88,11 @@ def cases(tmp_path_factory):
     out = {n: Case(n, tmp) for n in TINY}
     out["C_sharp"] = Case("C", tmp, sharp=True)
     out["A_sharp"] = Case("A", tmp, sharp=True)
+    out["B_sharp"] = Case("B", tmp, sharp=True)
     return out
 
 
-CASE_NAMES = ["A", "B", "C", "D", "C_sharp", "A_sharp"]
+CASE_NAMES = ["A", "B", "C", "D", "C_sharp", "A_sharp", "B_sharp"]
 
 
 def replay(engine, records):
@@ -210,6 +212,67 @@ def test_first_tokens(cases, name, dtype):
                         "end": ["r9"] if i == len(toks) - 1 else []})
     got = collect_positions(records, replay(case.engine(dtype), records))
     check_against_plain(case, got, dtype, "first tokens")
+
+
+def portions_trace(case):
+    """r200 arrives in portions of 63, 2, 63, 1 and 71 tokens: one starts in the middle of a page, one is two tokens
+    long, one ends exactly at a page's edge, one is a single token. Beside it r131 starts with 127 tokens and then
+    goes on one token a step, so every later step mixes a portion of a prompt with a decoding row; r17 joins the
+    first step only. Logits are wanted everywhere."""
+    long, short, tiny = case.requests["r200"], case.requests["r131"], case.requests["r17"]
+    cuts = [0, 63, 65, 128, 129, 200]
+    records = []
+    for i in range(5):
+        part = long[cuts[i]:cuts[i + 1]]
+        entries = [{"id": "r200", "tokens": part, "want": list(range(len(part)))}]
+        if i == 0:
+            entries.append({"id": "r131", "tokens": short[:127], "want": list(range(127))})
+            entries.append({"id": "r17", "tokens": tiny, "want": list(range(17))})
+        else:
+            entries.insert(0, {"id": "r131", "tokens": [short[126 + i]], "want": [0]})
+        end = (["r17"] if i == 0 else []) + (["r200", "r131"] if i == 4 else [])
+        records.append({"step": i, "entries": entries, "end": end})
+    return records
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["B", "C_sharp", "A_sharp", "B_sharp", "D"])
+def test_prompt_in_portions_beside_decoding_rows(cases, name, dtype):
+    """How the tokens are cut into steps changes no logit: a prompt fed in portions, in steps that also hold
+    sequences going on by one token, against the plain implementation of whole sequences."""
+    case = cases[name]
+    records = portions_trace(case)
+    got = collect_positions(records, replay(case.engine(dtype), records))
+    assert len(got) == 200 + 131 + 17
+    check_against_plain(case, got, dtype, "portions")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["B_sharp", "C"])
+def test_sequences_that_sit_out_of_a_prompt_step(cases, name, dtype):
+    """Sequences with slot -1 keep their rows in a step but take no part: prompts beside them come out as alone,
+    no cache slot and no length changes for them, and what they leave in the residual stream is finite."""
+    from dryft_amd.engine.step import SeqStep
+    case = cases[name]
+    engine = case.engine(dtype)
+    a, b = case.requests["r70"], case.requests["r131"]
+    filler = case.requests["r200"]
+    slots = engine.acquire(2)
+    try:
+        steps = [SeqStep(-1, filler[:1], [0]), SeqStep(slots[0], a, list(range(len(a)))), SeqStep(-1, filler, []),
+                 SeqStep(slots[1], b[:-1], list(range(len(b) - 1))), SeqStep(-1, filler[:65], [3])]
+        first = engine.step(steps).float().cpu()
+        assert first.shape[0] == len(a) + len(b) - 1 and torch.isfinite(first).all()
+        last = engine.step([SeqStep(-1, [0], []), SeqStep(slots[1], b[-1:], [0])]).float().cpu()
+        host = engine.cache.lengths_host()
+        assert [int(host[s]) for s in slots] == [len(a), len(b)]
+        assert int(engine.cache.lengths_dev.sum()) == len(a) + len(b)
+    finally:
+        engine.release(slots)
+    got = {("r70", i): first[i] for i in range(len(a))}
+    got.update({("r131", i): first[len(a) + i] for i in range(len(b) - 1)})
+    got[("r131", len(b) - 1)] = last[0]
+    check_against_plain(case, got, dtype, "sitting out")
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -430,7 +493,7 @@ def test_layer_sizes_of_a_real_model_bfloat16_agrees_with_float32():
     then decoding through captured graphs at 3 sequences, and 40 sequences for the products of 17 to 64 rows."""
     from dryft_amd import Engine
     from dryft_amd.engine.step import SeqStep
-    from dryft_amd.models.qwen3 import load_preset
+    from dryft_amd.models import load_preset
     raw = dict(load_preset("qwen3-4b"))
     raw["num_hidden_layers"] = 2
     vocab = raw["vocab_size"]
@@ -461,6 +524,123 @@ def test_layer_sizes_of_a_real_model_bfloat16_agrees_with_float32():
     out = engines["bfloat16"].generate_all([p[:200] for p in prompts], 5)
     assert [len(r) for r in out] == [5, 5, 5] and all(0 <= t < vocab for r in out for t in r)
     assert engines["bfloat16"].cache.slots.free_count == 40
+
+
+REAL_LENGTHS = [78, 308, 1108] + list(range(20, 44))
+
+
+@pytest.fixture(scope="module")
+def real_cases(tmp_path_factory):
+    """Two layers with Qwen3-4B's layer sizes (head size 128, four query heads to a kv head, widths 2560 / 9728) and a
+    vocabulary of 2,048, small enough for the plain implementation in float64; once as drawn and once with
+    sharpened attention."""
+    from dryft_amd.models import load_preset
+    raw = dict(load_preset("qwen3-4b"))
+    raw.update(num_hidden_layers=2, vocab_size=2048)
+    tmp = str(tmp_path_factory.mktemp("real"))
+    kw = dict(seed=77, norm_std=0.1, std=0.02)
+    return {False: Case("real", tmp, raw=raw, kw=kw, lengths=REAL_LENGTHS),
+            True: Case("real", tmp, sharp=True, raw=raw, kw=kw, lengths=REAL_LENGTHS, sharpness=3.0)}
+
+
+@pytest.mark.parametrize("sharp", [False, True])
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_real_layer_sizes_against_plain(real_cases, dtype, sharp):
+    """The sizes at which the matrix-core kernels take their fast paths, against the plain implementation (not
+    against the other precision of the engine): prompts of 70, 300 and 1,100 tokens in one step with logits
+    everywhere, then 8 given tokens each through the captured decoding graph; then 24 short sequences, whose
+    decoding steps take the products of 17 to 64 rows."""
+    from dryft_amd.engine.step import SeqStep
+    case = real_cases[sharp]
+    engine = case.engine(dtype, max_batch=24, max_len=1280, max_tokens=3 * 1280 + 24 * 64, use_graph=True)
+    names = ["r78", "r308", "r1108"]
+    got = {}
+    slots = engine.acquire(3)
+    try:
+        prompts = [case.requests[n][:-8] for n in names]
+        logits = engine.step([SeqStep(s, p, list(range(len(p)))) for s, p in zip(slots, prompts)]).float().cpu()
+        row = 0
+        for n, p in zip(names, prompts):
+            for i in range(len(p)):
+                got[(n, i)] = logits[row + i]
+            row += len(p)
+        graph = engine._graph_for(3)
+        for t in range(8):
+            engine.cache.begin_step(slots, [1, 1, 1])
+            lg = graph.replay(slots, [case.requests[n][len(case.requests[n]) - 8 + t] for n in names]).float().cpu()
+            engine.cache.end_step(slots, [1, 1, 1])
+            for b, n in enumerate(names):
+                got[(n, len(case.requests[n]) - 8 + t)] = lg[b].clone()
+    finally:
+        engine.release(slots)
+    assert len(got) == 78 + 308 + 1108
+    check_against_plain(case, got, dtype, "real sizes")
+    # 24 sequences: their prompts in one step, then two decoding steps of 24 rows, eager and through the graph
+    many = [f"r{n}" for n in range(20, 44)]
+    got = {}
+    slots = engine.acquire(24)
+    try:
+        prompts = [case.requests[n][:-2] for n in many]
+        logits = engine.step([SeqStep(s, p, [len(p) - 1]) for s, p in zip(slots, prompts)]).float().cpu()
+        for b, n in enumerate(many):
+            got[(n, len(prompts[b]) - 1)] = logits[b]
+        lg = engine.step([SeqStep(s, [case.requests[n][-2]], [0]) for s, n in zip(slots, many)]).float().cpu()
+        for b, n in enumerate(many):
+            got[(n, len(case.requests[n]) - 2)] = lg[b]
+        graph = engine._graph_for(24)
+        engine.cache.begin_step(slots, [1] * 24)
+        lg = graph.replay(slots, [case.requests[n][-1] for n in many]).float().cpu()
+        engine.cache.end_step(slots, [1] * 24)
+        for b, n in enumerate(many):
+            got[(n, len(case.requests[n]) - 1)] = lg[b].clone()
+    finally:
+        engine.release(slots)
+    check_against_plain(case, got, dtype, "real sizes, 24 sequences")
+
+
+# --------------------------------------------------------------------------------- the command line
+def run_cli(*argv, timeout=600):
+    proc = subprocess.run([sys.executable, "-m", "dryft_amd", *argv], capture_output=True, text=True, timeout=timeout,
+                          cwd=ROOT)
+    assert proc.returncode == 0, proc.stderr[-3000:]
+    return proc.stdout
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_command_line_generate(cases, dtype):
+    """`python -m dryft_amd generate` prints what the entry point generates, and what the plain greedy loop does."""
+    case = cases["B"]
+    prompts = [random_tokens(n, case.vocab, seed=300 + n) for n in (4, 17, 9)]
+    text = ";".join(",".join(map(str, p)) for p in prompts)
+    out = run_cli("generate", "--model", case.dir, "--dtype", dtype, "--prompt-ids", text, "--max-new-tokens", "7",
+                  "--max-len", "64")
+    printed = [[int(t) for t in line.split(",")] for line in out.strip().splitlines()]
+    assert printed == case.engine(dtype, max_batch=3, max_len=64, use_graph=True).generate_all(prompts, 7)
+    check_generation(case, prompts, [[col[t] for col in printed] for t in range(7)], 7, dtype)
+    # one JSON list per step with --stream, stop tokens and a temperature with its seed
+    stop = printed[1][3]
+    out = run_cli("generate", "--model", case.dir, "--dtype", dtype, "--prompt-ids", text, "--max-new-tokens", "7",
+                  "--max-len", "64", "--stream", "--stop-ids", str(stop), "--temperature", "0.7", "--sample-seed", "5")
+    steps = [json.loads(line) for line in out.strip().splitlines()]
+    want = list(case.engine(dtype, max_batch=3, max_len=64, use_graph=True).generate(
+        prompts, 7, temperature=0.7, sample_seed=5, stop_token_ids=[stop]))
+    assert steps == want
+
+
+def test_command_line_bench_and_profile():
+    """`bench` prints one JSON line per workload with the reference's quantities (agent/bench.py:61-81); `profile`
+    prints a per-kernel table in which this library's kernels appear by name."""
+    out = run_cli("bench", "--tiny", "--workload", "t,2,16,4", "--workload", "u,1,5,3", "--samples", "1")
+    lines = [json.loads(line) for line in out.strip().splitlines()]
+    assert [(r["workload"], r["batch"], r["in"], r["out"]) for r in lines] == [("t", 2, 16, 4), ("u", 1, 5, 3)]
+    for r in lines:
+        assert r["tok_s"] > 0 and r["total_ms"] >= r["ttft_ms"] > 0 and r["tpot_ms"] > 0
+    out = run_cli("profile", "--tiny", "--batch", "2", "--prompt-len", "16", "--steps", "2")
+    assert "2 decoding steps of 2 sequences" in out and "implied bandwidth" in out
+    table = out.splitlines()
+    assert any("attn_split_kernel" in row for row in table) and any("add_rmsnorm" in row for row in table)
+    out = run_cli("profile", "--tiny", "--batch", "2", "--prompt-len", "70", "--prefill")
+    assert "one step of 2 prompts of 70 tokens" in out and any("attn_causal_kernel" in row for row in out.splitlines())
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

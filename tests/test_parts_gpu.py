@@ -87,14 +87,13 @@ def test_embedding_and_head_parts(dtype):
     emb = load_part(TokenEmbedding(331, 80), {"weight": table}, dtype)
     toks = torch.tensor([0, 330, 7, 7], dtype=torch.int32)
     assert torch.equal(emb.forward(toks.to(DEV)).cpu(), table[toks.long()])
-    head = LMHead(331, 80, tied=True)
-    assert head.tensor_specs() == {}
-    head.tie(emb.weight)
+    head = LMHead(331, 80)
+    head.load({"weight": emb.weight})                       # a tied head is handed the embedding's own tensor
     h = torch.randn(5, 80).to(dtype)
     logits = head.forward(h.to(DEV))
     assert logits.dtype == torch.float32
     close(logits, h.double() @ table.double().T, torch.float32 if dtype == torch.float32 else dtype, "tied head", ulps=0.5)
-    own = load_part(LMHead(331, 80, tied=False), {"weight": table * 2}, dtype)
+    own = load_part(LMHead(331, 80), {"weight": table * 2}, dtype)
     close(own.forward(h.to(DEV)), 2 * (h.double() @ table.double().T), torch.float32 if dtype == torch.float32 else dtype,
           "own head", ulps=0.5)
 
@@ -251,7 +250,7 @@ def toy_plan(cfg):
     return ModelPlan(vocab_size=cfg.vocab_size, hidden_size=H,
                      embedding=PartSpec("token_embedding", dict(vocab_size=cfg.vocab_size, hidden_size=H), {"weight": "emb"}),
                      layers=layers, schedule=(Run(0, 0), Run(1, 1)), final_norm=norm("final"),
-                     head=PartSpec("lm_head", dict(vocab_size=cfg.vocab_size, hidden_size=H, tied=True), {}),
+                     head=PartSpec("lm_head", dict(vocab_size=cfg.vocab_size, hidden_size=H), {"weight": "emb"}),   # tied: the embedding's tensor
                      positions={"rotary": PartSpec("rotary", dict(dim=16, theta=1e4))})
 
 
@@ -525,7 +524,7 @@ def routed_plan(cfg):
     return ModelPlan(vocab_size=cfg.vocab_size, hidden_size=H,
                      embedding=PartSpec("token_embedding", dict(vocab_size=cfg.vocab_size, hidden_size=H), {"weight": "emb"}),
                      layers=(layer(0), layer(1)), schedule=(Run(0, 0), Run(1, 1)), final_norm=norm("final"),
-                     head=PartSpec("lm_head", dict(vocab_size=cfg.vocab_size, hidden_size=H, tied=True), {}),
+                     head=PartSpec("lm_head", dict(vocab_size=cfg.vocab_size, hidden_size=H), {"weight": "emb"}),   # tied: the embedding's tensor
                      positions={"sinusoid": PartSpec("toy_sinusoid_positions", dict(width=H))})
 
 

@@ -9,8 +9,8 @@ from safetensors.torch import load_file, save_file
 
 from dryft_amd.engine.model import DecoderModel
 from dryft_amd.models import resolve_architecture
-from dryft_amd.weights import (INT_TABLE, MATRIX, VECTOR, TensorSpec, WeightError, load_tensors, random_tensors,
-                               write_model_dir)
+from dryft_amd.weights import (INT_TABLE, MATRIX, VECTOR, ShardSet, TensorSpec, WeightError, load_tensors,
+                               random_tensors, write_model_dir)
 from helpers import TINY_A, TINY_B, make_model_dir
 
 
@@ -96,7 +96,7 @@ def test_untied_model_needs_its_head_and_tied_copy_must_match(tmp_path):
     t["lm_head.weight"] = t["lm_head.weight"] + 1
     save_file(t, file)
     model = model_for(TINY_A)
-    with pytest.raises(ValueError, match="differs from the embedding"):
+    with pytest.raises(ValueError, match="differs from model.embed_tokens.weight"):
         model.load(load_tensors(path, model.tensor_specs(), torch.float32, ignore=model.optional_names()))
 
 
@@ -131,6 +131,18 @@ def test_shards_are_found_through_the_index(tmp_path):
         json.dump(index, f)
     got = load_tensors(path, model_for(TINY_A).tensor_specs(), torch.bfloat16)
     assert all(torch.equal(got[n], t[n]) for n in names)
+    # the index alone says where a tensor lives: a file of the folder that it does not name is never opened,
+    # and a tensor that the named shard lacks is reported as missing
+    with open(os.path.join(path, "stray.safetensors"), "w") as f:
+        f.write("not a safetensors file")
+    assert ShardSet(path).files() == [os.path.join(path, f"model-0000{i}-of-00002.safetensors") for i in (1, 2)]
+    load_tensors(path, model_for(TINY_A).tensor_specs(), torch.bfloat16)
+    index["weight_map"][names[0]] = "model-00002-of-00002.safetensors"
+    with open(os.path.join(path, "model.safetensors.index.json"), "w") as f:
+        json.dump(index, f)
+    with pytest.raises(WeightError) as e:
+        load_tensors(path, model_for(TINY_A).tensor_specs(), torch.bfloat16)
+    assert e.value.missing == [names[0]]
     with pytest.raises(FileNotFoundError):
         load_tensors(str(tmp_path / "empty"), [], torch.bfloat16)
 
@@ -148,3 +160,36 @@ def test_fused_rows_equal_their_parts(tmp_path):
     assert torch.equal(att.w_qkv[320:], tensors[p + "self_attn.v_proj.weight"])
     assert torch.equal(ffn.w_gate_up[:224], tensors[p + "mlp.gate_proj.weight"])
     assert torch.equal(ffn.w_gate_up[224:], tensors[p + "mlp.up_proj.weight"])
+
+
+def test_command_line_make_model_round_trip(tmp_path):
+    """`python -m dryft_amd make-model` writes the folder that the random-weights mode describes: the same
+    configuration and, tensor for tensor, what the seed gives."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    out = str(tmp_path / "made")
+    proc = subprocess.run([sys.executable, "-m", "dryft_amd", "make-model", "--preset", "tiny-b", "--weight-seed", "3",
+                           "--norm-std", "0.1", "--out", out], capture_output=True, text=True, cwd=root, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert proc.stdout.strip() == out
+    with open(os.path.join(out, "config.json")) as f:
+        raw = json.load(f)
+    from dryft_amd.models import load_preset
+    assert raw == load_preset("tiny-b")
+    model = model_for(raw)
+    specs = model.tensor_specs()
+    loaded = load_tensors(out, specs, torch.bfloat16)
+    want = random_tensors(specs, 3, torch.bfloat16, norm_std=0.1)
+    assert all(torch.equal(loaded[s.name], want[s.name]) for s in specs)
+    # a config.json of one's own instead of a preset, in float32
+    cfg_path = str(tmp_path / "c.json")
+    with open(cfg_path, "w") as f:
+        json.dump(dict(TINY_A, vocab_size=300), f)
+    out2 = str(tmp_path / "made2")
+    proc = subprocess.run([sys.executable, "-m", "dryft_amd", "make-model", "--config", cfg_path, "--dtype", "fp32",
+                           "--out", out2], capture_output=True, text=True, cwd=root, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    t = load_file(os.path.join(out2, "model.safetensors"))
+    assert t["model.embed_tokens.weight"].shape == (300, 64) and t["model.embed_tokens.weight"].dtype == torch.float32
+    assert "lm_head.weight" not in t
