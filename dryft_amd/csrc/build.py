@@ -26,7 +26,8 @@ ARCH = "gfx950"
 HIPCC_FLAGS = ["-O3", f"--offload-arch={ARCH}", "-std=c++17", "-shared", "-fPIC", "-fvisibility=hidden",
                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 MODULES = ("batch", "embed", "norm", "activation", "rope_kv", "attn_rows", "attn_mfma", "gemm", "sampling")
-_HEADERS = ("common.h",)
+_HEADERS = ("common.h",)                       # every library includes these
+_OWN_HEADERS = {"sampling": ("sampling.h",)}    # and some a header of their own
 
 _loaded: dict[str, ctypes.CDLL] = {}
 _lock = threading.Lock()
@@ -42,7 +43,7 @@ def _say(msg: str) -> None:
 
 def _source_digest(name: str) -> str:
     h = hashlib.sha256()
-    for f in (name + ".hip",) + _HEADERS:
+    for f in (name + ".hip",) + _HEADERS + _OWN_HEADERS.get(name, ()):
         with open(os.path.join(_HERE, f), "rb") as fh:
             h.update(fh.read())
     h.update(" ".join(HIPCC_FLAGS).encode())

@@ -5,6 +5,9 @@
 //    reaches u * sum(p), u in [0,1) given per row by the caller. The reference has no temperature
 //    sampling; this is this library's own.
 #include "common.h"
+#include "sampling.h"
+#include <mutex>
+#include <stdio.h>
 
 #define SAMPLE_THREADS 1024
 
@@ -270,4 +273,52 @@ DRYFT_API int dryft_sample_rows(const float* logits, int n_rows, int vocab, int6
   hipLaunchKernelGGL(sample_pick_kernel, dim3(n_rows), dim3(PICK_THREADS), 0, stream, logits, vocab, row_stride, chunks,
                      1.f / temperature, chunk_max, chunk_sum, uniforms, out);
   return DRYFT_LAUNCH_CHECK();
+}
+
+// ---------------------------------------------------------------------------------------------------
+// The greedy choice with the library's own scratch memory (see sampling.h). `scratch` is a host-side stand-in
+// in host code, not a device address: the address on each device is looked up once and kept, and only that
+// pointer is handed to kernels.
+static __device__ __align__(256) unsigned char scratch[DRYFT_ARGMAX_NOALLOC_ENTRIES * (sizeof(float) + sizeof(int))];
+
+#define NOALLOC_MAX_DEVICES 64
+static void* scratch_on_device[NOALLOC_MAX_DEVICES];   // address of `scratch` on each device, null until looked up
+static std::mutex scratch_lock;
+
+// The current device's copy of the array. Returns 0 or a HIP error code.
+static int scratch_of_current_device(void** ptr) {
+  int device = -1;
+  hipError_t err = hipGetDevice(&device);
+  if (err != hipSuccess) return (int)err;
+  if (device < 0 || device >= NOALLOC_MAX_DEVICES) return (int)hipErrorInvalidDevice;
+  std::lock_guard<std::mutex> guard(scratch_lock);
+  if (scratch_on_device[device] == nullptr) {
+    void* found = nullptr;
+    err = hipGetSymbolAddress(&found, HIP_SYMBOL(scratch));
+    if (err != hipSuccess) return (int)err;
+    if (found == nullptr) return (int)hipErrorInvalidSymbol;
+    scratch_on_device[device] = found;
+  }
+  *ptr = scratch_on_device[device];
+  return 0;
+}
+
+int dryft_argmax_rows_noalloc(const float* logits, int n_rows, int vocab, int64_t row_stride, int* out, int chunks,
+                              hipStream_t stream) {
+  if (n_rows <= 0) return 0;
+  if (logits == nullptr || out == nullptr || vocab <= 0 || chunks > 65535) return -1;
+  if (chunks <= 1) return dryft_argmax_rows(logits, n_rows, vocab, row_stride, out, 1, nullptr, nullptr, stream);
+  const long long entries = (long long)n_rows * chunks;
+  if (entries > DRYFT_ARGMAX_NOALLOC_ENTRIES) {
+    fprintf(stderr, "dryft_argmax_rows_noalloc: %d rows x %d stretches = %lld entries exceed the library's scratch of "
+                    "%d entries; use fewer stretches or rows, or dryft_argmax_rows with buffers of your own\n",
+            n_rows, chunks, entries, DRYFT_ARGMAX_NOALLOC_ENTRIES);
+    return -2;
+  }
+  void* base = nullptr;
+  const int rc = scratch_of_current_device(&base);
+  if (rc) return rc;
+  float* best_v = (float*)base;                                   // [entries] floats, then [entries] ints
+  int* best_i = (int*)((unsigned char*)base + DRYFT_ARGMAX_NOALLOC_ENTRIES * sizeof(float));
+  return dryft_argmax_rows(logits, n_rows, vocab, row_stride, out, chunks, best_v, best_i, stream);
 }
