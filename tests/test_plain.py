@@ -128,6 +128,91 @@ def test_swiglu_is_silu_gate_times_up():
     assert not P.swiglu(h, zero_up, "").any()
 
 
+# The reference states four of its formulas a second time, element by element, in the docstrings and bodies of
+# its kernels. The tests below write those second statements out as scalar arithmetic and hold the plain
+# implementation (written from the first statements, model.py) against them; in each, the plausible other
+# reading is shown to give another number.
+
+def test_rotation_pairs_element_by_element():
+    """kernels/rope_qknorm.py:15-20, 39-47: with x1, x2 the two halves of a head and c, s the first half of a table
+    row, o1 = x1 c - x2 s and o2 = x2 c + x1 s: element j is paired with element j + d/2 (not with j + 1)."""
+    d, pos, theta = 8, 3, 100.0
+    x = torch.tensor([0.5, -1.0, 2.0, 0.25, 1.5, 3.0, -0.75, 1.0], dtype=torch.float64)
+    cos, sin = P.rope_tables(d, theta, pos + 1, torch.float64)
+    got = P.apply_rope(x.view(1, 1, d), cos[pos:pos + 1], sin[pos:pos + 1]).view(d)
+    want = torch.empty(d, dtype=torch.float64)
+    interleaved = torch.empty(d, dtype=torch.float64)
+    for j in range(d // 2):
+        angle = float(torch.tensor(pos, dtype=torch.float32) * (1.0 / torch.tensor(theta, dtype=torch.float32) ** (2 * j / d)))
+        c, sn = math.cos(angle), math.sin(angle)
+        x1, x2 = float(x[j]), float(x[j + d // 2])
+        want[j], want[j + d // 2] = x1 * c - x2 * sn, x2 * c + x1 * sn
+        a, b = float(x[2 * j]), float(x[2 * j + 1])                     # the other convention: neighbours
+        interleaved[2 * j], interleaved[2 * j + 1] = a * c - b * sn, b * c + a * sn
+    assert torch.allclose(got, want, atol=1e-6)
+    assert not torch.allclose(got, interleaved, atol=1e-2)
+    # the sign: a quarter turn takes (1, 0) to (0, 1), i.e. x1 goes to the second half with a plus
+    quarter = P.apply_rope(torch.tensor([1.0, 0.0]).view(1, 1, 2), torch.zeros(1, 2), torch.ones(1, 2)).view(2)
+    assert quarter.tolist() == [0.0, 1.0]
+
+
+def test_norm_then_rotation_element_by_element(tiny_b):
+    """kernels/rope_qknorm.py:15-18 and 39-47 (`_norm_rope`): n = x * rsqrt(mean(x^2) + eps) * w first, then the
+    rotation of n. `attention_block` applied to one head must give keys that are exactly that."""
+    raw, w = tiny_b
+    d, eps = raw["head_dim"], raw["rms_norm_eps"]
+    w64 = {k: v.double() for k, v in w.items()}
+    torch.manual_seed(8)
+    h = torch.randn(3, raw["hidden_size"], dtype=torch.float64)
+    p = "model.layers.0.self_attn."
+    cos, sin = P.rope_tables(d, raw["rope_theta"], 3, torch.float64)
+    k = (h @ w64[p + "k_proj.weight"].T).view(3, raw["num_key_value_heads"], d)
+    kn = P.apply_rope(P.rms_norm(k, w64[p + "k_norm.weight"], eps), cos, sin)
+    pos, head = 2, 1
+    x, wt = k[pos, head], w64[p + "k_norm.weight"]
+    inv = 1.0 / math.sqrt(float((x * x).sum()) / d + eps)
+    for j in range(d // 2):
+        n1, n2 = float(x[j]) * inv * float(wt[j]), float(x[j + d // 2]) * inv * float(wt[j + d // 2])
+        c, sn = float(cos[pos, j]), float(sin[pos, j])
+        assert math.isclose(float(kn[pos, head, j]), n1 * c - n2 * sn, rel_tol=1e-9, abs_tol=1e-12)
+        assert math.isclose(float(kn[pos, head, j + d // 2]), n2 * c + n1 * sn, rel_tol=1e-9, abs_tol=1e-12)
+
+
+def test_gate_columns_come_first_and_carry_the_silu():
+    """kernels/silu_mul.py:3-5, 29-32: of the fused product's [M, 2I] columns the first I are the gate, the next I
+    the up projection (weights.py:98-100 stacks gate above up), and y = silu(g) * u with silu(x) = x / (1 + exp(-x)).
+    A gate far below zero closes the unit whatever `up` says; an `up` far below zero does not."""
+    w = {"mlp.gate_proj.weight": torch.tensor([[1.0, 0.0], [0.0, 1.0]], dtype=torch.float64),
+         "mlp.up_proj.weight": torch.tensor([[0.0, 1.0], [1.0, 0.0]], dtype=torch.float64),
+         "mlp.down_proj.weight": torch.eye(2, dtype=torch.float64)}
+    h = torch.tensor([[-40.0, 3.0]], dtype=torch.float64)              # g = (-40, 3), u = (3, -40)
+    y = P.swiglu(h, w, "")[0]
+    assert abs(float(y[0])) < 1e-12                                    # silu(-40) * 3: closed
+    silu3 = 3.0 / (1.0 + math.exp(-3.0))
+    assert math.isclose(float(y[1]), silu3 * -40.0, rel_tol=1e-12)     # silu(3) * (-40): open, and large
+    # were the silu on `up`, the first unit would give -40 * silu(3) and the second one nothing
+
+
+def test_scores_are_scaled_by_one_over_root_head_dim():
+    """model.py:65 (`self.scale = 1.0 / math.sqrt(cfg.head_dim)`) and kernels/attn_decode.py:180-196: with head
+    size 4, a query and a key that are both (1, -1, 1, -1) after the norm score 4 * 1/2 = 2 against 0 for an
+    orthogonal key, so the second position's probabilities are (1, e^2) / (1 + e^2) and its output
+    p0 * h0 + p1 * h1, whose second element is 1 - 2 p1 = -tanh(1)."""
+    cfg = {"num_attention_heads": 1, "num_key_value_heads": 1, "head_dim": 4, "hidden_size": 4, "rms_norm_eps": 1e-12}
+    eye = torch.eye(4, dtype=torch.float64)
+    p = "l."
+    w = {p + f"self_attn.{n}_proj.weight": eye for n in "qkvo"}
+    w[p + "self_attn.q_norm.weight"] = w[p + "self_attn.k_norm.weight"] = torch.ones(4, dtype=torch.float64)
+    h = torch.tensor([[1.0, 1.0, 1.0, 1.0], [1.0, -1.0, 1.0, -1.0]], dtype=torch.float64)
+    no_turn = (torch.ones(2, 4, dtype=torch.float64), torch.zeros(2, 4, dtype=torch.float64))
+    out = P.attention_block(h, w, p, cfg, *no_turn)
+    assert torch.allclose(out[0], h[0], atol=1e-9)
+    assert math.isclose(float(out[1, 0]), 1.0, rel_tol=1e-9)
+    assert math.isclose(float(out[1, 1]), -math.tanh(1.0), rel_tol=1e-9)            # scale 1/2
+    assert not math.isclose(float(out[1, 1]), -math.tanh(0.5), rel_tol=1e-3)        # scale 1/4 (1 / head_dim)
+    assert not math.isclose(float(out[1, 1]), -math.tanh(2.0), rel_tol=1e-3)        # no scale
+
+
 @pytest.fixture(scope="module")
 def tiny_b(tmp_path_factory):
     path = make_model_dir(str(tmp_path_factory.mktemp("plain") / "b"), TINY_B, seed=22, norm_std=0.1)
