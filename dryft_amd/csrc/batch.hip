@@ -4,6 +4,8 @@
 // tensor for the same reason, engine/dryft_qwen3/cache.py:8-10).
 #include "common.h"
 
+#define PREPARE_THREADS 256
+
 // One block. Inputs: seq_slot[B] (-1 = not taking part), q_len[B] (new tokens of
 // each sequence), lengths[slots] (cached tokens per slot). Outputs: cu_rows[B+1],
 // tile_cu[B+1] (prefix sums of rows and of tiles of `tile_rows` rows), kv_len[B] (cached
@@ -14,20 +16,36 @@ __global__ void prepare_batch_kernel(const int* __restrict__ seq_slot, const int
                                      int* __restrict__ kv_len, int* __restrict__ seq_start,
                                      int* __restrict__ row_seq, int* __restrict__ row_slot,
                                      int* __restrict__ row_pos) {
-  if (threadIdx.x == 0) {
-    int rows = 0, tiles = 0;
-    for (int s = 0; s < n_seqs; ++s) {
-      cu_rows[s] = rows;
-      tile_cu[s] = tiles;
-      const int slot = seq_slot[s];
-      const int q = slot >= 0 ? q_len[s] : 0;
-      const int past = slot >= 0 ? lengths[slot] : 0;
-      seq_start[s] = past;
-      kv_len[s] = past + q;
-      rows += q_len[s];                         // rows of a sequence that sits out still occupy their places
-      tiles += (q + tile_rows - 1) / tile_rows;
-      if (slot >= 0) lengths[slot] = past + q;
-    }
+  // prefix sums over the sequences: every thread sums a run of them, the runs' sums are added up in LDS
+  __shared__ int run_rows[PREPARE_THREADS], run_tiles[PREPARE_THREADS];
+  const int per = (n_seqs + PREPARE_THREADS - 1) / PREPARE_THREADS;
+  const int s0 = min(n_seqs, (int)threadIdx.x * per), s1 = min(n_seqs, s0 + per);
+  int rows = 0, tiles = 0;
+  for (int s = s0; s < s1; ++s) {
+    rows += q_len[s];                           // rows of a sequence that sits out still occupy their places
+    tiles += seq_slot[s] >= 0 ? (q_len[s] + tile_rows - 1) / tile_rows : 0;
+  }
+  run_rows[threadIdx.x] = rows;
+  run_tiles[threadIdx.x] = tiles;
+  __syncthreads();
+  rows = tiles = 0;
+  for (int t = 0; t < (int)threadIdx.x; ++t) {
+    rows += run_rows[t];
+    tiles += run_tiles[t];
+  }
+  for (int s = s0; s < s1; ++s) {
+    cu_rows[s] = rows;
+    tile_cu[s] = tiles;
+    const int slot = seq_slot[s];
+    const int q = slot >= 0 ? q_len[s] : 0;
+    const int past = slot >= 0 ? lengths[slot] : 0;
+    seq_start[s] = past;
+    kv_len[s] = past + q;
+    rows += q_len[s];
+    tiles += (q + tile_rows - 1) / tile_rows;
+    if (slot >= 0) lengths[slot] = past + q;
+  }
+  if (threadIdx.x == PREPARE_THREADS - 1) {     // its runs come last: what it has summed is the total
     cu_rows[n_seqs] = rows;
     tile_cu[n_seqs] = tiles;
   }
@@ -51,7 +69,7 @@ DRYFT_API int dryft_prepare_batch(const int* seq_slot, const int* q_len, int* le
                                   int tile_rows, int* cu_rows, int* tile_cu, int* kv_len, int* seq_start, int* row_seq,
                                   int* row_slot, int* row_pos, hipStream_t stream) {
   if (tile_rows <= 0) return -1;
-  hipLaunchKernelGGL(prepare_batch_kernel, dim3(1), dim3(256), 0, stream, seq_slot, q_len, lengths, n_seqs, n_rows,
+  hipLaunchKernelGGL(prepare_batch_kernel, dim3(1), dim3(PREPARE_THREADS), 0, stream, seq_slot, q_len, lengths, n_seqs, n_rows,
                      tile_rows, cu_rows, tile_cu, kv_len, seq_start, row_seq, row_slot, row_pos);
   return DRYFT_LAUNCH_CHECK();
 }

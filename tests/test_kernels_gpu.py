@@ -670,3 +670,36 @@ def test_prepare_batch():
     assert rseq.tolist() == [0] * 70 + [1] + [2] + [3] * 130
     assert rslot.tolist() == [3] * 70 + [-1] + [1] + [5] * 130
     assert rpos.tolist() == list(range(7, 77)) + [0] + [10] + list(range(3, 133))
+
+
+@pytest.mark.parametrize("n_seqs", [1, 64, 255, 256, 257, 1000])
+def test_prepare_batch_many_sequences(n_seqs):
+    """More sequences than the kernel has threads: every thread sums a run of them; against plain prefix sums."""
+    o = ops()
+    rng = np.random.default_rng(n_seqs)
+    q = rng.integers(1, 200, size=n_seqs)
+    q[rng.random(n_seqs) < 0.5] = 1
+    slots = rng.permutation(n_seqs + 5)[:n_seqs]
+    slots[rng.random(n_seqs) < 0.2] = -1
+    past = rng.integers(0, 500, size=n_seqs + 5)
+    i32 = lambda x: torch.tensor(np.asarray(x), dtype=torch.int32, device=DEV)
+    lengths, seq_slot, q_len = i32(past), i32(slots), i32(q)
+    n_rows = int(q.sum())
+    z = lambda n: torch.full((n,), -7, dtype=torch.int32, device=DEV)
+    cu, tiles, kv, start = z(n_seqs + 1), z(n_seqs + 1), z(n_seqs), z(n_seqs)
+    rseq, rslot, rpos = z(n_rows), z(n_rows), z(n_rows)
+    o.prepare_batch(seq_slot, q_len, lengths, n_seqs, n_rows, cu, tiles, kv, start, rseq, rslot, rpos)
+    live = slots >= 0
+    want_start = np.where(live, past[np.maximum(slots, 0)], 0)
+    assert cu.tolist() == [0] + np.cumsum(q).tolist()
+    assert tiles.tolist() == [0] + np.cumsum(np.where(live, (q + 63) // 64, 0)).tolist()
+    assert start.tolist() == want_start.tolist()
+    assert kv.tolist() == (want_start + np.where(live, q, 0)).tolist()
+    new_len = past.copy()
+    new_len[slots[live]] += q[live]
+    assert lengths.tolist() == new_len.tolist()
+    seq_of_row = np.repeat(np.arange(n_seqs), q)
+    assert rseq.tolist() == seq_of_row.tolist()
+    assert rslot.tolist() == slots[seq_of_row].tolist()
+    within = np.arange(n_rows) - np.repeat(np.cumsum(q) - q, q)
+    assert rpos.tolist() == np.where(live[seq_of_row], want_start[seq_of_row] + within, 0).tolist()
