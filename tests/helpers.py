@@ -37,8 +37,16 @@ TINY_D = {
     "rope_theta": 20000.0, "rms_norm_eps": 2e-6, "tie_word_embeddings": True, "max_position_embeddings": 1024,
     "hidden_act": "silu", "attention_bias": False,
 }
+# a fifth one whose head size (40) is no multiple of 16: the matrix-core attention kernels do not take it, so
+# bfloat16 runs on the plain attention kernel like float32; three query heads on one kv head
+TINY_E = {
+    "architectures": ["Qwen3ForCausalLM"], "model_type": "qwen3", "num_hidden_layers": 2, "hidden_size": 72,
+    "num_attention_heads": 3, "num_key_value_heads": 1, "head_dim": 40, "intermediate_size": 104, "vocab_size": 300,
+    "rope_theta": 30000.0, "rms_norm_eps": 4e-6, "tie_word_embeddings": False, "max_position_embeddings": 512,
+    "hidden_act": "silu", "attention_bias": False,
+}
 TINY = {"D": (TINY_D, dict(seed=44, norm_std=0.1, std=0.04)), "A": (TINY_A, dict(seed=11, norm_std=0.0, std=0.02)), "B": (TINY_B, dict(seed=22, norm_std=0.1, std=0.02)),
-        "C": (TINY_C, dict(seed=33, norm_std=0.1, std=0.05))}
+        "C": (TINY_C, dict(seed=33, norm_std=0.1, std=0.05)), "E": (TINY_E, dict(seed=55, norm_std=0.1, std=0.05))}
 
 
 def make_model_dir(path: str, raw_config: dict, seed: int, norm_std: float = 0.0, std: float = 0.02,

@@ -92,7 +92,7 @@ def cases(tmp_path_factory):
     return out
 
 
-CASE_NAMES = ["A", "B", "C", "D", "C_sharp", "A_sharp", "B_sharp"]
+CASE_NAMES = ["A", "B", "C", "D", "E", "C_sharp", "A_sharp", "B_sharp"]
 
 
 def replay(engine, records):
@@ -236,7 +236,7 @@ def portions_trace(case):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name", ["B", "C_sharp", "A_sharp", "B_sharp", "D"])
+@pytest.mark.parametrize("name", ["B", "C_sharp", "A_sharp", "B_sharp", "D", "E"])
 def test_prompt_in_portions_beside_decoding_rows(cases, name, dtype):
     """How the tokens are cut into steps changes no logit: a prompt fed in portions, in steps that also hold
     sequences going on by one token, against the plain implementation of whole sequences."""
