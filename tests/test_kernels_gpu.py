@@ -703,3 +703,29 @@ def test_prepare_batch_many_sequences(n_seqs):
     assert rslot.tolist() == slots[seq_of_row].tolist()
     within = np.arange(n_rows) - np.repeat(np.cumsum(q) - q, q)
     assert rpos.tolist() == np.where(live[seq_of_row], want_start[seq_of_row] + within, 0).tolist()
+
+
+@pytest.mark.parametrize("D", list(range(16, 257, 16)))
+def test_attention_kernels_take_every_head_size_in_steps_of_16(D):
+    """Every head size a configuration may have in steps of 16, up to 256, through the three bfloat16 matrix-core
+    kernels and the plain one: a prompt that continues cached tokens, and one row per sequence with and without
+    splits. Three query heads to a kv head, lengths that end inside a page."""
+    for kind, tq in (("causal1", 70), ("causal0", 200), ("rows", 33), (1, 1), (3, 1)):
+        run_attention_case(kind, torch.bfloat16, 6, 2, D, [200, 70, 131], tq)
+    if D <= 128:
+        run_attention_case("causal3", torch.bfloat16, 6, 2, D, [200, 70, 131], 200)
+        run_attention_case("causal2", torch.bfloat16, 8, 2, D, [200, 70, 131], 200)
+    else:                                           # 32 rows or two heads a wave hold head sizes up to 128 only
+        for mode in (2, 3):
+            with pytest.raises(Exception, match="refuses these sizes"):
+                run_attention_case(f"causal{mode}", torch.bfloat16, 8, 2, D, [200, 70, 131], 200)
+
+
+@pytest.mark.parametrize("D", [8, 24, 40, 72, 100, 250])
+def test_plain_attention_takes_head_sizes_the_matrix_cores_do_not(D):
+    for dtype in DTYPES:
+        run_attention_case("rows", dtype, 6, 2, D, [200, 70, 131], 33)
+    with pytest.raises(Exception, match="refuses these sizes"):
+        run_attention_case("causal0", torch.bfloat16, 6, 2, D, [200, 70, 131], 70)
+    with pytest.raises(Exception, match="refuses these sizes"):
+        run_attention_case(2, torch.bfloat16, 6, 2, D, [200, 70, 131], 1)
