@@ -752,11 +752,6 @@ __global__ __launch_bounds__(128) void attn_combine_kernel(const float* __restri
   const float* ml = part_ml + ((int64_t)seq * n_heads + head) * n_splits * 2;
   const float* po = part_o + ((int64_t)seq * n_heads + head) * n_splits * head_dim;
   const bool live = seq_slot[seq] >= 0;
-  // the first splits' partial results are asked for before their weights are known: one trip to memory, not two
-  constexpr int EARLY = 16;
-  float early[EARLY];
-#pragma unroll
-  for (int s = 0; s < EARLY; ++s) early[s] = (tid < head_dim && s < n_splits) ? po[s * head_dim + tid] : 0.f;
   if (tid < WAVE) {                       // the first wave turns (m_s, l_s) into weights
     const float ms = (live && tid < n_splits) ? ml[2 * tid] : -INFINITY;
     const float ls = (live && tid < n_splits) ? ml[2 * tid + 1] : 0.f;
@@ -769,14 +764,8 @@ __global__ __launch_bounds__(128) void attn_combine_kernel(const float* __restri
   __syncthreads();
   for (int d = tid; d < head_dim; d += blockDim.x) {
     float num = 0.f;
-    if (d == tid) {                       // splits in their order, whichever way they were fetched
-#pragma unroll
-      for (int s = 0; s < EARLY; ++s)
-        if (s < n_splits) num += wgt[s] * early[s];
-      for (int s = EARLY; s < n_splits; ++s) num += wgt[s] * po[s * head_dim + d];
-    } else {
-      for (int s = 0; s < n_splits; ++s) num += wgt[s] * po[s * head_dim + d];
-    }
+#pragma unroll 8
+    for (int s = 0; s < n_splits; ++s) num += wgt[s] * po[s * head_dim + d];
     o[d] = float_to_bf16(num * inv_l);
   }
 }

@@ -29,7 +29,8 @@ __global__ void prepare_batch_kernel(const int* __restrict__ seq_slot, const int
   run_tiles[threadIdx.x] = tiles;
   __syncthreads();
   rows = tiles = 0;
-  for (int t = 0; t < (int)threadIdx.x; ++t) {
+  const int runs = (n_seqs + per - 1) / per;              // threads beyond them have summed nothing
+  for (int t = 0; t < min((int)threadIdx.x, runs); ++t) {
     rows += run_rows[t];
     tiles += run_tiles[t];
   }

@@ -31,6 +31,7 @@ from .model import DecoderModel
 from .step import SeqStep, Stepper
 
 DEFAULT_MAX_LEN = 8192
+SHORTEST_GRAPH_CONTEXT = 256       # captured decoding steps come in context ranges of 256, 512, 1,024, ... tokens
 DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32}
 
 
@@ -96,7 +97,7 @@ class Engine:
                                 max_len=self.max_len, dtype=self.dtype, device=self.device)
         self.stepper = Stepper(self.model, self.cache)
         self.use_graph = bool(use_graph)
-        self._graphs: dict[int, DecodeGraph] = {}
+        self._graphs: dict[tuple[int, int], DecodeGraph] = {}     # (batch size, context range) -> captured step
         self._sampler = Sampler()
         self._last_choice: torch.Tensor | None = None
         if verbose:
@@ -159,8 +160,9 @@ class Engine:
         """Launches one more token each and returns without waiting. ``tokens`` None: every sequence goes on
         with the token the step launched before this one chose for it, handed over on the device."""
         n = len(slots)
-        graph = self._graph_for(n)
         live = [s for s in slots if s >= 0]
+        lengths = self.cache.slots.lengths
+        graph = self._graph_for(n, max((int(lengths[s]) + 1 for s in live), default=1))
         self.cache.begin_step(live, [1] * len(live))
         if tokens is None:
             if self._last_choice is None or self._last_choice.numel() != n:
@@ -203,14 +205,22 @@ class Engine:
         uniforms = None if self._sampler.greedy else self._sampler.draw(n)
         return self._sampler.choose(logits, uniforms).tolist()
 
-    def _graph_for(self, batch: int) -> DecodeGraph | None:
+    def _graph_for(self, batch: int, context: int | None = None) -> DecodeGraph | None:
+        """The captured step for ``batch`` sequences whose longest will hold ``context`` tokens after the step
+        (default: as long as the cache allows): one graph per batch size and power-of-two range of contexts."""
         if not self.use_graph:
             return None
-        g = self._graphs.get(batch)
+        reach = self.max_len
+        if context is not None:
+            reach = SHORTEST_GRAPH_CONTEXT
+            while reach < context:
+                reach *= 2
+            reach = min(reach, self.max_len)
+        g = self._graphs.get((batch, reach))
         if g is None:
-            g = DecodeGraph(self.stepper, batch)
+            g = DecodeGraph(self.stepper, batch, reach)
             g.capture()
-            self._graphs[batch] = g
+            self._graphs[(batch, reach)] = g
         return g
 
     # ------------------------------------------------------------------ generation

@@ -4,9 +4,11 @@ The reference captures one graph per (batch bucket, length bucket) after three w
 runs on a side stream and checks a replay against eager (engine/dryft_qwen3/graphs.py:108-135,
 146-169). Here every quantity that changes from step to step (tokens, slots, positions,
 lengths, page tables) is read from device memory, so one graph per batch size serves
-every position and length. Warm runs and the capture itself run with every row marked
-dead (slot -1), which launches the same kernels but writes to no cache slot and advances
-no length.
+every position and length; the engine keeps one more per range of context lengths
+(powers of two), because how attention cuts a sequence's keys into runs is fixed when a
+graph is captured and should fit the sequences it runs on. Warm runs and the capture
+itself run with every row marked dead (slot -1), which launches the same kernels but
+writes to no cache slot and advances no length.
 """
 
 from __future__ import annotations
@@ -19,13 +21,17 @@ from .step import BatchBuffers, Stepper, make_context
 
 
 class DecodeGraph:
-    def __init__(self, stepper: Stepper, batch_size: int):
+    def __init__(self, stepper: Stepper, batch_size: int, max_kv_len: int | None = None):
+        """``max_kv_len``: the longest sequence the graph is meant for (default: the longest the cache holds). Parts
+        size their launches by it (attention: into how many runs a sequence's keys are cut); a replay on longer
+        sequences is still right, only sized for shorter ones."""
         self.stepper, self.batch = stepper, int(batch_size)
         dev = stepper.device
         self.buf = BatchBuffers(self.batch, self.batch, dev)
         self.buf.q_len.fill_(1)
+        self.max_kv_len = min(int(max_kv_len), stepper.cache.max_len) if max_kv_len else stepper.cache.max_len
         self.ctx: StepContext = make_context(self.buf, self.batch, self.batch, stepper.model.dtype, max_q_len=1,
-                                             max_tiles=self.batch, max_kv_len=stepper.cache.max_len, host=None)
+                                             max_tiles=self.batch, max_kv_len=self.max_kv_len, host=None)
         self.logits: torch.Tensor | None = None
         self.graph: torch.cuda.CUDAGraph | None = None
         # Host-side staging for tokens and slots. Steps may be launched one ahead of the host reading their

@@ -448,6 +448,21 @@ def test_steps_launched_ahead_change_nothing(cases, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+def test_decoding_across_context_ranges(cases, dtype):
+    """Captured steps come per range of context lengths (256, 512, ... tokens): a batch whose longest sequence
+    grows from 250 to 262 tokens moves from one graph to the next, and the tokens stay the plain loop's."""
+    case = cases["B"]
+    engine = case.engine(dtype, max_batch=3, max_len=512, use_graph=True)
+    prompts = [random_tokens(n, case.vocab, seed=400 + n) for n in (250, 3, 100)]
+    ours = list(engine.generate(prompts, 12))
+    check_generation(case, prompts, ours, 12, dtype)
+    assert {key for key in engine._graphs if key[0] == 3} >= {(3, 256), (3, 512)}
+    short = list(engine.generate([p[:40] for p in prompts], 5))          # back to the first range
+    check_generation(case, [p[:40] for p in prompts], short, 5, dtype)
+    assert list(engine.generate(prompts, 12)) == ours
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_graph_replay_equals_eager(cases, dtype):
     """A captured decoding step gives bit-identical logits to the same step run eagerly."""
     case = cases["B"]
