@@ -447,6 +447,26 @@ def test_steps_launched_ahead_change_nothing(cases, dtype):
     assert ahead.generate_all(prompts, 9) == plain_loop.generate_all(prompts, 9)
 
 
+def test_slots_longer_than_the_model_allows_are_refused(cases, tmp_path):
+    """`max_position_embeddings` bounds the slot length (reference: config.py:154): asking for more is an error,
+    asking for nothing gives at most that, and the replay program clamps its budget to it."""
+    from dryft_amd import Engine
+    case = cases["D"]                                            # allows 1,024 positions
+    with pytest.raises(ValueError, match="1024 positions"):
+        Engine(case.dir, dtype="float32", max_batch=2, max_len=1025)
+    engine = Engine(case.dir, dtype="float32", max_batch=1)
+    assert engine.max_len == 1024
+    del engine
+    record = {"step": 0, "entries": [{"id": "a", "tokens": case.requests["r9"], "want": [8]}], "end": ["a"]}
+    out_dir = str(tmp_path / "out")
+    proc = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", case.dir, "--dtype",
+                           "float32", "--out", out_dir, "--max-tokens", "4096"], input=json.dumps(record) + "\n",
+                          capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    got = torch.from_numpy(np.fromfile(os.path.join(out_dir, "0.f32"), dtype="<f4").reshape(1, case.vocab))
+    check_against_plain(case, {("r9", 8): got[0]}, "float32", "clamped budget")
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_decoding_across_context_ranges(cases, dtype):
     """Captured steps come per range of context lengths (256, 512, ... tokens): a batch whose longest sequence
