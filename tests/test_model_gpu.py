@@ -214,6 +214,46 @@ def test_first_tokens(cases, name, dtype):
     check_against_plain(case, got, dtype, "first tokens")
 
 
+def random_trace(case, seed, max_batch=8):
+    """Batches drawn at random, one after another: one to ``max_batch`` requests each, lengths around the edges of
+    the 64-token pages as often as anywhere, each request's last tokens (none to forty) fed one by one, logits wanted
+    at random places of the prompts (nowhere, everywhere, a few) and at most decoding steps. Requests are added to
+    ``case.requests`` under names that say seed, batch and place."""
+    rng = np.random.default_rng(seed)
+    edges = [1, 2, 63, 64, 65, 127, 128, 129, 191, 192, 193, 255, 256, 257]
+    records, step = [], 0
+    for b in range(4):
+        batch = {}
+        for i in range(int(rng.integers(1, max_batch + 1))):
+            n = int(rng.choice(edges)) if rng.random() < 0.5 else int(rng.integers(1, 260))
+            rid = f"s{seed}b{b}i{i}n{n}"
+            case.requests[rid] = random_tokens(n, case.vocab, seed=7000 + 100 * seed + 10 * b + i)
+            batch[rid] = (case.requests[rid], int(rng.integers(0, min(n, 41))))
+        for rec in trace_batches([batch]):
+            rec["step"] = step
+            step += 1
+            for e in rec["entries"]:
+                n = len(e["tokens"])
+                kind = rng.random()
+                if n > 1:                                        # a prompt: nowhere, everywhere, or a few places
+                    e["want"] = [] if kind < 0.2 else list(range(n)) if kind < 0.5 else \
+                        sorted(set(int(x) for x in rng.integers(0, n, size=3)) | {n - 1})
+                elif kind < 0.15:
+                    e["want"] = []
+            records.append(rec)
+    return records
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name,seed", [(n, 10 * i + k) for i, n in enumerate(["A_sharp", "B_sharp", "C_sharp", "D", "E", "B"])
+                                       for k in range(3)])
+def test_random_batches_against_plain(cases, name, seed, dtype):
+    case = cases[name]
+    records = random_trace(case, seed)
+    got = collect_positions(records, replay(case.engine(dtype), records))
+    check_against_plain(case, got, dtype, f"random batches, seed {seed}")
+
+
 def portions_trace(case):
     """r200 arrives in portions of 63, 2, 63, 1 and 71 tokens: one starts in the middle of a page, one is two tokens
     long, one ends exactly at a page's edge, one is a single token. Beside it r131 starts with 127 tokens and then
