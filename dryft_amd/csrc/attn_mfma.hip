@@ -288,6 +288,42 @@ __device__ __forceinline__ void stage_store_v(const PageStage<KB>& st, bf16_t* v
   }
 }
 
+// Tiles of 64 * RP rows over all sequences of the step, and the sequence and place of one of them. A sequence that
+// sits out (slot < 0) keeps its rows in cu_rows but has no tiles. tile_cu holds the prefix sums for 64-row tiles.
+template <int RP>
+__device__ __forceinline__ int count_tiles(const int* __restrict__ seq_slot, const int* __restrict__ cu_rows,
+                                           const int* __restrict__ tile_cu, int n_seqs) {
+  if (RP == 1) return tile_cu[n_seqs];
+  int n_tiles = 0;
+  for (int sq = 0; sq < n_seqs; ++sq)
+    if (seq_slot[sq] >= 0) n_tiles += (cu_rows[sq + 1] - cu_rows[sq] + 64 * RP - 1) / (64 * RP);
+  return n_tiles;
+}
+
+template <int RP>
+__device__ __forceinline__ void locate_tile(int tile, const int* __restrict__ seq_slot, const int* __restrict__ cu_rows,
+                                            const int* __restrict__ tile_cu, int n_seqs, int& seq, int& tile_in_seq) {
+  if (RP == 1) {
+    int lo = 0, hi = n_seqs;
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) >> 1;
+      if (tile_cu[mid] <= tile) lo = mid; else hi = mid;
+    }
+    while (lo + 1 < n_seqs && tile_cu[lo + 1] <= tile) ++lo;
+    seq = lo;
+    tile_in_seq = tile - tile_cu[seq];
+  } else {
+    seq = 0;
+    tile_in_seq = tile;
+    for (;;) {
+      const int cnt = seq_slot[seq] >= 0 ? (cu_rows[seq + 1] - cu_rows[seq] + 64 * RP - 1) / (64 * RP) : 0;
+      if (tile_in_seq < cnt || seq + 1 >= n_seqs) break;
+      tile_in_seq -= cnt;
+      ++seq;
+    }
+  }
+}
+
 // A wave serves U = GP * RP units: GP query heads of one kv group, each over RP tiles of 16 consecutive rows. Every
 // piece of a page that a wave reads from LDS is used for all its units, so two units halve the LDS reads per
 // matrix instruction. A workgroup's tile is 64 * RP rows.
@@ -305,15 +341,7 @@ __global__ __launch_bounds__(256, (GP * RP * KB <= 8 && KB <= 4) ? (GP * RP == 1
   constexpr bool PAIRED = GP != 1;
   const int head0 = (PAIRED ? blockIdx.y : blockIdx.x) * GP;
   const int first_tile = PAIRED ? blockIdx.x : blockIdx.y;
-  int n_tiles;                                                // tiles of TILE_ROWS rows over all sequences
-  // A sequence that sits out (slot < 0) keeps its rows in cu_rows but has no tiles, here as in tile_cu.
-  if (RP == 1) {
-    n_tiles = tile_cu[n_seqs];
-  } else {
-    n_tiles = 0;
-    for (int sq = 0; sq < n_seqs; ++sq)
-      if (seq_slot[sq] >= 0) n_tiles += (cu_rows[sq + 1] - cu_rows[sq] + TILE_ROWS - 1) / TILE_ROWS;
-  }
+  const int n_tiles = count_tiles<RP>(seq_slot, cu_rows, tile_cu, n_seqs);   // tiles of TILE_ROWS rows over all sequences
   // A tile late in a sequence sees many keys, an early one few. With pairs every workgroup takes one tile from
   // each end of the list, so all of them have about the same work.
   for (int half = 0; half < 2; ++half) {
@@ -321,25 +349,7 @@ __global__ __launch_bounds__(256, (GP * RP * KB <= 8 && KB <= 4) ? (GP * RP == 1
   const int tile = half == 0 ? n_tiles - 1 - first_tile : first_tile;
   if (tile < 0 || tile >= n_tiles || (half == 1 && tile >= n_tiles - 1 - first_tile)) continue;
   int seq, tile_in_seq;                                       // the sequence whose tiles include `tile`
-  if (RP == 1) {
-    int lo = 0, hi = n_seqs;
-    while (hi - lo > 1) {
-      const int mid = (lo + hi) >> 1;
-      if (tile_cu[mid] <= tile) lo = mid; else hi = mid;
-    }
-    while (lo + 1 < n_seqs && tile_cu[lo + 1] <= tile) ++lo;
-    seq = lo;
-    tile_in_seq = tile - tile_cu[seq];
-  } else {
-    seq = 0;
-    tile_in_seq = tile;
-    for (;;) {
-      const int cnt = seq_slot[seq] >= 0 ? (cu_rows[seq + 1] - cu_rows[seq] + TILE_ROWS - 1) / TILE_ROWS : 0;
-      if (tile_in_seq < cnt || seq + 1 >= n_seqs) break;
-      tile_in_seq -= cnt;
-      ++seq;
-    }
-  }
+  locate_tile<RP>(tile, seq_slot, cu_rows, tile_cu, n_seqs, seq, tile_in_seq);
   const int slot = seq_slot[seq];
   if (slot < 0) continue;                                     // the whole workgroup skips the tile together
   __syncthreads();                                            // the previous tile's pages are no longer read
@@ -470,6 +480,198 @@ __global__ __launch_bounds__(256, (GP * RP * KB <= 8 && KB <= 4) ? (GP * RP == 1
     }
   }
   }  // the two tiles of the workgroup
+}
+
+// ---------------------------------------------------------------------------------------------------
+// The same kernel for head size 128 with one head per wave, with the pages going from the cache straight into
+// LDS (global_load_lds_dwordx4: 16 bytes a lane, no registers in between and nothing for the waves to store;
+// about a quarter of the staged kernel's time goes into that copying). One instruction fills 1,024 contiguous
+// bytes of LDS, lane l at byte 16 l. Which 16 bytes of the page a lane fetches is free, and that choice
+// swizzles the layout so that operand reads meet no bank twice without padding:
+//   keys   [64 positions][16 pieces of 16 bytes]: piece p of row r sits at place p ^ (r % 16);
+//   values [128 features][8 pieces]:              piece p of row d sits at place p ^ ((d / 2) % 8).
+// The compiler does not know that these loads write LDS (it would otherwise wait for all of them before every
+// LDS read that follows one): each wave waits for its own (s_waitcnt vmcnt(0)) before the barrier after which
+// the page is read. The LDS address of an instruction goes through M0.
+#define DIRECT_D 128
+#define DIRECT_PAGE_BYTES (PAGE_TOKENS * DIRECT_D * 2)
+
+__device__ __forceinline__ void load_to_lds16(const bf16_t* src, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_base), "v"(src) : "memory");
+}
+
+// s_waitcnt vmcnt(0), leaving the other counters alone (vmcnt in bits 3:0 and 15:14, expcnt 6:4, lgkmcnt 11:8). As a
+// builtin rather than text, so that the compiler's own count of loads in flight takes it into account: it would
+// otherwise wait again, inside the loop, for the query loads of the prologue, and with them for the page on its way.
+__device__ __forceinline__ void wait_direct_loads() {
+  __builtin_amdgcn_s_waitcnt(0x0f70);
+  asm volatile("" ::: "memory");
+}
+
+// A wave's quarter of a page of keys, or of values: four instructions of 1,024 bytes each.
+__device__ __forceinline__ void direct_page_k(const bf16_t* __restrict__ k_page, uint32_t lds_base) {
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE), lane = threadIdx.x % WAVE;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int chunk = 4 * i + wave;                          // rows 4 chunk .. 4 chunk + 3
+    const int row = 4 * chunk + lane / 16, place = lane % 16;
+    load_to_lds16(k_page + row * DIRECT_D + ((place ^ (row & 15)) << 3), lds_base + chunk * 1024);
+  }
+}
+
+__device__ __forceinline__ void direct_page_v(const bf16_t* __restrict__ v_page, uint32_t lds_base) {
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE), lane = threadIdx.x % WAVE;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int chunk = 4 * i + wave;                          // rows 8 chunk .. 8 chunk + 7
+    const int row = 8 * chunk + lane / 8, place = lane % 8;
+    load_to_lds16(v_page + row * PAGE_TOKENS + ((place ^ ((row >> 1) & 7)) << 3), lds_base + chunk * 1024);
+  }
+}
+
+// RP tiles of 16 consecutive rows per wave; a workgroup's tile is 64 * RP rows. Grid: (heads, tiles), the
+// tiles with the most pages first. With 16 rows a wave, keys and values have one buffer each and a page takes two
+// barriers (the values arrive during the first product and the softmax, the next keys during the second
+// product): 32 KB of LDS and under 128 registers put four workgroups on a compute unit, which covers more
+// latency than a second buffer would (0.67 against 0.63 PFLOP/s at 3,000 positions, 0.76 against 0.70 at 4,096,
+// the same at 2,048). With 32 rows a wave the registers allow two workgroups a unit anyway, so both have two
+// buffers and a page takes one barrier.
+template <int RP>
+__global__ __launch_bounds__(256, RP == 1 ? 4 : 2) void attn_causal_direct_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
+    const int* __restrict__ page_table, int max_pages, const int* __restrict__ seq_slot,
+    const int* __restrict__ cu_rows, const int* __restrict__ tile_cu, const int* __restrict__ seq_start, int n_seqs,
+    bf16_t* __restrict__ out, int n_heads, int n_kv, float scale, int window) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  constexpr int KB = DIRECT_D / 32, TILE_ROWS = 64 * RP, WAVE_ROWS = 16 * RP, head_dim = DIRECT_D;
+  constexpr bool TWO = RP != 1;                               // two buffers each for keys and values
+  const int head = blockIdx.x;
+  const int n_tiles = count_tiles<RP>(seq_slot, cu_rows, tile_cu, n_seqs);
+  const int tile = n_tiles - 1 - (int)blockIdx.y;
+  if (tile < 0) return;
+  int seq, tile_in_seq;
+  locate_tile<RP>(tile, seq_slot, cu_rows, tile_cu, n_seqs, seq, tile_in_seq);
+  const int slot = seq_slot[seq];
+  if (slot < 0) return;
+  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE, c = lane % 16, g = lane / 16;
+  const int q_len = cu_rows[seq + 1] - cu_rows[seq];
+  const int tile_first = tile_in_seq * TILE_ROWS;
+  const int wave_first = tile_first + WAVE_ROWS * wave;
+  const int wave_rows = max(0, min(WAVE_ROWS, q_len - wave_first));
+  const int pos_tile = seq_start[seq] + tile_first;
+  const int pos_wave = pos_tile + WAVE_ROWS * wave;
+  int rows[RP], pos0[RP], pos_row[RP], lo_row[RP];
+  bool row_valid[RP];
+  int64_t row[RP];
+  RowBlock<KB> st[RP];
+#pragma unroll
+  for (int rt = 0; rt < RP; ++rt) {
+    const int first = wave_first + 16 * rt;
+    rows[rt] = max(0, min(16, q_len - first));
+    row_valid[rt] = c < rows[rt];
+    row[rt] = (int64_t)cu_rows[seq] + first + c;
+    pos0[rt] = pos_wave + 16 * rt;
+    pos_row[rt] = row_valid[rt] ? pos0[rt] + c : -1;
+    lo_row[rt] = window > 0 ? max(0, pos_row[rt] - window + 1) : 0;
+    init_rows<KB>(st[rt], q + (row[rt] * n_heads + head) * head_dim, row_valid[rt], head_dim);
+  }
+  const int kvh = head / (n_heads / n_kv);
+  const int lo_wave = window > 0 ? max(0, pos_wave - window + 1) : 0;
+  const int hi_wave = pos_wave + wave_rows - 1;
+  const int lo_tile = window > 0 ? max(0, pos_tile - window + 1) : 0;
+  const int hi_tile = pos_tile + min(TILE_ROWS, q_len - tile_first) - 1;
+  const float scale_log2 = scale * 1.44269504088896340736f;
+  const int64_t page_elems = (int64_t)PAGE_TOKENS * head_dim;
+  const int* table = page_table + (int64_t)slot * max_pages;
+  const int pg_first = lo_tile / PAGE_TOKENS, pg_last = hi_tile / PAGE_TOKENS;
+  // LDS: one or two pages of keys, then as many of values
+  const uint32_t lds0 = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)lds_raw);
+  const uint32_t v_lds0 = lds0 + (TWO ? 2 : 1) * DIRECT_PAGE_BYTES;
+  // where this lane's operands sit within a page: keys (16 t + c, piece 4 kb + g), values (16 dt + c, piece 4 h + g)
+  int k_at[KB], v_at[2];
+#pragma unroll
+  for (int kb = 0; kb < KB; ++kb) k_at[kb] = c * (2 * DIRECT_D) + (((4 * kb + g) ^ c) << 4);
+#pragma unroll
+  for (int h = 0; h < 2; ++h) v_at[h] = c * (2 * PAGE_TOKENS) + (((4 * h + g) ^ (c >> 1)) << 4);
+  int page = table[pg_first];
+  if (page >= 0) {
+    direct_page_k(k_pages + ((int64_t)page * n_kv + kvh) * page_elems, lds0);
+    if (TWO) direct_page_v(v_pages + ((int64_t)page * n_kv + kvh) * page_elems, v_lds0);
+  }
+  for (int pg = pg_first; pg <= pg_last; ++pg) {
+    const int buf = TWO ? (pg - pg_first) & 1 : 0;
+    const unsigned char* k_lds = lds_raw + buf * DIRECT_PAGE_BYTES;
+    const unsigned char* v_lds = lds_raw + ((TWO ? 2 : 1) + buf) * DIRECT_PAGE_BYTES;
+    wait_direct_loads();
+    __syncthreads();   // this page's keys are in LDS; every wave is done with the page before and the buffers it used
+    const int page_now = page;
+    page = pg < pg_last ? table[pg + 1] : -1;
+    if (!TWO && page_now >= 0) direct_page_v(v_pages + ((int64_t)page_now * n_kv + kvh) * page_elems, v_lds0);
+    if (TWO && page >= 0) {
+      direct_page_k(k_pages + ((int64_t)page * n_kv + kvh) * page_elems, lds0 + (buf ^ 1) * DIRECT_PAGE_BYTES);
+      direct_page_v(v_pages + ((int64_t)page * n_kv + kvh) * page_elems, v_lds0 + (buf ^ 1) * DIRECT_PAGE_BYTES);
+    }
+    const int key0 = pg * PAGE_TOKENS;
+    const bool sees = page_now >= 0 && key0 <= hi_wave && key0 + PAGE_TOKENS > lo_wave;   // some row sees some key
+    bf16x8 p[RP][2];
+    if (sees) {
+      float alpha[RP];
+      bool moved[RP];
+      f32x4 s[RP][4];
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+#pragma unroll
+        for (int u = 0; u < RP; ++u) s[u][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb) {
+          const bf16x8 a = *(const bf16x8*)(k_lds + 16 * t * (2 * DIRECT_D) + k_at[kb]);
+#pragma unroll
+          for (int u = 0; u < RP; ++u) s[u][t] = MFMA16(a, st[u].q[kb], s[u][t]);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < RP; ++u) {
+        const bool masked = key0 + PAGE_TOKENS - 1 > pos0[u] || rows[u] < 16 ||
+                            (window > 0 && key0 < pos0[u] + 15 - window + 1);
+        alpha[u] = masked ? page_softmax<KB, true>(st[u], s[u], p[u], scale_log2, key0, lo_row[u], pos_row[u], moved[u])
+                          : page_softmax<KB, false>(st[u], s[u], p[u], scale_log2, key0, lo_row[u], pos_row[u], moved[u]);
+      }
+#pragma unroll
+      for (int u = 0; u < RP; ++u)
+        if (moved[u]) {                                       // rare once the maxima have settled
+#pragma unroll
+          for (int dt = 0; dt < 2 * KB; ++dt) st[u].o[dt] *= alpha[u];
+        }
+    }
+    if (!TWO) {
+      wait_direct_loads();
+      __syncthreads();                                       // the values are in LDS; every wave is done with the keys
+      if (page >= 0) direct_page_k(k_pages + ((int64_t)page * n_kv + kvh) * page_elems, lds0);
+    }
+    if (sees) {
+#pragma unroll
+      for (int dt = 0; dt < 2 * KB; ++dt)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          const bf16x8 a = *(const bf16x8*)(v_lds + 16 * dt * (2 * PAGE_TOKENS) + v_at[h]);
+#pragma unroll
+          for (int u = 0; u < RP; ++u) st[u].o[dt] = MFMA16(a, p[u][h], st[u].o[dt]);
+        }
+    }
+  }
+  float row_l[RP];
+#pragma unroll
+  for (int u = 0; u < RP; ++u) row_l[u] = row_sum<KB>(st[u]);
+#pragma unroll
+  for (int u = 0; u < RP; ++u) {
+    if (!row_valid[u]) continue;
+    const float inv = 1.f / row_l[u];
+    bf16_t* o = out + (row[u] * n_heads + head) * head_dim;
+#pragma unroll
+    for (int dt = 0; dt < 2 * KB; ++dt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) o[16 * dt + 4 * g + i] = float_to_bf16(st[u].o[dt][i] * inv);
+  }
 }
 
 // ---------------------------------------------------------------------------------------------------
@@ -818,8 +1020,24 @@ static int launch_causal(const void* q, const void* k_pages, const void* v_pages
   return DRYFT_LAUNCH_CHECK();
 }
 
+template <int RP>
+static int launch_causal_direct(const void* q, const void* k_pages, const void* v_pages, const int* page_table,
+                                int max_pages, const int* seq_slot, const int* cu_rows, const int* tile_cu,
+                                const int* seq_start, int n_seqs, int max_tiles, void* out, int n_heads, int n_kv,
+                                float scale, int window, hipStream_t stream) {
+  // max_tiles bounds the 64-row tiles of the sequences that take part; a sequence with t of them has ceil(t / RP)
+  dim3 grid(n_heads, (max_tiles + (RP - 1) * (n_seqs + 1)) / RP), block(256);
+  if (grid.y > 65535) return -1;
+  const size_t lds = (size_t)(RP == 1 ? 2 : 4) * DIRECT_PAGE_BYTES;
+  hipLaunchKernelGGL(attn_causal_direct_kernel<RP>, grid, block, lds, stream, (const bf16_t*)q, (const bf16_t*)k_pages,
+                     (const bf16_t*)v_pages, page_table, max_pages, seq_slot, cu_rows, tile_cu, seq_start, n_seqs,
+                     (bf16_t*)out, n_heads, n_kv, scale, window);
+  return DRYFT_LAUNCH_CHECK();
+}
+
 // mode: 0 = chosen here; 1 = one head and 16 rows per wave; 2 = two heads of a kv group per wave (even groups,
-// head_dim <= 128); 3 = one head and 32 rows per wave (head_dim <= 128)
+// head_dim <= 128); 3 = one head and 32 rows per wave (head_dim <= 128). At head size 128, modes 1 and 3 bring
+// the pages straight into LDS; 5 and 7 are 1 and 3 with the pages staged through registers, as at other sizes.
 DRYFT_API int dryft_attn_causal_bf16(const void* q, const void* k_pages, const void* v_pages, const int* page_table,
                                      int max_pages, const int* seq_slot, const int* cu_rows, const int* tile_cu,
                                      const int* seq_start, int n_seqs, int max_tiles, void* out, int n_heads,
@@ -827,19 +1045,32 @@ DRYFT_API int dryft_attn_causal_bf16(const void* q, const void* k_pages, const v
   if (n_seqs <= 0 || max_tiles <= 0) return 0;
   if (!head_shape_ok(n_heads, n_kv, head_dim)) return -1;
   const int group = n_heads / n_kv;
+  const bool staged = mode == 5 || mode == 7;
+  if (staged) mode -= 4;
   if (mode < 0 || mode > 3 || (mode == 2 && (group % 2 || head_dim > 128)) || (mode == 3 && head_dim > 128)) return -1;
   if (mode == 0) {
     // Two units per wave (twice the rows of one head, or two heads of a kv group) use every piece of a page that
     // is read from LDS twice, and LDS reads are what the kernel waits for most; they also halve the number of
     // workgroups, so they pay once there are still four for every compute unit. Measured on Qwen3-4B's heads,
-    // one sequence, PFLOP/s with 16 rows / 32 rows / two heads per wave: 0.46 / 0.40 / 0.34 at 2,048 positions,
-    // 0.55 / 0.53 / 0.45 at 3,000, 0.59 / 0.72 / 0.62 at 4,096, 0.63 / 0.77 / 0.69 at 8,192, 0.71 / 0.92 / 0.78 at
-    // 30,000. (Two heads per wave stay available as mode 2; nothing chooses them.)
+    // one sequence, PFLOP/s with 16 rows / 32 rows / two heads per wave, pages staged through registers: 0.46 /
+    // 0.40 / 0.34 at 2,048 positions, 0.55 / 0.53 / 0.45 at 3,000, 0.59 / 0.72 / 0.62 at 4,096, 0.63 / 0.77 / 0.69 at
+    // 8,192, 0.71 / 0.92 / 0.78 at 30,000; with the pages straight into LDS (head size 128), 16 / 32 rows: 0.56 /
+    // 0.50, 0.66 / 0.59, 0.72 / 0.76, 0.77 / 0.82, 0.89 / 0.99. (Two heads per wave stay available as mode 2;
+    // nothing chooses them.)
     mode = head_dim <= 128 && (int64_t)((max_tiles + 1) / 2) * n_heads >= 1024 ? 3 : 1;
   }
 #define CAUSAL(GPV, RPV)                                                                                          \
   return launch_causal<GPV, RPV>(q, k_pages, v_pages, page_table, max_pages, seq_slot, cu_rows, tile_cu, seq_start, \
                                  n_seqs, max_tiles, out, n_heads, n_kv, head_dim, scale, window, stream)
+  if (head_dim == DIRECT_D && !staged && mode != 2) {
+    const bool aligned = (((uintptr_t)k_pages | (uintptr_t)v_pages) & 15) == 0;
+    if (aligned && mode == 3)
+      return launch_causal_direct<2>(q, k_pages, v_pages, page_table, max_pages, seq_slot, cu_rows, tile_cu, seq_start,
+                                     n_seqs, max_tiles, out, n_heads, n_kv, scale, window, stream);
+    if (aligned)
+      return launch_causal_direct<1>(q, k_pages, v_pages, page_table, max_pages, seq_slot, cu_rows, tile_cu, seq_start,
+                                     n_seqs, max_tiles, out, n_heads, n_kv, scale, window, stream);
+  }
   if (mode == 2) CAUSAL(2, 1);
   if (mode == 3) CAUSAL(1, 2);
   CAUSAL(1, 1);

@@ -261,7 +261,9 @@ def attn_causal_bf16(q, k_pages, v_pages, page_table, seq_slot, cu_rows, tile_cu
                      max_tiles: int, out, n_heads: int, n_kv: int, head_dim: int, scale: float, window: int,
                      mode: int = 0) -> None:
     """Causal attention of steps with many rows per sequence. ``mode``: 0 lets the library choose how much a wave
-    takes; 1 = one head and 16 rows, 2 = two heads of a kv group, 3 = one head and 32 rows."""
+    takes; 1 = one head and 16 rows, 2 = two heads of a kv group, 3 = one head and 32 rows. At head size 128, 1 and
+    3 bring the pages straight into LDS; 5 and 7 are 1 and 3 with the pages staged through registers, as at every
+    other head size."""
     _gpu(q, "q", torch.bfloat16)
     _gpu(out, "out", torch.bfloat16)
     _require(q.is_contiguous() and out.is_contiguous() and out.numel() == q.numel(), "attn_causal: q and out contiguous")

@@ -247,9 +247,11 @@ CASES = [  # n_heads, n_kv, D, lengths (cached tokens incl. the rows'), q rows p
 ]
 
 
-def run_attention_case(kind, dtype, n_heads, n_kv, D, lengths, tq, window=None, seed=0, misaligned=False, dead=()):
+def run_attention_case(kind, dtype, n_heads, n_kv, D, lengths, tq, window=None, seed=0, misaligned=False, dead=(),
+                       drop_pages_behind_window=False):
     """``dead``: sequences that sit the step out (slot -1). They keep their rows, which every kernel leaves at
-    zero (the tiled prompt kernel by never visiting them), and have no tiles."""
+    zero (the tiled prompt kernel by never visiting them), and have no tiles. ``drop_pages_behind_window``: pages
+    that no row of the step can see any more are gone from the page table (-1), as in a windowed cache."""
     torch.manual_seed(seed + D + len(lengths))
     B, L = len(lengths), max(lengths)
     n_slots, n_pages = B + 2, sum((n + 63) // 64 for n in lengths) + 3
@@ -269,6 +271,9 @@ def run_attention_case(kind, dtype, n_heads, n_kv, D, lengths, tq, window=None, 
         q_pos[b] = -1                                            # the reference leaves these rows at zero
     want = attention_ref(q.float(), k.float(), v.float(), lengths, q_pos, scale, window)
     k_pages, v_pages, table, slots = build_pages(k, v, lengths, n_pages, n_slots, seed=seed, poison=1e4)
+    if drop_pages_behind_window:
+        for b, (n, ql) in enumerate(zip(lengths, q_lens)):
+            table[slots[b], : max(0, n - ql - window + 1) // 64] = -1
     slots = [-1 if b in dead else s for b, s in enumerate(slots)]
     rows = sum(q_lens)
     q_packed = torch.cat([q[b, :ql] for b, ql in enumerate(q_lens)]).contiguous()
@@ -328,7 +333,12 @@ CAUSAL_CASES = CASES + [      # many rows: several tiles per sequence, sequences
 ]
 
 
-@pytest.mark.parametrize("mode", [0, 1, 2, 3])      # chosen by the kernel; 16 rows; two heads; 32 rows a wave
+# chosen by the kernel; 16 rows; two heads; 32 rows a wave; 16 and 32 rows with the pages staged through registers
+# also at head size 128, where 1 and 3 bring them straight into LDS
+CAUSAL_MODES = [0, 1, 2, 3, 5, 7]
+
+
+@pytest.mark.parametrize("mode", CAUSAL_MODES)
 @pytest.mark.parametrize("case", CAUSAL_CASES)
 def test_attn_causal_bf16(case, mode):
     if mode == 2 and (case[0] // case[1]) % 2:
@@ -343,7 +353,7 @@ DEAD_CASES = [((8, 2, 32, [1, 200, 330, 150, 70], 330), (0, 2)),
               ((32, 8, 128, [300, 260, 1, 129], 300), (0, 2, 3))]
 
 
-@pytest.mark.parametrize("mode", [0, 1, 2, 3])
+@pytest.mark.parametrize("mode", CAUSAL_MODES)
 @pytest.mark.parametrize("case,dead", DEAD_CASES)
 def test_attn_causal_bf16_with_sequences_that_sit_out(case, dead, mode):
     run_attention_case(f"causal{mode}", torch.bfloat16, *case, dead=dead)
@@ -423,12 +433,17 @@ def test_attn_decode_fused_equals_the_two_kernels(n_heads, n_kv, D, splits, wind
     assert torch.equal(k3, k1) and torch.equal(v3, v1) and torch.equal(out3, out2)
 
 
-@pytest.mark.parametrize("kind", ["rows", "causal1", "causal2", "causal3", 3])
+@pytest.mark.parametrize("kind", ["rows", "causal1", "causal2", "causal3", "causal5", "causal7", 3])
 def test_attention_window(kind):
     tq = 1 if kind == 3 else 90
     run_attention_case(kind, torch.bfloat16, 8, 2, 32, [200, 70, 130], tq, window=70)
     if kind == "rows":
         run_attention_case(kind, torch.float32, 8, 2, 32, [200, 70, 130], tq, window=70)
+    # head size 128, windows shorter and longer than a page, rows that continue cached tokens, and the pages that
+    # no row sees any more taken out of the table
+    for window, drop in ((70, False), (70, True), (40, True), (200, True)):
+        run_attention_case(kind, torch.bfloat16, 8, 2, 128, [700, 330, 129], 1 if kind == 3 else 150, window=window,
+                           drop_pages_behind_window=drop)
 
 
 # -------------------------------------------------------------------------------------------- gemm
