@@ -496,8 +496,9 @@ __global__ __launch_bounds__(256, (GP * RP * KB <= 8 && KB <= 4) ? (GP * RP == 1
 #define DIRECT_D 128
 #define DIRECT_PAGE_BYTES (PAGE_TOKENS * DIRECT_D * 2)
 
-__device__ __forceinline__ void load_to_lds16(const bf16_t* src, uint32_t lds_base) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_base), "v"(src) : "memory");
+// 16 bytes from base + offset (a base the whole wave shares, an offset per lane) to LDS byte lds_base + 16 * lane
+__device__ __forceinline__ void load_to_lds16(const void* base, uint32_t offset, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_base), "v"(offset), "s"(base) : "memory");
 }
 
 // s_waitcnt vmcnt(0), leaving the other counters alone (vmcnt in bits 3:0 and 15:14, expcnt 6:4, lgkmcnt 11:8). As a
@@ -508,25 +509,26 @@ __device__ __forceinline__ void wait_direct_loads() {
   asm volatile("" ::: "memory");
 }
 
-// A wave's quarter of a page of keys, or of values: four instructions of 1,024 bytes each.
-__device__ __forceinline__ void direct_page_k(const bf16_t* __restrict__ k_page, uint32_t lds_base) {
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE), lane = threadIdx.x % WAVE;
+// A wave's quarter of a page of keys or of values: a page is 16 KB, an instruction moves 1 KB, and wave w takes the
+// pieces of 1 KB number w, 4 + w, 8 + w and 12 + w. They are 4,096 bytes apart in the page and in LDS, and the
+// swizzle repeats with that period (16 rows of keys, 32 rows of values), so one offset per lane serves all four:
+// where the lane reads within the first of them (`lane_offset`); `lds_wave` is the LDS address of the page's
+// buffer plus 1,024 w. Base addresses are the wave's, in scalar registers: no vector arithmetic per page.
+__device__ __forceinline__ void direct_page(const bf16_t* page, uint32_t lane_offset, uint32_t lds_wave) {
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int chunk = 4 * i + wave;                          // rows 4 chunk .. 4 chunk + 3
-    const int row = 4 * chunk + lane / 16, place = lane % 16;
-    load_to_lds16(k_page + row * DIRECT_D + ((place ^ (row & 15)) << 3), lds_base + chunk * 1024);
-  }
+  for (int i = 0; i < 4; ++i) load_to_lds16((const unsigned char*)page + 4096 * i, lane_offset, lds_wave + 4096 * i);
 }
 
-__device__ __forceinline__ void direct_page_v(const bf16_t* __restrict__ v_page, uint32_t lds_base) {
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE), lane = threadIdx.x % WAVE;
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int chunk = 4 * i + wave;                          // rows 8 chunk .. 8 chunk + 7
-    const int row = 8 * chunk + lane / 8, place = lane % 8;
-    load_to_lds16(v_page + row * PAGE_TOKENS + ((place ^ ((row >> 1) & 7)) << 3), lds_base + chunk * 1024);
-  }
+// Where a lane reads within its wave's first piece of a page of keys: row 4 w + lane / 16 of 256 bytes, and the
+// 16-byte piece that belongs at place lane % 16 of that row; of values: row 8 w + lane / 8 of 128 bytes, place lane % 8.
+__device__ __forceinline__ uint32_t direct_offset_k(int wave, int lane) {
+  const int row = 4 * wave + lane / 16, place = lane % 16;
+  return row * (2 * DIRECT_D) + ((place ^ (row & 15)) << 4);
+}
+
+__device__ __forceinline__ uint32_t direct_offset_v(int wave, int lane) {
+  const int row = 8 * wave + lane / 8, place = lane % 8;
+  return row * (2 * PAGE_TOKENS) + ((place ^ ((row >> 1) & 7)) << 4);
 }
 
 // RP tiles of 16 consecutive rows per wave; a workgroup's tile is 64 * RP rows. Grid: (heads, tiles), the
@@ -584,9 +586,10 @@ __global__ __launch_bounds__(256, RP == 1 ? 4 : 2) void attn_causal_direct_kerne
   const int64_t page_elems = (int64_t)PAGE_TOKENS * head_dim;
   const int* table = page_table + (int64_t)slot * max_pages;
   const int pg_first = lo_tile / PAGE_TOKENS, pg_last = hi_tile / PAGE_TOKENS;
-  // LDS: one or two pages of keys, then as many of values
-  const uint32_t lds0 = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)lds_raw);
+  // LDS: one or two pages of keys, then as many of values; these are the addresses of this wave's first piece
+  const uint32_t lds0 = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)lds_raw + 1024 * wave);
   const uint32_t v_lds0 = lds0 + (TWO ? 2 : 1) * DIRECT_PAGE_BYTES;
+  const uint32_t k_from = direct_offset_k(wave, lane), v_from = direct_offset_v(wave, lane);
   // where this lane's operands sit within a page: keys (16 t + c, piece 4 kb + g), values (16 dt + c, piece 4 h + g)
   int k_at[KB], v_at[2];
 #pragma unroll
@@ -595,8 +598,8 @@ __global__ __launch_bounds__(256, RP == 1 ? 4 : 2) void attn_causal_direct_kerne
   for (int h = 0; h < 2; ++h) v_at[h] = c * (2 * PAGE_TOKENS) + (((4 * h + g) ^ (c >> 1)) << 4);
   int page = table[pg_first];
   if (page >= 0) {
-    direct_page_k(k_pages + ((int64_t)page * n_kv + kvh) * page_elems, lds0);
-    if (TWO) direct_page_v(v_pages + ((int64_t)page * n_kv + kvh) * page_elems, v_lds0);
+    direct_page(k_pages + ((int64_t)page * n_kv + kvh) * page_elems, k_from, lds0);
+    if (TWO) direct_page(v_pages + ((int64_t)page * n_kv + kvh) * page_elems, v_from, v_lds0);
   }
   for (int pg = pg_first; pg <= pg_last; ++pg) {
     const int buf = TWO ? (pg - pg_first) & 1 : 0;
@@ -606,10 +609,10 @@ __global__ __launch_bounds__(256, RP == 1 ? 4 : 2) void attn_causal_direct_kerne
     __syncthreads();   // this page's keys are in LDS; every wave is done with the page before and the buffers it used
     const int page_now = page;
     page = pg < pg_last ? table[pg + 1] : -1;
-    if (!TWO && page_now >= 0) direct_page_v(v_pages + ((int64_t)page_now * n_kv + kvh) * page_elems, v_lds0);
+    if (!TWO && page_now >= 0) direct_page(v_pages + ((int64_t)page_now * n_kv + kvh) * page_elems, v_from, v_lds0);
     if (TWO && page >= 0) {
-      direct_page_k(k_pages + ((int64_t)page * n_kv + kvh) * page_elems, lds0 + (buf ^ 1) * DIRECT_PAGE_BYTES);
-      direct_page_v(v_pages + ((int64_t)page * n_kv + kvh) * page_elems, v_lds0 + (buf ^ 1) * DIRECT_PAGE_BYTES);
+      direct_page(k_pages + ((int64_t)page * n_kv + kvh) * page_elems, k_from, lds0 + (buf ^ 1) * DIRECT_PAGE_BYTES);
+      direct_page(v_pages + ((int64_t)page * n_kv + kvh) * page_elems, v_from, v_lds0 + (buf ^ 1) * DIRECT_PAGE_BYTES);
     }
     const int key0 = pg * PAGE_TOKENS;
     const bool sees = page_now >= 0 && key0 <= hi_wave && key0 + PAGE_TOKENS > lo_wave;   // some row sees some key
@@ -646,7 +649,7 @@ __global__ __launch_bounds__(256, RP == 1 ? 4 : 2) void attn_causal_direct_kerne
     if (!TWO) {
       wait_direct_loads();
       __syncthreads();                                       // the values are in LDS; every wave is done with the keys
-      if (page >= 0) direct_page_k(k_pages + ((int64_t)page * n_kv + kvh) * page_elems, lds0);
+      if (page >= 0) direct_page(k_pages + ((int64_t)page * n_kv + kvh) * page_elems, k_from, lds0);
     }
     if (sees) {
 #pragma unroll
@@ -1048,27 +1051,29 @@ DRYFT_API int dryft_attn_causal_bf16(const void* q, const void* k_pages, const v
   const bool staged = mode == 5 || mode == 7;
   if (staged) mode -= 4;
   if (mode < 0 || mode > 3 || (mode == 2 && (group % 2 || head_dim > 128)) || (mode == 3 && head_dim > 128)) return -1;
+  const bool direct_ok = head_dim == DIRECT_D && (((uintptr_t)k_pages | (uintptr_t)v_pages) & 15) == 0;
   if (mode == 0) {
     // Two units per wave (twice the rows of one head, or two heads of a kv group) use every piece of a page that
-    // is read from LDS twice, and LDS reads are what the kernel waits for most; they also halve the number of
-    // workgroups, so they pay once there are still four for every compute unit. Measured on Qwen3-4B's heads,
-    // one sequence, PFLOP/s with 16 rows / 32 rows / two heads per wave, pages staged through registers: 0.46 /
-    // 0.40 / 0.34 at 2,048 positions, 0.55 / 0.53 / 0.45 at 3,000, 0.59 / 0.72 / 0.62 at 4,096, 0.63 / 0.77 / 0.69 at
-    // 8,192, 0.71 / 0.92 / 0.78 at 30,000; with the pages straight into LDS (head size 128), 16 / 32 rows: 0.56 /
-    // 0.50, 0.66 / 0.59, 0.72 / 0.76, 0.77 / 0.82, 0.89 / 0.99. (Two heads per wave stay available as mode 2;
-    // nothing chooses them.)
-    mode = head_dim <= 128 && (int64_t)((max_tiles + 1) / 2) * n_heads >= 1024 ? 3 : 1;
+    // is read from LDS twice; they also halve the number of workgroups, so they need four of them for every
+    // compute unit. Measured on Qwen3-4B's heads, PFLOP/s with 16 rows / 32 rows / two heads per wave, pages
+    // staged through registers, one sequence: 0.46 / 0.40 / 0.34 at 2,048 positions, 0.55 / 0.53 / 0.45 at 3,000,
+    // 0.59 / 0.72 / 0.62 at 4,096, 0.63 / 0.77 / 0.69 at 8,192, 0.71 / 0.92 / 0.78 at 30,000; eight sequences of 2,048:
+    // 0.58 / 0.67. With the pages straight into LDS, 16 rows a wave put four workgroups on a compute unit and stay
+    // ahead while sequences are short: 16 / 32 rows a wave 0.57 / 0.51 at 2,048 positions, 0.71 / 0.62 at 3,000,
+    // 0.82 / 0.80 at 4,096, 0.84 / 0.88 at 8,192, 1.00 / 1.07 at 30,000; eight sequences of 2,048: 0.84 / 0.75, two of
+    // 4,096: 0.93 / 0.98. (Two heads per wave stay available as mode 2; nothing chooses them.)
+    const bool enough = (int64_t)((max_tiles + 1) / 2) * n_heads >= 1024;
+    const bool long_ones = (int64_t)max_tiles >= 64 * (int64_t)n_seqs;          // 4,096 rows a sequence on average
+    mode = head_dim <= 128 && enough && (!direct_ok || long_ones) ? 3 : 1;
   }
 #define CAUSAL(GPV, RPV)                                                                                          \
   return launch_causal<GPV, RPV>(q, k_pages, v_pages, page_table, max_pages, seq_slot, cu_rows, tile_cu, seq_start, \
                                  n_seqs, max_tiles, out, n_heads, n_kv, head_dim, scale, window, stream)
-  if (head_dim == DIRECT_D && !staged && mode != 2) {
-    const bool aligned = (((uintptr_t)k_pages | (uintptr_t)v_pages) & 15) == 0;
-    if (aligned && mode == 3)
+  if (direct_ok && !staged && mode != 2) {
+    if (mode == 3)
       return launch_causal_direct<2>(q, k_pages, v_pages, page_table, max_pages, seq_slot, cu_rows, tile_cu, seq_start,
                                      n_seqs, max_tiles, out, n_heads, n_kv, scale, window, stream);
-    if (aligned)
-      return launch_causal_direct<1>(q, k_pages, v_pages, page_table, max_pages, seq_slot, cu_rows, tile_cu, seq_start,
+    return launch_causal_direct<1>(q, k_pages, v_pages, page_table, max_pages, seq_slot, cu_rows, tile_cu, seq_start,
                                      n_seqs, max_tiles, out, n_heads, n_kv, scale, window, stream);
   }
   if (mode == 2) CAUSAL(2, 1);
