@@ -9,6 +9,7 @@ agent/bench.py:180-192).
     python -m dryft_amd make-model --preset tiny-a --weight-seed 1 --out DIR
     python -m dryft_amd bench --preset qwen3-4b --workload b8,8,2048,64
     python -m dryft_amd profile --preset qwen3-4b --batch 8 --prompt-len 2048 --steps 8
+    python -m dryft_amd attention --shapes 1x2048,8x2048 --modes 1,3,5,7
     python -m dryft_amd replay --model DIR --dtype float32 --out DIR --max-tokens 4096 < steps.jsonl
     python -m dryft_amd build [names...]
 """
@@ -210,6 +211,53 @@ def cmd_profile(args) -> int:
     return 0
 
 
+def cmd_attention(args) -> int:
+    """Times the bfloat16 prompt-attention kernel alone: for each ``BxL`` (B sequences of L new positions each, nothing
+    cached before them) and each way of running it (``ops.attn_causal_bf16``'s ``mode``), the best of four timings
+    of about two milliseconds of calls each, the ways taking turns. PFLOP/s count the causal half of both products."""
+    import torch
+
+    from .cache.spec import PAGE_TOKENS, pages_for
+    from .csrc import ops
+    from .engine.engine import require_gpu
+
+    dev = require_gpu("cuda:0")
+    heads, kv, dim = args.heads, args.kv_heads, args.head_dim
+    modes = [int(m) for m in args.modes.split(",")]
+    gen = torch.Generator(device=dev).manual_seed(args.seed)
+    rand = lambda *shape: torch.randn(*shape, device=dev, generator=gen).to(torch.bfloat16)
+    ints = lambda values: torch.tensor(values, dtype=torch.int32, device=dev)
+    for shape in args.shapes.split(","):
+        n_seqs, length = (int(x) for x in shape.lower().split("x"))
+        pages = pages_for(length)
+        k, v = rand(n_seqs * pages, kv, PAGE_TOKENS, dim), rand(n_seqs * pages, kv, dim, PAGE_TOKENS)
+        q = rand(n_seqs * length, heads, dim)
+        out = torch.empty_like(q)
+        table = torch.arange(n_seqs * pages, dtype=torch.int32, device=dev).view(n_seqs, pages)
+        seq_slot, seq_start = ints(list(range(n_seqs))), ints([0] * n_seqs)
+        cu_rows = ints([length * i for i in range(n_seqs + 1)])
+        tile_cu = ints([ops.row_tiles(length) * i for i in range(n_seqs + 1)])
+        flops = 2.0 * n_seqs * length * length * heads * dim
+        calls = max(3, int(2e-3 * 0.8e15 / flops))
+        best = {m: float("inf") for m in modes}
+        for _ in range(4):
+            for m in modes:
+                run = lambda: ops.attn_causal_bf16(q, k, v, table, seq_slot, cu_rows, tile_cu, seq_start, n_seqs,
+                                                   n_seqs * ops.row_tiles(length), out, heads, kv, dim, dim ** -0.5, 0, m)
+                run()
+                torch.cuda.synchronize()
+                begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                begin.record()
+                for _ in range(calls):
+                    run()
+                end.record()
+                torch.cuda.synchronize()
+                best[m] = min(best[m], begin.elapsed_time(end) / calls * 1e-3)
+        print(f"{n_seqs} x {length}: " + "  ".join(f"mode {m}: {best[m] * 1e6:8.1f} us {flops / best[m] / 1e15:5.3f} PFLOP/s"
+                                                  for m in modes), flush=True)
+    return 0
+
+
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser(prog="dryft_amd", description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     sub = ap.add_subparsers(dest="command", required=True)
@@ -257,6 +305,15 @@ def main(argv=None) -> int:
     pr.add_argument("--rows", type=int, default=20, help="kernels to list")
     pr.add_argument("--seed", type=int, default=0)
     pr.set_defaults(fn=cmd_profile)
+
+    at = sub.add_parser("attention", help="time the prompt-attention kernel alone, in each way of running it")
+    at.add_argument("--shapes", default="1x2048,1x4096,8x2048", help="BxL,...: B sequences of L positions each")
+    at.add_argument("--modes", default="0", help="ways of running the kernel (ops.attn_causal_bf16's mode), e.g. 1,3,5,7")
+    at.add_argument("--heads", type=int, default=32)
+    at.add_argument("--kv-heads", type=int, default=8)
+    at.add_argument("--head-dim", type=int, default=128)
+    at.add_argument("--seed", type=int, default=0)
+    at.set_defaults(fn=cmd_attention)
 
     bd = sub.add_parser("build", help="compile the HIP kernel libraries (needs hipcc, no GPU)")
     bd.add_argument("names", nargs="*", help="libraries to build (default: all)")

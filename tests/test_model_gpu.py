@@ -716,6 +716,9 @@ def test_command_line_bench_and_profile():
     assert any("attn_split_kernel" in row for row in table) and any("add_rmsnorm" in row for row in table)
     out = run_cli("profile", "--tiny", "--batch", "2", "--prompt-len", "70", "--prefill")
     assert "one step of 2 prompts of 70 tokens" in out and any("attn_causal_kernel" in row for row in out.splitlines())
+    out = run_cli("attention", "--shapes", "2x200,1x70", "--modes", "0,1,5", "--heads", "8", "--kv-heads", "2")
+    rows = out.strip().splitlines()
+    assert len(rows) == 2 and rows[0].startswith("2 x 200:") and rows[0].count("PFLOP/s") == 3
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
