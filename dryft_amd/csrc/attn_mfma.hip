@@ -531,6 +531,77 @@ __device__ __forceinline__ uint32_t direct_offset_v(int wave, int lane) {
   return row * (2 * PAGE_TOKENS) + ((place ^ ((row >> 1) & 7)) << 4);
 }
 
+// What the kernel needs to take a row's query heads straight from the fused projection: per-head RMSNorm
+// (optional) and the rotation of pairs (j, j + 64) over the full head, with the roundings of the stand-alone kernel
+// (rope_kv.hip). Saves writing the queries out and reading them back.
+struct ProjectedQ {
+  const bf16_t* qkv;       // [rows, stride]: the row's query heads come first; null: q is given ready
+  int64_t stride;
+  const void* q_w;
+  int w_f32, has_norm;
+  float eps;
+  const bf16_t* cos_t;     // [positions, 64]
+  const bf16_t* sin_t;
+};
+
+// A lane holds 8 features 32 kb + 8 g .. of its row for kb = 0..3 (the first product's B operand): the four lanes
+// of a row add up their sums of squares, and a feature's rotation partner (64 further on) sits in the same lane.
+__device__ __forceinline__ void init_rows_projected(RowBlock<4>& st, const ProjectedQ& pq, int64_t row, int head,
+                                                    int pos, bool row_valid) {
+  const int g = (threadIdx.x % WAVE) / 16;
+  float x[4][8];
+#pragma unroll
+  for (int kb = 0; kb < 4; ++kb) {
+    if (row_valid) {
+      load8_as_float(pq.qkv + row * pq.stride + (int64_t)head * DIRECT_D + 32 * kb + 8 * g, x[kb]);
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) x[kb][i] = 0.f;
+    }
+  }
+  if (pq.has_norm) {
+    float ss = 0.f;
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+      for (int i = 0; i < 8; ++i) ss += x[kb][i] * x[kb][i];
+    ss += __shfl_xor(ss, 16, WAVE);
+    ss += __shfl_xor(ss, 32, WAVE);
+    const float inv = rsqrtf(ss / (float)DIRECT_D + pq.eps);
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb) {
+      float w[8];
+      if (pq.w_f32) load8_as_float((const float*)pq.q_w + 32 * kb + 8 * g, w);
+      else load8_as_float((const bf16_t*)pq.q_w + 32 * kb + 8 * g, w);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) x[kb][i] = rounded_as<bf16_t>(rounded_as<bf16_t>(x[kb][i] * inv) * w[i]);
+    }
+  }
+#pragma unroll
+  for (int kb = 0; kb < 2; ++kb) {
+    float c[8], sn[8];
+    if (row_valid) {
+      load8_as_float(pq.cos_t + (int64_t)pos * (DIRECT_D / 2) + 32 * kb + 8 * g, c);
+      load8_as_float(pq.sin_t + (int64_t)pos * (DIRECT_D / 2) + 32 * kb + 8 * g, sn);
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) { c[i] = 1.f; sn[i] = 0.f; }
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float x1 = x[kb][i], x2 = x[kb + 2][i];
+      const float o1 = rounded_as<bf16_t>(x1 * c[i]) - rounded_as<bf16_t>(x2 * sn[i]);   // x1*c - x2*s
+      const float o2 = rounded_as<bf16_t>(x2 * c[i]) + rounded_as<bf16_t>(x1 * sn[i]);   // x2*c + x1*s
+      st.q[kb][i] = to_bf16(o1);
+      st.q[kb + 2][i] = to_bf16(o2);
+    }
+  }
+#pragma unroll
+  for (int dt = 0; dt < 8; ++dt) st.o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  st.m = -INFINITY;
+  st.l = 0.f;
+}
+
 // RP tiles of 16 consecutive rows per wave; a workgroup's tile is 64 * RP rows. Grid: (heads, tiles), the
 // tiles with the most pages first. With 16 rows a wave, keys and values have one buffer each and a page takes two
 // barriers (the values arrive during the first product and the softmax, the next keys during the second
@@ -543,7 +614,7 @@ __global__ __launch_bounds__(256, RP == 1 ? 4 : 2) void attn_causal_direct_kerne
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
     const int* __restrict__ page_table, int max_pages, const int* __restrict__ seq_slot,
     const int* __restrict__ cu_rows, const int* __restrict__ tile_cu, const int* __restrict__ seq_start, int n_seqs,
-    bf16_t* __restrict__ out, int n_heads, int n_kv, float scale, int window) {
+    bf16_t* __restrict__ out, int n_heads, int n_kv, float scale, int window, ProjectedQ projected) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   constexpr int KB = DIRECT_D / 32, TILE_ROWS = 64 * RP, WAVE_ROWS = 16 * RP, head_dim = DIRECT_D;
   constexpr bool TWO = RP != 1;                               // two buffers each for keys and values
@@ -575,7 +646,10 @@ __global__ __launch_bounds__(256, RP == 1 ? 4 : 2) void attn_causal_direct_kerne
     pos0[rt] = pos_wave + 16 * rt;
     pos_row[rt] = row_valid[rt] ? pos0[rt] + c : -1;
     lo_row[rt] = window > 0 ? max(0, pos_row[rt] - window + 1) : 0;
-    init_rows<KB>(st[rt], q + (row[rt] * n_heads + head) * head_dim, row_valid[rt], head_dim);
+    if (projected.qkv != nullptr)
+      init_rows_projected(st[rt], projected, row[rt], head, pos0[rt] + c, row_valid[rt]);
+    else
+      init_rows<KB>(st[rt], q + (row[rt] * n_heads + head) * head_dim, row_valid[rt], head_dim);
   }
   const int kvh = head / (n_heads / n_kv);
   const int lo_wave = window > 0 ? max(0, pos_wave - window + 1) : 0;
@@ -1027,24 +1101,24 @@ template <int RP>
 static int launch_causal_direct(const void* q, const void* k_pages, const void* v_pages, const int* page_table,
                                 int max_pages, const int* seq_slot, const int* cu_rows, const int* tile_cu,
                                 const int* seq_start, int n_seqs, int max_tiles, void* out, int n_heads, int n_kv,
-                                float scale, int window, hipStream_t stream) {
+                                float scale, int window, ProjectedQ projected, hipStream_t stream) {
   // max_tiles bounds the 64-row tiles of the sequences that take part; a sequence with t of them has ceil(t / RP)
   dim3 grid(n_heads, (max_tiles + (RP - 1) * (n_seqs + 1)) / RP), block(256);
   if (grid.y > 65535) return -1;
   const size_t lds = (size_t)(RP == 1 ? 2 : 4) * DIRECT_PAGE_BYTES;
   hipLaunchKernelGGL(attn_causal_direct_kernel<RP>, grid, block, lds, stream, (const bf16_t*)q, (const bf16_t*)k_pages,
                      (const bf16_t*)v_pages, page_table, max_pages, seq_slot, cu_rows, tile_cu, seq_start, n_seqs,
-                     (bf16_t*)out, n_heads, n_kv, scale, window);
+                     (bf16_t*)out, n_heads, n_kv, scale, window, projected);
   return DRYFT_LAUNCH_CHECK();
 }
 
 // mode: 0 = chosen here; 1 = one head and 16 rows per wave; 2 = two heads of a kv group per wave (even groups,
 // head_dim <= 128); 3 = one head and 32 rows per wave (head_dim <= 128). At head size 128, modes 1 and 3 bring
 // the pages straight into LDS; 5 and 7 are 1 and 3 with the pages staged through registers, as at other sizes.
-DRYFT_API int dryft_attn_causal_bf16(const void* q, const void* k_pages, const void* v_pages, const int* page_table,
-                                     int max_pages, const int* seq_slot, const int* cu_rows, const int* tile_cu,
-                                     const int* seq_start, int n_seqs, int max_tiles, void* out, int n_heads,
-                                     int n_kv, int head_dim, float scale, int window, int mode, hipStream_t stream) {
+static int causal_entry(const void* q, const void* k_pages, const void* v_pages, const int* page_table, int max_pages,
+                        const int* seq_slot, const int* cu_rows, const int* tile_cu, const int* seq_start, int n_seqs,
+                        int max_tiles, void* out, int n_heads, int n_kv, int head_dim, float scale, int window, int mode,
+                        ProjectedQ projected, hipStream_t stream) {
   if (n_seqs <= 0 || max_tiles <= 0) return 0;
   if (!head_shape_ok(n_heads, n_kv, head_dim)) return -1;
   const int group = n_heads / n_kv;
@@ -1072,14 +1146,44 @@ DRYFT_API int dryft_attn_causal_bf16(const void* q, const void* k_pages, const v
   if (direct_ok && !staged && mode != 2) {
     if (mode == 3)
       return launch_causal_direct<2>(q, k_pages, v_pages, page_table, max_pages, seq_slot, cu_rows, tile_cu, seq_start,
-                                     n_seqs, max_tiles, out, n_heads, n_kv, scale, window, stream);
+                                     n_seqs, max_tiles, out, n_heads, n_kv, scale, window, projected, stream);
     return launch_causal_direct<1>(q, k_pages, v_pages, page_table, max_pages, seq_slot, cu_rows, tile_cu, seq_start,
-                                     n_seqs, max_tiles, out, n_heads, n_kv, scale, window, stream);
+                                   n_seqs, max_tiles, out, n_heads, n_kv, scale, window, projected, stream);
   }
+  if (projected.qkv != nullptr) return -1;                   // only the kernel above takes the projection itself
   if (mode == 2) CAUSAL(2, 1);
   if (mode == 3) CAUSAL(1, 2);
   CAUSAL(1, 1);
 #undef CAUSAL
+}
+
+DRYFT_API int dryft_attn_causal_bf16(const void* q, const void* k_pages, const void* v_pages, const int* page_table,
+                                     int max_pages, const int* seq_slot, const int* cu_rows, const int* tile_cu,
+                                     const int* seq_start, int n_seqs, int max_tiles, void* out, int n_heads,
+                                     int n_kv, int head_dim, float scale, int window, int mode, hipStream_t stream) {
+  ProjectedQ none = {};
+  return causal_entry(q, k_pages, v_pages, page_table, max_pages, seq_slot, cu_rows, tile_cu, seq_start, n_seqs,
+                      max_tiles, out, n_heads, n_kv, head_dim, scale, window, mode, none, stream);
+}
+
+// Can the causal kernel take the queries from the fused projection itself (norm, rotation over `rot` features)?
+DRYFT_API int dryft_attn_causal_takes_projection(int head_dim, int rot) { return head_dim == DIRECT_D && rot == DIRECT_D; }
+
+// The same with the queries taken from the projection output qkv[rows, stride] (query heads first): per-head
+// RMSNorm with q_w (has_norm) and rotation by the tables cos_t / sin_t [positions, head_dim / 2] happen on the way
+// into the kernel's registers. Only where dryft_attn_causal_takes_projection says so; mode 0, 1 or 3.
+DRYFT_API int dryft_attn_causal_projected_bf16(const void* qkv, int64_t qkv_stride, const void* q_w, int w_f32,
+                                               int has_norm, float eps, const void* cos_t, const void* sin_t,
+                                               const void* k_pages, const void* v_pages, const int* page_table,
+                                               int max_pages, const int* seq_slot, const int* cu_rows,
+                                               const int* tile_cu, const int* seq_start, int n_seqs, int max_tiles,
+                                               void* out, int n_heads, int n_kv, int head_dim, float scale, int window,
+                                               int mode, hipStream_t stream) {
+  if (qkv == nullptr || cos_t == nullptr || sin_t == nullptr || (has_norm && q_w == nullptr)) return -1;
+  if (head_dim != DIRECT_D || (mode != 0 && mode != 1 && mode != 3) || qkv_stride % 8 || ((uintptr_t)qkv & 15)) return -1;
+  ProjectedQ projected = {(const bf16_t*)qkv, qkv_stride, q_w, w_f32, has_norm, eps, (const bf16_t*)cos_t, (const bf16_t*)sin_t};
+  return causal_entry(nullptr, k_pages, v_pages, page_table, max_pages, seq_slot, cu_rows, tile_cu, seq_start, n_seqs,
+                      max_tiles, out, n_heads, n_kv, head_dim, scale, window, mode, projected, stream);
 }
 
 static int launch_split(const void* q, const void* k_pages, const void* v_pages, const int* page_table, int max_pages,

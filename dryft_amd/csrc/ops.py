@@ -27,6 +27,9 @@ _SIGNATURES = {
                                           _I, _I, _I, _I, _I, _P]},
     "attn_rows": {"dryft_attn_rows": [_P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _F, _I, _I, _P]},
     "attn_mfma": {"dryft_attn_causal_bf16": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _P, _I, _I, _I, _F, _I, _I, _P],
+                  "dryft_attn_causal_takes_projection": [_I, _I],
+                  "dryft_attn_causal_projected_bf16": [_P, _L, _P, _I, _I, _F, _P, _P, _P, _P, _P, _I, _P, _P, _P, _P, _I,
+                                                       _I, _P, _I, _I, _I, _F, _I, _I, _P],
                   "dryft_attn_split_bf16": [_P, _P, _P, _P, _I, _P, _P, _P, _I, _P, _P, _I, _P, _I, _I, _I, _F, _I,
                                             _P],
                   "dryft_attn_decode_fused_bf16": [_P, _L, _P, _P, _I, _I, _F, _P, _P, _I, _I, _P, _P, _P, _I, _P, _P,
@@ -192,8 +195,10 @@ def silu_mul(gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
 
 # ----------------------------------------------------------------------------------------- rope_kv
 def qk_norm_rope_kv(qkv: torch.Tensor, q_weight, k_weight, eps: float, cos, sin, rot: int, row_slot, row_pos,
-                    q_out: torch.Tensor, k_pages, v_pages, page_table, write_kv: bool, n_heads: int, n_kv: int,
+                    q_out, k_pages, v_pages, page_table, write_kv: bool, n_heads: int, n_kv: int,
                     head_dim: int) -> None:
+    """Per-head norm and rotation of a step's query and key heads, and the append of keys and values to the cache.
+    ``q_out`` None: only keys and values are handled (the attention kernel takes the queries from ``qkv`` itself)."""
     _gpu(qkv, "qkv")
     is_f32 = _float_flag(qkv, "qkv")
     rows = qkv.shape[0]
@@ -216,8 +221,11 @@ def qk_norm_rope_kv(qkv: torch.Tensor, q_weight, k_weight, eps: float, cos, sin,
     for name, t in (("row_slot", row_slot), ("row_pos", row_pos)):
         _gpu(t, name, torch.int32)
         _require(t.numel() >= rows and t.is_contiguous(), f"{name}: needs {rows} entries")
-    _gpu(q_out, "q_out", qkv.dtype)
-    _require(q_out.is_contiguous() and q_out.numel() == rows * n_heads * head_dim, "q_out: must be [rows, heads, head_dim]")
+    if q_out is not None:
+        _gpu(q_out, "q_out", qkv.dtype)
+        _require(q_out.is_contiguous() and q_out.numel() == rows * n_heads * head_dim, "q_out: must be [rows, heads, head_dim]")
+    else:
+        _require(write_kv, "qk_norm_rope_kv: nothing to do without q_out and without a cache to write")
     max_pages = 0
     if write_kv:
         _check_pages(k_pages, v_pages, page_table, n_kv, head_dim, qkv.dtype)
@@ -277,6 +285,46 @@ def attn_causal_bf16(q, k_pages, v_pages, page_table, seq_slot, cu_rows, tile_cu
         _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(page_table), page_table.shape[1], _ptr(seq_slot), _ptr(cu_rows),
         _ptr(tile_cu), _ptr(seq_start), n_seqs, max_tiles, _ptr(out), n_heads, n_kv, head_dim, float(scale),
         int(window), int(mode), _stream()), "attn_causal_bf16")
+
+
+def attn_causal_takes_projection(head_dim: int, rot: int) -> bool:
+    """Can ``attn_causal_projected_bf16`` run heads of this size, rotated over ``rot`` features?"""
+    return bool(_fn("attn_mfma", "dryft_attn_causal_takes_projection")(int(head_dim), int(rot)))
+
+
+def attn_causal_projected_bf16(qkv, q_weight, eps: float, cos, sin, k_pages, v_pages, page_table, seq_slot, cu_rows,
+                               tile_cu, seq_start, n_seqs: int, max_tiles: int, out, n_heads: int, n_kv: int,
+                               head_dim: int, scale: float, window: int, mode: int = 0) -> None:
+    """``attn_causal_bf16`` with the queries taken from the fused projection ``qkv`` [rows, >= n_heads * head_dim]
+    (query heads first): their per-head norm (``q_weight`` or None) and rotation happen inside the kernel, so they
+    are neither written out nor read back. Keys and values must be in the cache already."""
+    _gpu(qkv, "qkv", torch.bfloat16)
+    _gpu(out, "out", torch.bfloat16)
+    rows = qkv.shape[0]
+    _require(qkv.dim() == 2 and qkv.stride(1) == 1 and qkv.shape[1] >= n_heads * head_dim and qkv.stride(0) % 8 == 0,
+             "attn_causal_projected: qkv must be [rows, >= heads * head_dim] with rows 16 bytes apart or a multiple")
+    _require(out.is_contiguous() and out.numel() == rows * n_heads * head_dim, "attn_causal_projected: out [rows, heads, head_dim]")
+    _require(attn_causal_takes_projection(head_dim, 2 * cos.shape[1] if cos is not None else 0),
+             "attn_causal_projected: the kernel refuses these sizes")
+    w_f32 = 0
+    if q_weight is not None:
+        _gpu(q_weight, "q_weight")
+        _require(q_weight.shape == (head_dim,) and q_weight.is_contiguous(), f"q_weight: must be [{head_dim}]")
+        w_f32 = _float_flag(q_weight, "q_weight")
+    for name, t in (("cos", cos), ("sin", sin)):
+        _gpu(t, name, torch.bfloat16)
+        _require(t.dim() == 2 and t.shape[1] == head_dim // 2 and t.is_contiguous(), f"{name}: must be [positions, {head_dim // 2}]")
+    _check_pages(k_pages, v_pages, page_table, n_kv, head_dim, torch.bfloat16)
+    for name, t, n in (("seq_slot", seq_slot, n_seqs), ("cu_rows", cu_rows, n_seqs + 1),
+                       ("tile_cu", tile_cu, n_seqs + 1), ("seq_start", seq_start, n_seqs)):
+        _gpu(t, name, torch.int32)
+        _require(t.numel() >= n, f"{name}: needs {n} entries")
+    _require(n_heads <= 65535, "attn_causal: too many heads")
+    _check(_fn("attn_mfma", "dryft_attn_causal_projected_bf16")(
+        _ptr(qkv), qkv.stride(0), _ptr(q_weight), w_f32, int(q_weight is not None), float(eps), _ptr(cos), _ptr(sin),
+        _ptr(k_pages), _ptr(v_pages), _ptr(page_table), page_table.shape[1], _ptr(seq_slot), _ptr(cu_rows), _ptr(tile_cu),
+        _ptr(seq_start), n_seqs, max_tiles, _ptr(out), n_heads, n_kv, head_dim, float(scale), int(window), int(mode),
+        _stream()), "attn_causal_projected_bf16")
 
 
 def attn_split_bf16(q, k_pages, v_pages, page_table, seq_slot, cu_rows, kv_len, n_seqs: int, part_o, part_ml,

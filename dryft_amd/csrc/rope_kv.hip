@@ -31,6 +31,7 @@ __global__ void qk_norm_rope_kv_kernel(const T* __restrict__ qkv, int64_t qkv_st
   const int pos = row_pos[row];
   const bool is_q = job < n_heads, is_k = !is_q && job < n_heads + n_kv;
   const T* src = qkv + row * qkv_stride + (int64_t)job * head_dim;
+  if (is_q && q_out == nullptr) return;                // the caller takes the queries from the projection itself
   if (is_q) {
     T* dst = q_out + (row * n_heads + job) * head_dim;
     if (slot < 0) {
@@ -108,7 +109,8 @@ __global__ __launch_bounds__(256) void qk_norm_rope_vec_kernel(const T* __restri
   const int job = blockIdx.y * (256 / lph) + threadIdx.x / lph;
   const int part = threadIdx.x % lph;
   const int jobs = n_heads + (write_kv ? (with_v ? 2 : 1) * n_kv : 0);   // q heads, k heads, then v heads
-  const bool live_job = job < jobs;                    // lanes of a dead job still take part in the shuffles
+  // lanes of a dead job still take part in the shuffles; without q_out the query heads are dead jobs
+  const bool live_job = job < jobs && (q_out != nullptr || job >= n_heads);
   const bool is_v = job >= n_heads + n_kv;
   const int slot = row_slot[row], pos = row_pos[row];
   const bool is_q = job < n_heads;
@@ -185,7 +187,8 @@ __device__ __forceinline__ void qk_norm_rope_row(int64_t row, const T* __restric
   const int slot = row_slot[row], pos = row_pos[row];
   if (slot < 0) {                                       // a dead row: its q is zero, nothing is cached
     const float z[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    for (int job = lane_head; job < n_heads; job += PER) store8_from_float(q_out + (row * n_heads + job) * D + 8 * part, z);
+    if (q_out != nullptr)
+      for (int job = lane_head; job < n_heads; job += PER) store8_from_float(q_out + (row * n_heads + job) * D + 8 * part, z);
     return;
   }
   const bool first = part < LPH / 2;
@@ -205,7 +208,7 @@ __device__ __forceinline__ void qk_norm_rope_row(int64_t row, const T* __restric
   const int page = write_kv ? page_of(page_table, max_pages, slot, pos) : -1;
   const int jobs = n_heads + (page >= 0 ? n_kv : 0);    // q heads, then k heads
   const T* src = qkv + row * qkv_stride + 8 * part;
-  for (int j0 = lane_head; j0 < jobs; j0 += 4 * PER) {
+  for (int j0 = (q_out != nullptr ? 0 : n_heads) + lane_head; j0 < jobs; j0 += 4 * PER) {   // without q_out: keys only
     float v[4][8];
 #pragma unroll
     for (int u = 0; u < 4; ++u)

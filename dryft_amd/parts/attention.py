@@ -101,6 +101,18 @@ class GQAAttention(Mixer):
                                        ctx.kv_len, ctx.n_seqs, part_o, part_ml, splits, out, self.n_heads, self.n_kv,
                                        self.head_dim, self.scale, window)
             return linear(out.view(rows, self.q_dim), self.w_o, allow_partials=True)
+        if matrix_cores and not decoding and cos is not None and \
+                ops.attn_causal_takes_projection(self.head_dim, self.rotary_dim):
+            # the prompt kernel norms and rotates the queries on their way in: only keys and values go to the cache here
+            if writes_cache:
+                ops.qk_norm_rope_kv(qkv, self.q_norm, self.k_norm, self.qk_norm_eps or 0.0, cos, sin, self.rotary_dim,
+                                    ctx.row_slot, ctx.row_pos, None, line.k, line.v, line.page_table, True,
+                                    self.n_heads, self.n_kv, self.head_dim)
+            ops.attn_causal_projected_bf16(qkv, self.q_norm, self.qk_norm_eps or 0.0, cos, sin, line.k, line.v,
+                                           line.page_table, ctx.seq_slot, ctx.cu_rows, ctx.tile_cu, ctx.seq_start,
+                                           ctx.n_seqs, ctx.max_tiles, out, self.n_heads, self.n_kv, self.head_dim,
+                                           self.scale, window)
+            return linear(out.view(rows, self.q_dim), self.w_o, allow_partials=True)
         q = torch.empty((rows, self.n_heads, self.head_dim), dtype=h.dtype, device=h.device)
         ops.qk_norm_rope_kv(qkv, self.q_norm, self.k_norm, self.qk_norm_eps or 0.0, cos, sin, self.rotary_dim,
                             ctx.row_slot, ctx.row_pos, q, line.k, line.v, line.page_table, writes_cache,

@@ -433,6 +433,69 @@ def test_attn_decode_fused_equals_the_two_kernels(n_heads, n_kv, D, splits, wind
     assert torch.equal(k3, k1) and torch.equal(v3, v1) and torch.equal(out3, out2)
 
 
+@pytest.mark.parametrize("mode,few_rows,w_f32,window", [(1, False, False, 0), (3, False, True, 0), (0, True, False, 0),
+                                                      (1, False, False, 100)])
+def test_prompt_attention_that_takes_the_queries_from_the_projection(mode, few_rows, w_f32, window):
+    """At head size 128 the prompt kernel norms and rotates the queries itself. It gives what the stand-alone
+    kernel plus the prompt kernel give (the sum of squares is added up in another order, so a value may land on the
+    neighbouring bfloat16 now and then), and the cache gets the same keys and values whether or not the queries are
+    written out. Sequences continue cached tokens, one sits out, one has a single row."""
+    torch.manual_seed(7 + mode)
+    o = ops()
+    n_heads, n_kv, D = 8, 2, 128
+    assert o.attn_causal_takes_projection(D, D) and not o.attn_causal_takes_projection(64, 64)
+    assert not o.attn_causal_takes_projection(D, 64)
+    q_lens = [3, 1, 5, 2] if few_rows else [150, 1, 70, 260]        # few rows: the append goes through the other kernels
+    starts = [40, 0, 100, 9]
+    B, n_slots, max_pages = len(q_lens), 6, 6
+    n_pages = n_slots * max_pages
+    rng = np.random.default_rng(mode)
+    table = torch.tensor(rng.permutation(n_pages).reshape(n_slots, max_pages), dtype=torch.int32, device=DEV)
+    slots = [int(x) for x in rng.permutation(n_slots)[:B]]
+    slots[2] = -1                                                 # this sequence sits out
+    rows = sum(q_lens)
+    cu = np.concatenate([[0], np.cumsum(q_lens)]).astype(np.int32)
+    tiles = np.concatenate([[0], np.cumsum([0 if s < 0 else (n + 63) // 64 for s, n in zip(slots, q_lens)])]).astype(np.int32)
+    row_slot = torch.tensor([slots[b] for b, n in enumerate(q_lens) for _ in range(n)], dtype=torch.int32, device=DEV)
+    row_pos = torch.tensor([starts[b] + i for b, n in enumerate(q_lens) for i in range(n)], dtype=torch.int32, device=DEV)
+    seq_slot = torch.tensor(slots, dtype=torch.int32, device=DEV)
+    cu_d, tiles_d = torch.from_numpy(cu).to(DEV), torch.from_numpy(tiles).to(DEV)
+    seq_start = torch.tensor(starts, dtype=torch.int32, device=DEV)
+    qkv = (2 * torch.randn(rows, (n_heads + 2 * n_kv) * D)).to(torch.bfloat16).to(DEV)
+    wdt = torch.float32 if w_f32 else torch.bfloat16
+    wq, wk = (1 + 0.1 * torch.randn(D)).to(wdt).to(DEV), (1 + 0.1 * torch.randn(D)).to(wdt).to(DEV)
+    ang = torch.arange(512).float()[:, None] * (1.0 / (1e4 ** (torch.arange(0, D, 2).float() / D)))[None]
+    cos, sin = ang.cos().to(torch.bfloat16).to(DEV), ang.sin().to(torch.bfloat16).to(DEV)
+    k0 = torch.randn(n_pages, n_kv, 64, D).to(torch.bfloat16).to(DEV)
+    v0 = torch.randn(n_pages, n_kv, D, 64).to(torch.bfloat16).to(DEV)
+    scale = D ** -0.5
+    k1, v1 = k0.clone(), v0.clone()
+    q = torch.empty(rows, n_heads, D, dtype=torch.bfloat16, device=DEV)
+    out1 = torch.zeros(rows, n_heads, D, dtype=torch.bfloat16, device=DEV)
+    o.qk_norm_rope_kv(qkv, wq, wk, 1e-6, cos, sin, D, row_slot, row_pos, q, k1, v1, table, True, n_heads, n_kv, D)
+    o.attn_causal_bf16(q, k1, v1, table, seq_slot, cu_d, tiles_d, seq_start, B, int(tiles[-1]), out1, n_heads, n_kv, D,
+                       scale, window, mode)
+    k2, v2 = k0.clone(), v0.clone()
+    out2 = torch.zeros_like(out1)
+    o.qk_norm_rope_kv(qkv, wq, wk, 1e-6, cos, sin, D, row_slot, row_pos, None, k2, v2, table, True, n_heads, n_kv, D)
+    o.attn_causal_projected_bf16(qkv, wq, 1e-6, cos, sin, k2, v2, table, seq_slot, cu_d, tiles_d, seq_start, B,
+                                 int(tiles[-1]), out2, n_heads, n_kv, D, scale, window, mode)
+    assert torch.equal(k1, k2) and torch.equal(v1, v2), "the cache differs"
+    assert not torch.equal(k1, k0), "nothing was appended"
+    dead = slice(int(cu[2]), int(cu[3]))
+    assert not out2[dead].any(), "rows of the sequence that sits out were written"
+    assert out1.abs().max() > 0.1
+    close(out2, out1.float().cpu(), torch.bfloat16, ulps=2.0, floor=1e-3, what=f"queries from the projection, mode {mode}")
+    assert (out1 != out2).float().mean() < 0.02, "more than a rounding here and there"
+    # without the norm
+    o.qk_norm_rope_kv(qkv, None, None, 0.0, cos, sin, D, row_slot, row_pos, q, k1, v1, table, True, n_heads, n_kv, D)
+    o.attn_causal_bf16(q, k1, v1, table, seq_slot, cu_d, tiles_d, seq_start, B, int(tiles[-1]), out1, n_heads, n_kv, D,
+                       scale, window, mode)
+    o.attn_causal_projected_bf16(qkv, None, 0.0, cos, sin, k1, v1, table, seq_slot, cu_d, tiles_d, seq_start, B,
+                                 int(tiles[-1]), out2, n_heads, n_kv, D, scale, window, mode)
+    assert torch.equal(out1, out2), "without a norm nothing is summed: bit for bit"
+
+
 @pytest.mark.parametrize("kind", ["rows", "causal1", "causal2", "causal3", "causal5", "causal7", 3])
 def test_attention_window(kind):
     tq = 1 if kind == 3 else 90
