@@ -530,6 +530,166 @@ DRYFT_API int dryft_gemm_wide_swiglu_bf16(const void* x, int64_t x_stride, const
 #undef WS
 }
 
+// ------------------------------------------------------------------------------------------- panel
+// The fused gate/up product with its activation for 17 to 64 rows, with the operands going from memory straight
+// into LDS (global_load_lds_dwordx4: 16 bytes a lane, no registers in between and nothing for the waves to store),
+// two groups of K ahead of the one that is multiplied. A workgroup of six waves owns 48 outputs: waves 0 to 2 hold
+// 16 gate rows each, waves 3 to 5 the up rows of the same outputs, and all MT tiles of 16 rows of x. A group is
+// 128 values of K: 256 bytes of every row, 16 pieces of 16 bytes, piece p of row r at place p ^ (r % 16), so that
+// operand reads meet no bank twice without padding; which piece a lane fetches is what places it. One instruction
+// fills 1 KB (four rows); a wave fetches its own 16 weight rows (four instructions) and its share of the rows of x
+// (dealt to the waves in turn; every wave issues the same number, the last piece again if need be). Three groups
+// have room in LDS (120 KB at 64 rows: one workgroup a compute unit). Every wave issues the same number of loads
+// per group, also past the end of K (the last group again, into a buffer nobody reads), so one constant says how
+// many may still be in flight when a group is needed. K must be a multiple of 128. The compiler does not know
+// that these loads write LDS; each wave waits for its own, then a barrier.
+// Measured beside it on Qwen3-4B's gate/up at 64 rows (26 us; the vendor library plus the activation kernel 31):
+// four waves and 32 outputs (304 workgroups, two rounds or shallow stages: 32 to 38 us), eight waves (28 to 34),
+// groups of 64 values (27 to 36), four stages (the same), weights and activations fetched by different waves with
+// depths of their own (26 at best). The plain product of the same form was no faster than what serves it now.
+__device__ __forceinline__ void panel_load16(const void* base, uint32_t offset, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_base), "v"(offset), "s"(base) : "memory");
+}
+
+// s_waitcnt vmcnt(N) alone (vmcnt sits in bits 3:0 and 15:14 of the immediate, the other counters stay at their
+// maxima); as a builtin, so that the compiler's own count of loads in flight takes it into account
+template <int N>
+__device__ __forceinline__ void panel_wait() {
+  __builtin_amdgcn_s_waitcnt(0x0f70 | (N & 15) | ((N >> 4) << 14));
+  asm volatile("" ::: "memory");
+}
+
+#define PANEL_GROUP 128                      // values of K in a group; K must be a multiple of it
+#define PANEL_WAVES 6
+#define PANEL_STAGES 3
+#define PANEL_OUTPUTS (8 * PANEL_WAVES)      // of a workgroup
+
+template <int MT>
+__global__ __launch_bounds__(64 * PANEL_WAVES) void gemm_panel_swiglu_kernel(const bf16_t* __restrict__ x,
+                                                                             int64_t x_stride,
+                                                                             const bf16_t* __restrict__ w,
+                                                                             bf16_t* __restrict__ y, int M, int N,
+                                                                             int K) {
+  extern __shared__ __align__(16) unsigned char panel_lds[];
+  constexpr int WAVES = PANEL_WAVES, STAGES = PANEL_STAGES, HALF = WAVES / 2;
+  constexpr int RB = 2 * PANEL_GROUP;                      // bytes of a row in a group
+  constexpr int X_ALL = 4 * MT;                            // 1 KB pieces of x in a group, dealt to the waves in turn
+  constexpr int X_LOADS = (X_ALL + WAVES - 1) / WAVES;     // every wave issues this many
+  constexpr int LOADS = 4 + X_LOADS;                       // per wave and group
+  constexpr int W_BYTES = 16 * WAVES * RB, X_BYTES = 16 * MT * RB, STAGE_BYTES = W_BYTES + X_BYTES;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
+  const int lane = threadIdx.x % WAVE, c = lane % 16, g = lane / 16;
+  const int n0 = blockIdx.x * PANEL_OUTPUTS + 16 * (wave % HALF);                 // first output of this wave
+  const int w_row0 = (wave >= HALF ? N : 0) + n0;          // its first weight row (W = [Wg; Wu])
+  const int w_last = (wave >= HALF ? 2 * N : N) - 1;
+  const int groups = K / PANEL_GROUP;
+  // where this lane fetches: its place within an instruction's 1 KB is fixed, the piece that belongs there follows
+  uint32_t w_from[4], x_from[X_LOADS];
+  int x_piece[X_LOADS];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = 4 * i + lane / 16;                       // row within the wave's 16
+    w_from[i] = (uint32_t)min(w_row0 + r, w_last) * (uint32_t)K * 2u + (((lane % 16) ^ r) << 4);
+  }
+#pragma unroll
+  for (int i = 0; i < X_LOADS; ++i) {
+    x_piece[i] = min(wave + WAVES * i, X_ALL - 1);
+    const int r = 4 * x_piece[i] + lane / 16;              // row of x
+    x_from[i] = (uint32_t)min(r, M - 1) * (uint32_t)x_stride * 2u + (((lane % 16) ^ (r & 15)) << 4);
+  }
+  const uint32_t lds0 = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)panel_lds);
+  auto fetch = [&](int group, int stage) {
+    const int gk = min(group, groups - 1);                 // past the end: the last group again, into a free buffer
+    const unsigned char* wb = (const unsigned char*)w + (int64_t)gk * RB;
+    const unsigned char* xb = (const unsigned char*)x + (int64_t)gk * RB;
+    const uint32_t at = lds0 + stage * STAGE_BYTES;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) panel_load16(wb, w_from[i], at + (16 * wave + 4 * i) * RB);
+#pragma unroll
+    for (int i = 0; i < X_LOADS; ++i) panel_load16(xb, x_from[i], at + W_BYTES + x_piece[i] * 1024);
+  };
+  f32x4 acc[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int s = 0; s < STAGES - 1; ++s) fetch(s, s);
+  int stage = 0;
+  for (int group = 0; group < groups; ++group) {
+    panel_wait<(STAGES - 2) * LOADS>();                    // this group has arrived; the later ones may be on their way
+    __syncthreads();                                       // everybody's part of it too; the group before is done with
+    fetch(group + STAGES - 1, stage == 0 ? STAGES - 1 : stage - 1);
+    const unsigned char* ws = panel_lds + stage * STAGE_BYTES + (16 * wave + c) * RB;
+    const unsigned char* xs = panel_lds + stage * STAGE_BYTES + W_BYTES + c * RB;
+#pragma unroll
+    for (int u = 0; u < PANEL_GROUP / 32; ++u) {           // 32 values of K at a time
+      const int place = ((4 * u + g) ^ c) << 4;            // row 16 t + c of any tile is swizzled like row c
+      const bf16x8 a = *(const bf16x8*)(ws + place);
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        const bf16x8 b = *(const bf16x8*)(xs + 16 * mt * RB + place);
+        acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[mt], 0, 0, 0);
+      }
+    }
+    stage = stage + 1 == STAGES ? 0 : stage + 1;
+  }
+  panel_wait<0>();                                         // the loads past the end have landed before LDS is reused
+  __syncthreads();                                         // the stages are free: up passes through them
+  // acc[mt][i] is output n0 + 4g + i of activation row 16 mt + c, gate in waves 0 to 2 and up in waves 3 to 5
+  f32x4 (*pass)[MT][WAVE] = (f32x4 (*)[MT][WAVE])panel_lds;
+  if (wave >= HALF) {
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) pass[wave - HALF][mt][lane] = acc[mt];
+  }
+  __syncthreads();
+  if (wave >= HALF) return;
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const f32x4 up = pass[wave][mt][lane];
+    const int m = 16 * mt + c;
+    if (m >= M) continue;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int n = n0 + 4 * g + i;
+      if (n >= N) continue;
+      const float gv = rounded_as<bf16_t>(acc[mt][i]), uv = rounded_as<bf16_t>(up[i]);
+      const float sv = rounded_as<bf16_t>(gv / (1.f + expf(-gv)));
+      store_from_float(y + (int64_t)m * N + n, sv * uv);
+    }
+  }
+}
+
+template <int MT>
+static int launch_panel_swiglu(const void* x, int64_t x_stride, const void* w, void* y, int M, int N, int K,
+                               hipStream_t stream) {
+  constexpr int lds = PANEL_STAGES * (16 * PANEL_WAVES + 16 * MT) * 2 * PANEL_GROUP;
+  static_assert(lds <= 160 * 1024, "the stages must fit a compute unit's LDS");
+  static bool raised = false;                              // more dynamic LDS than the default limit allows
+  auto kernel = gemm_panel_swiglu_kernel<MT>;
+  if (lds > 64 * 1024 && !raised) {
+    if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess) return -2;
+    raised = true;
+  }
+  dim3 grid((N + PANEL_OUTPUTS - 1) / PANEL_OUTPUTS), block(64 * PANEL_WAVES);
+  hipLaunchKernelGGL(kernel, grid, block, lds, stream, (const bf16_t*)x, x_stride, (const bf16_t*)w, (bf16_t*)y, M, N, K);
+  return DRYFT_LAUNCH_CHECK();
+}
+
+// M <= 64 (17 to 64 is what it is for). y[M, N] = T(T(silu(x . Wg^T)) * (x . Wu^T)) with W = [Wg; Wu] of 2N rows;
+// K a multiple of 128; x and W within reach of 32-bit byte offsets.
+DRYFT_API int dryft_gemm_panel_swiglu_bf16(const void* x, int64_t x_stride, const void* w, void* y, int M, int N, int K,
+                                           hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (M > 64 || K <= 0 || K % PANEL_GROUP || x_stride % 8 || (((uintptr_t)x | (uintptr_t)w) & 15) ||
+      (int64_t)2 * N * K * 2 >= (int64_t)4 << 30 || (int64_t)M * x_stride * 2 >= (int64_t)4 << 30)
+    return -1;
+  switch ((M + 15) / 16) {
+    case 1: return launch_panel_swiglu<1>(x, x_stride, w, y, M, N, K, stream);
+    case 2: return launch_panel_swiglu<2>(x, x_stride, w, y, M, N, K, stream);
+    case 3: return launch_panel_swiglu<3>(x, x_stride, w, y, M, N, K, stream);
+    default: return launch_panel_swiglu<4>(x, x_stride, w, y, M, N, K, stream);
+  }
+}
+
 // ------------------------------------------------------------------------------------------- block
 // Many rows: a workgroup owns a block of rows by outputs (128 x 128 with four waves, 256 x 256 with eight) and
 // walks K in steps of 64. Its threads copy the block's rows of x and of W for one step into LDS (whole cache

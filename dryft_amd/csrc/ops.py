@@ -38,6 +38,7 @@ _SIGNATURES = {
              "dryft_gemm_stream_bf16": [_P, _L, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
              "dryft_gemm_stream_swiglu_bf16": [_P, _L, _P, _P, _I, _I, _I, _I, _I, _P],
              "dryft_gemm_wide_bf16": [_P, _L, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
+             "dryft_gemm_panel_swiglu_bf16": [_P, _L, _P, _P, _I, _I, _I, _P],
              "dryft_gemm_block_bf16": [_P, _L, _P, _P, _I, _I, _I, _I, _I, _I, _P],
              "dryft_gemm_block_f32": [_P, _L, _P, _P, _I, _I, _I, _I, _P],
              "dryft_gemm_rows_f32": [_P, _L, _P, _P, _I, _I, _I, _P],
@@ -484,6 +485,29 @@ def gemm_wide_bf16(x, w, out, partials=None, group_blocks: int = 2, splits: int 
                  f"gemm_wide: out must be contiguous [{m},{n}]")
     _check(_fn("gemm", "dryft_gemm_wide_bf16")(_ptr(x), x.stride(0), _ptr(w), _ptr(out), _ptr(partials), m, n, k,
                                                int(group_blocks), int(depth), int(splits), out_f32, _stream()), "gemm_wide_bf16")
+
+
+PANEL_GROUP = 128     # values of K the panel kernel moves at a time; K must be a multiple of it
+PANEL_OUTPUTS = 48    # gate/up outputs one of its workgroups owns
+
+
+def gemm_panel_swiglu_bf16(x, w_gate_up, out) -> torch.Tensor:
+    """``silu(x @ Wg.T) * (x @ Wu.T)`` for ``w_gate_up = [Wg; Wu]``, at most 64 rows, by the kernel whose operands go
+    from memory straight into LDS. K must be a multiple of 128."""
+    _gpu(x, "x", torch.bfloat16)
+    _gpu(w_gate_up, "w_gate_up", torch.bfloat16)
+    _gpu(out, "out", torch.bfloat16)
+    m, k = x.shape
+    two_n = w_gate_up.shape[0]
+    _require(two_n % 2 == 0 and w_gate_up.shape == (two_n, k) and w_gate_up.is_contiguous() and x.stride(1) == 1,
+             "gemm_panel_swiglu: x [M,K] row-major, w [2N,K] contiguous")
+    _require(m <= 64 and k % PANEL_GROUP == 0 and x.stride(0) % 8 == 0,
+             f"gemm_panel_swiglu: needs M <= 64 and K % {PANEL_GROUP} == 0, got M={m} K={k}")
+    _require(x.data_ptr() % 16 == 0 and w_gate_up.data_ptr() % 16 == 0, "gemm_panel_swiglu: operands must be 16-byte aligned")
+    _require(out.shape == (m, two_n // 2) and out.is_contiguous(), f"gemm_panel_swiglu: out must be [{m},{two_n // 2}]")
+    _check(_fn("gemm", "dryft_gemm_panel_swiglu_bf16")(_ptr(x), x.stride(0), _ptr(w_gate_up), _ptr(out), m, two_n // 2, k,
+                                                       _stream()), "gemm_panel_swiglu_bf16")
+    return out
 
 
 def gemm_wide_swiglu_bf16(x, w_gate_up, out, group_blocks: int = 2, depth: int = 1) -> torch.Tensor:

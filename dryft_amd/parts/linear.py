@@ -10,6 +10,8 @@ engine/dryft_qwen3/model.py:153, 179-180, 237, 258-261). Here:
 * bfloat16, at most 16 rows (decoding at small batch): this library's weight-streaming
   matrix-core kernel, which stages whole cache lines through LDS and can leave its result
   as float32 partial sums over K for the consumer to add;
+* bfloat16, 17 to 64 rows, the fused gate/up product with its activation: this library's kernel that brings
+  its operands straight into LDS, where its workgroups all run at once (``panel_swiglu_ok``);
 * bfloat16, 17 to 64 rows: this library's shared-activation kernel where the consumer adds
   partial sums (the projections back to the hidden width, which give the vendor library too
   few tiles to fill the chip), where the result is wanted in float32 (the output head) and
@@ -68,6 +70,17 @@ def wide_plan(n: int, k: int, may_split: bool) -> tuple[int, int, int]:
 def few_rows_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
     """Can the few-row kernels read these operands? (16-byte pieces of rows.)"""
     return x.shape[1] % 8 == 0 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0
+
+
+def panel_swiglu_ok(x: torch.Tensor, w_gate_up: torch.Tensor) -> bool:
+    """Does the fused gate/up product for 17 to 64 rows go to the kernel that brings its operands straight into LDS?
+    It keeps one workgroup on a compute unit, so it pays while all of them run at once: measured against the vendor
+    library plus the activation kernel, 26 against 31 us at 64 rows and 22 against 27 at 24 to 32 rows on Qwen3-4B's
+    sizes (203 workgroups), 46 against 52 and 44 against 45 on Qwen3-8B's (256), no gain on Qwen3-32B's (534)."""
+    m, k = x.shape
+    outputs = w_gate_up.shape[0] // 2
+    return (STREAM_ROWS < m <= WIDE_ROWS and k % ops.PANEL_GROUP == 0 and few_rows_ok(x, w_gate_up)
+            and -(-outputs // ops.PANEL_OUTPUTS) <= _COMPUTE_UNITS)
 
 
 def linear(x: torch.Tensor, w: torch.Tensor, *, out_dtype: torch.dtype | None = None, allow_partials: bool = False):

@@ -11,7 +11,7 @@ import torch
 from ..csrc import ops
 from . import register_part
 from .base import FeedForward, matrix
-from .linear import STREAM_ROWS, linear, few_rows_ok
+from .linear import STREAM_ROWS, few_rows_ok, linear, panel_swiglu_ok
 
 
 class SwiGLU(FeedForward):
@@ -35,6 +35,8 @@ class SwiGLU(FeedForward):
         act = torch.empty((h.shape[0], self.inter), dtype=h.dtype, device=h.device)
         if h.dtype == torch.bfloat16 and h.shape[0] <= STREAM_ROWS and few_rows_ok(h, self.w_gate_up):
             ops.gemm_stream_swiglu_bf16(h, self.w_gate_up, act)       # product and activation in one kernel
+        elif h.dtype == torch.bfloat16 and panel_swiglu_ok(h, self.w_gate_up):
+            ops.gemm_panel_swiglu_bf16(h, self.w_gate_up, act)      # 17 to 64 rows: operands straight into LDS
         else:
             ops.silu_mul(linear(h, self.w_gate_up), act)
         return linear(act, self.w_down, allow_partials=True)

@@ -609,6 +609,28 @@ def test_gemm_wide_swiglu(m, inter, k, group):
     close(out, want, torch.bfloat16, what="wide swiglu")
 
 
+@pytest.mark.parametrize("m", [5, 17, 33, 48, 64])
+@pytest.mark.parametrize("inter,k", [(9728, 2560), (224, 128), (136, 384), (37 * 8, 640), (47, 128), (49, 256)])
+def test_gemm_panel_swiglu(m, inter, k):
+    """Operands straight into LDS: row counts with one to four tiles of 16, output counts that are no multiple of
+    the 48 a workgroup owns, one group of K and many; a row of x strided wider than K."""
+    torch.manual_seed(m + inter)
+    x = torch.randn(m, k).to(torch.bfloat16)
+    w = (torch.randn(2 * inter, k) * 2 / math.sqrt(k)).to(torch.bfloat16)
+    gu = (x.double() @ w.double().T).to(torch.bfloat16).float()            # the unfused path rounds the product first
+    want = (torch.nn.functional.silu(gu[:, :inter]).to(torch.bfloat16).float() * gu[:, inter:]).to(torch.bfloat16)
+    out = torch.full((m, inter), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ops().gemm_panel_swiglu_bf16(x.to(DEV), w.to(DEV), out)
+    close(out, want, torch.bfloat16, what="panel swiglu")
+    wide = torch.zeros(m, k + 8, dtype=torch.bfloat16, device=DEV)
+    wide[:, :k] = x.to(DEV)
+    out2 = torch.full((m, inter), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ops().gemm_panel_swiglu_bf16(wide[:, :k], w.to(DEV), out2)
+    assert torch.equal(out, out2)
+    with pytest.raises(Exception, match="K % 128"):
+        ops().gemm_panel_swiglu_bf16(x.to(DEV)[:, :64].contiguous(), w.to(DEV)[:, :64].contiguous(), out)
+
+
 @pytest.mark.parametrize("m,n,k", [(130, 331, 72), (1, 17, 8), (257, 128, 64), (300, 100, 1000), (128, 129, 136),
                                    (513, 2560, 2560), (64, 64, 9728)])
 @pytest.mark.parametrize("shape", [0, 1])
