@@ -545,8 +545,10 @@ DRYFT_API int dryft_gemm_wide_swiglu_bf16(const void* x, int64_t x_stride, const
 // that these loads write LDS; each wave waits for its own, then a barrier.
 // Measured beside it on Qwen3-4B's gate/up at 64 rows (26 us; the vendor library plus the activation kernel 31):
 // four waves and 32 outputs (304 workgroups, two rounds or shallow stages: 32 to 38 us), eight waves (28 to 34),
-// groups of 64 values (27 to 36), four stages (the same), weights and activations fetched by different waves with
-// depths of their own (26 at best). The plain product of the same form was no faster than what serves it now.
+// groups of 64 values (27 to 36), four or five stages (the same), weights and activations fetched by different waves
+// with depths of their own (26 at best). The plain product of the same form was no faster than what serves it now.
+// Walking K from a different starting group in every workgroup took Qwen3-8B's gate/up (rows 8,192 bytes apart)
+// from 44 to 38 us at 8 to 40 rows; at Qwen3-4B's 5,120 bytes it changes nothing.
 __device__ __forceinline__ void panel_load16(const void* base, uint32_t offset, uint32_t lds_base) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_base), "v"(offset), "s"(base) : "memory");
 }
@@ -564,14 +566,14 @@ __device__ __forceinline__ void panel_wait() {
 #define PANEL_STAGES 3
 #define PANEL_OUTPUTS (8 * PANEL_WAVES)      // of a workgroup
 
-template <int MT>
+template <int MT, int STAGES>
 __global__ __launch_bounds__(64 * PANEL_WAVES) void gemm_panel_swiglu_kernel(const bf16_t* __restrict__ x,
                                                                              int64_t x_stride,
                                                                              const bf16_t* __restrict__ w,
                                                                              bf16_t* __restrict__ y, int M, int N,
                                                                              int K) {
   extern __shared__ __align__(16) unsigned char panel_lds[];
-  constexpr int WAVES = PANEL_WAVES, STAGES = PANEL_STAGES, HALF = WAVES / 2;
+  constexpr int WAVES = PANEL_WAVES, HALF = WAVES / 2;
   constexpr int RB = 2 * PANEL_GROUP;                      // bytes of a row in a group
   constexpr int X_ALL = 4 * MT;                            // 1 KB pieces of x in a group, dealt to the waves in turn
   constexpr int X_LOADS = (X_ALL + WAVES - 1) / WAVES;     // every wave issues this many
@@ -598,8 +600,12 @@ __global__ __launch_bounds__(64 * PANEL_WAVES) void gemm_panel_swiglu_kernel(con
     x_from[i] = (uint32_t)min(r, M - 1) * (uint32_t)x_stride * 2u + (((lane % 16) ^ (r & 15)) << 4);
   }
   const uint32_t lds0 = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)panel_lds);
+  // Workgroups walk K from different starting groups (and wrap around): at a row stride that is a multiple of the
+  // memory channels' interleave, all of them asking for the same columns at the same time would queue on one channel.
+  const int first_group = (int)((blockIdx.x * 5u) % (unsigned)groups);
   auto fetch = [&](int group, int stage) {
-    const int gk = min(group, groups - 1);                 // past the end: the last group again, into a free buffer
+    int gk = min(group, groups - 1) + first_group;         // past the end: the last group again, into a free buffer
+    gk = gk >= groups ? gk - groups : gk;
     const unsigned char* wb = (const unsigned char*)w + (int64_t)gk * RB;
     const unsigned char* xb = (const unsigned char*)x + (int64_t)gk * RB;
     const uint32_t at = lds0 + stage * STAGE_BYTES;
@@ -658,13 +664,13 @@ __global__ __launch_bounds__(64 * PANEL_WAVES) void gemm_panel_swiglu_kernel(con
   }
 }
 
-template <int MT>
+template <int MT, int STAGES>
 static int launch_panel_swiglu(const void* x, int64_t x_stride, const void* w, void* y, int M, int N, int K,
                                hipStream_t stream) {
-  constexpr int lds = PANEL_STAGES * (16 * PANEL_WAVES + 16 * MT) * 2 * PANEL_GROUP;
+  constexpr int lds = STAGES * (16 * PANEL_WAVES + 16 * MT) * 2 * PANEL_GROUP;
   static_assert(lds <= 160 * 1024, "the stages must fit a compute unit's LDS");
   static bool raised = false;                              // more dynamic LDS than the default limit allows
-  auto kernel = gemm_panel_swiglu_kernel<MT>;
+  auto kernel = gemm_panel_swiglu_kernel<MT, STAGES>;
   if (lds > 64 * 1024 && !raised) {
     if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess) return -2;
     raised = true;
@@ -683,10 +689,10 @@ DRYFT_API int dryft_gemm_panel_swiglu_bf16(const void* x, int64_t x_stride, cons
       (int64_t)2 * N * K * 2 >= (int64_t)4 << 30 || (int64_t)M * x_stride * 2 >= (int64_t)4 << 30)
     return -1;
   switch ((M + 15) / 16) {
-    case 1: return launch_panel_swiglu<1>(x, x_stride, w, y, M, N, K, stream);
-    case 2: return launch_panel_swiglu<2>(x, x_stride, w, y, M, N, K, stream);
-    case 3: return launch_panel_swiglu<3>(x, x_stride, w, y, M, N, K, stream);
-    default: return launch_panel_swiglu<4>(x, x_stride, w, y, M, N, K, stream);
+    case 1: return launch_panel_swiglu<1, PANEL_STAGES>(x, x_stride, w, y, M, N, K, stream);
+    case 2: return launch_panel_swiglu<2, PANEL_STAGES>(x, x_stride, w, y, M, N, K, stream);
+    case 3: return launch_panel_swiglu<3, PANEL_STAGES>(x, x_stride, w, y, M, N, K, stream);
+    default: return launch_panel_swiglu<4, PANEL_STAGES>(x, x_stride, w, y, M, N, K, stream);
   }
 }
 

@@ -76,7 +76,7 @@ def panel_swiglu_ok(x: torch.Tensor, w_gate_up: torch.Tensor) -> bool:
     """Does the fused gate/up product for 17 to 64 rows go to the kernel that brings its operands straight into LDS?
     It keeps one workgroup on a compute unit, so it pays while all of them run at once: measured against the vendor
     library plus the activation kernel, 26 against 31 us at 64 rows and 22 against 27 at 24 to 32 rows on Qwen3-4B's
-    sizes (203 workgroups), 46 against 52 and 44 against 45 on Qwen3-8B's (256), no gain on Qwen3-32B's (534)."""
+    sizes (203 workgroups), 39 to 40 against 46 to 52 on Qwen3-8B's (256), no gain on Qwen3-32B's (534)."""
     m, k = x.shape
     outputs = w_gate_up.shape[0] // 2
     return (STREAM_ROWS < m <= WIDE_ROWS and k % ops.PANEL_GROUP == 0 and few_rows_ok(x, w_gate_up)
