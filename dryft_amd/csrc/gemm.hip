@@ -533,13 +533,13 @@ DRYFT_API int dryft_gemm_wide_swiglu_bf16(const void* x, int64_t x_stride, const
 // ------------------------------------------------------------------------------------------- panel
 // The fused gate/up product with its activation for 17 to 64 rows, with the operands going from memory straight
 // into LDS (global_load_lds_dwordx4: 16 bytes a lane, no registers in between and nothing for the waves to store),
-// two groups of K ahead of the one that is multiplied. A workgroup of six waves owns 48 outputs: waves 0 to 2 hold
-// 16 gate rows each, waves 3 to 5 the up rows of the same outputs, and all MT tiles of 16 rows of x. A group is
+// two groups of K ahead of the one that is multiplied. A workgroup of four to eight waves owns 8 outputs a wave
+// (each wave the gate rows and the up rows of its own) and all MT tiles of 16 rows of x. A group is
 // 128 values of K: 256 bytes of every row, 16 pieces of 16 bytes, piece p of row r at place p ^ (r % 16), so that
 // operand reads meet no bank twice without padding; which piece a lane fetches is what places it. One instruction
 // fills 1 KB (four rows); a wave fetches its own 16 weight rows (four instructions) and its share of the rows of x
 // (dealt to the waves in turn; every wave issues the same number, the last piece again if need be). Three groups
-// have room in LDS (120 KB at 64 rows: one workgroup a compute unit). Every wave issues the same number of loads
+// have room in LDS (120 KB at 64 rows and six waves: one workgroup a compute unit). Every wave issues the same number of loads
 // per group, also past the end of K (the last group again, into a buffer nobody reads), so one constant says how
 // many may still be in flight when a group is needed. K must be a multiple of 128. The compiler does not know
 // that these loads write LDS; each wave waits for its own, then a barrier.
@@ -562,18 +562,17 @@ __device__ __forceinline__ void panel_wait() {
 }
 
 #define PANEL_GROUP 128                      // values of K in a group; K must be a multiple of it
-#define PANEL_WAVES 6
 #define PANEL_STAGES 3
-#define PANEL_OUTPUTS (8 * PANEL_WAVES)      // of a workgroup
 
-template <int MT, int STAGES>
-__global__ __launch_bounds__(64 * PANEL_WAVES) void gemm_panel_swiglu_kernel(const bf16_t* __restrict__ x,
-                                                                             int64_t x_stride,
-                                                                             const bf16_t* __restrict__ w,
-                                                                             bf16_t* __restrict__ y, int M, int N,
-                                                                             int K) {
+// WAVES waves, 8 outputs each: a wave's 16 weight rows are the gate rows of its 8 outputs and then their up rows, so
+// that gate and up of an output meet in lanes 32 apart and no LDS pass is needed at the end. The launcher picks
+// WAVES so that the workgroups are about as many as the compute units and all run at once.
+template <int MT, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void gemm_panel_swiglu_kernel(const bf16_t* __restrict__ x, int64_t x_stride,
+                                                                       const bf16_t* __restrict__ w,
+                                                                       bf16_t* __restrict__ y, int M, int N, int K) {
   extern __shared__ __align__(16) unsigned char panel_lds[];
-  constexpr int WAVES = PANEL_WAVES, HALF = WAVES / 2;
+  constexpr int STAGES = PANEL_STAGES;
   constexpr int RB = 2 * PANEL_GROUP;                      // bytes of a row in a group
   constexpr int X_ALL = 4 * MT;                            // 1 KB pieces of x in a group, dealt to the waves in turn
   constexpr int X_LOADS = (X_ALL + WAVES - 1) / WAVES;     // every wave issues this many
@@ -581,17 +580,16 @@ __global__ __launch_bounds__(64 * PANEL_WAVES) void gemm_panel_swiglu_kernel(con
   constexpr int W_BYTES = 16 * WAVES * RB, X_BYTES = 16 * MT * RB, STAGE_BYTES = W_BYTES + X_BYTES;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
   const int lane = threadIdx.x % WAVE, c = lane % 16, g = lane / 16;
-  const int n0 = blockIdx.x * PANEL_OUTPUTS + 16 * (wave % HALF);                 // first output of this wave
-  const int w_row0 = (wave >= HALF ? N : 0) + n0;          // its first weight row (W = [Wg; Wu])
-  const int w_last = (wave >= HALF ? 2 * N : N) - 1;
+  const int n0 = (blockIdx.x * WAVES + wave) * 8;          // first output of this wave
   const int groups = K / PANEL_GROUP;
   // where this lane fetches: its place within an instruction's 1 KB is fixed, the piece that belongs there follows
   uint32_t w_from[4], x_from[X_LOADS];
   int x_piece[X_LOADS];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    const int r = 4 * i + lane / 16;                       // row within the wave's 16
-    w_from[i] = (uint32_t)min(w_row0 + r, w_last) * (uint32_t)K * 2u + (((lane % 16) ^ r) << 4);
+    const int r = 4 * i + lane / 16;                       // row within the wave's 16: 0..7 gate, 8..15 up
+    const int row = (r < 8 ? 0 : N) + min(n0 + (r & 7), N - 1);
+    w_from[i] = (uint32_t)row * (uint32_t)K * 2u + (((lane % 16) ^ r) << 4);
   }
 #pragma unroll
   for (int i = 0; i < X_LOADS; ++i) {
@@ -638,61 +636,85 @@ __global__ __launch_bounds__(64 * PANEL_WAVES) void gemm_panel_swiglu_kernel(con
     }
     stage = stage + 1 == STAGES ? 0 : stage + 1;
   }
-  panel_wait<0>();                                         // the loads past the end have landed before LDS is reused
-  __syncthreads();                                         // the stages are free: up passes through them
-  // acc[mt][i] is output n0 + 4g + i of activation row 16 mt + c, gate in waves 0 to 2 and up in waves 3 to 5
-  f32x4 (*pass)[MT][WAVE] = (f32x4 (*)[MT][WAVE])panel_lds;
-  if (wave >= HALF) {
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) pass[wave - HALF][mt][lane] = acc[mt];
-  }
-  __syncthreads();
-  if (wave >= HALF) return;
+  panel_wait<0>();                                         // the loads past the end have landed before the waves leave
+  // acc[mt][i] is row 4g + i of the wave's 16 for activation row 16 mt + c: gate of output 4g + i in lanes with
+  // g < 2, its up 32 lanes further on
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
-    const f32x4 up = pass[wave][mt][lane];
     const int m = 16 * mt + c;
-    if (m >= M) continue;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
+      const float up = __shfl_xor(acc[mt][i], 32, WAVE);
       const int n = n0 + 4 * g + i;
-      if (n >= N) continue;
-      const float gv = rounded_as<bf16_t>(acc[mt][i]), uv = rounded_as<bf16_t>(up[i]);
+      if (g >= 2 || m >= M || n >= N) continue;
+      const float gv = rounded_as<bf16_t>(acc[mt][i]), uv = rounded_as<bf16_t>(up);
       const float sv = rounded_as<bf16_t>(gv / (1.f + expf(-gv)));
       store_from_float(y + (int64_t)m * N + n, sv * uv);
     }
   }
 }
 
-template <int MT, int STAGES>
+template <int MT, int WAVES>
 static int launch_panel_swiglu(const void* x, int64_t x_stride, const void* w, void* y, int M, int N, int K,
                                hipStream_t stream) {
-  constexpr int lds = STAGES * (16 * PANEL_WAVES + 16 * MT) * 2 * PANEL_GROUP;
+  constexpr int lds = PANEL_STAGES * (16 * WAVES + 16 * MT) * 2 * PANEL_GROUP;
   static_assert(lds <= 160 * 1024, "the stages must fit a compute unit's LDS");
   static bool raised = false;                              // more dynamic LDS than the default limit allows
-  auto kernel = gemm_panel_swiglu_kernel<MT, STAGES>;
+  auto kernel = gemm_panel_swiglu_kernel<MT, WAVES>;
   if (lds > 64 * 1024 && !raised) {
     if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess) return -2;
     raised = true;
   }
-  dim3 grid((N + PANEL_OUTPUTS - 1) / PANEL_OUTPUTS), block(64 * PANEL_WAVES);
+  dim3 grid((N + 8 * WAVES - 1) / (8 * WAVES)), block(64 * WAVES);
   hipLaunchKernelGGL(kernel, grid, block, lds, stream, (const bf16_t*)x, x_stride, (const bf16_t*)w, (bf16_t*)y, M, N, K);
   return DRYFT_LAUNCH_CHECK();
 }
 
-// M <= 64 (17 to 64 is what it is for). y[M, N] = T(T(silu(x . Wg^T)) * (x . Wu^T)) with W = [Wg; Wu] of 2N rows;
-// K a multiple of 128; x and W within reach of 32-bit byte offsets.
+template <int MT>
+static int panel_waves(const void* x, int64_t x_stride, const void* w, void* y, int M, int N, int K, int waves,
+                       hipStream_t stream) {
+  switch (waves) {
+    case 4: return launch_panel_swiglu<MT, 4>(x, x_stride, w, y, M, N, K, stream);
+    case 5: return launch_panel_swiglu<MT, 5>(x, x_stride, w, y, M, N, K, stream);
+    case 6: return launch_panel_swiglu<MT, 6>(x, x_stride, w, y, M, N, K, stream);
+    case 7: return launch_panel_swiglu<MT, 7>(x, x_stride, w, y, M, N, K, stream);
+    case 8: return launch_panel_swiglu<MT, 8>(x, x_stride, w, y, M, N, K, stream);
+    default: return -1;
+  }
+}
+
+// How many waves a workgroup gets for N outputs (8 outputs a wave): from four to eight, the count whose workgroups
+// fill whole rounds of the 256 compute units best (one workgroup runs on a unit at a time); among equals the fewest.
+// Qwen3-4B's 9,728 outputs: 5 waves, 244 workgroups; Qwen3-8B's 12,288: 6 waves, 256; Qwen3-32B's 25,600: 7 waves,
+// 458 in two rounds (measured best in each case).
+DRYFT_API int dryft_gemm_panel_waves(int N) {
+  int best = 4;
+  double best_fill = 0.0;
+  for (int waves = 4; waves <= 8; ++waves) {
+    const int groups = (N + 8 * waves - 1) / (8 * waves), rounds = (groups + 255) / 256;
+    const double fill = (double)groups / (256.0 * rounds);
+    if (fill > best_fill + 1e-9) {
+      best_fill = fill;
+      best = waves;
+    }
+  }
+  return best;
+}
+
+// M <= 64. y[M, N] = T(T(silu(x . Wg^T)) * (x . Wu^T)) with W = [Wg; Wu] of 2N rows; K a multiple of 128; x and W
+// within reach of 32-bit byte offsets; waves: 4 to 8, or 0 for dryft_gemm_panel_waves' choice.
 DRYFT_API int dryft_gemm_panel_swiglu_bf16(const void* x, int64_t x_stride, const void* w, void* y, int M, int N, int K,
-                                           hipStream_t stream) {
+                                           int waves, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (M > 64 || K <= 0 || K % PANEL_GROUP || x_stride % 8 || (((uintptr_t)x | (uintptr_t)w) & 15) ||
       (int64_t)2 * N * K * 2 >= (int64_t)4 << 30 || (int64_t)M * x_stride * 2 >= (int64_t)4 << 30)
     return -1;
+  if (waves == 0) waves = dryft_gemm_panel_waves(N);
   switch ((M + 15) / 16) {
-    case 1: return launch_panel_swiglu<1, PANEL_STAGES>(x, x_stride, w, y, M, N, K, stream);
-    case 2: return launch_panel_swiglu<2, PANEL_STAGES>(x, x_stride, w, y, M, N, K, stream);
-    case 3: return launch_panel_swiglu<3, PANEL_STAGES>(x, x_stride, w, y, M, N, K, stream);
-    default: return launch_panel_swiglu<4, PANEL_STAGES>(x, x_stride, w, y, M, N, K, stream);
+    case 1: return panel_waves<1>(x, x_stride, w, y, M, N, K, waves, stream);
+    case 2: return panel_waves<2>(x, x_stride, w, y, M, N, K, waves, stream);
+    case 3: return panel_waves<3>(x, x_stride, w, y, M, N, K, waves, stream);
+    default: return panel_waves<4>(x, x_stride, w, y, M, N, K, waves, stream);
   }
 }
 

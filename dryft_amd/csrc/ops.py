@@ -38,7 +38,8 @@ _SIGNATURES = {
              "dryft_gemm_stream_bf16": [_P, _L, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
              "dryft_gemm_stream_swiglu_bf16": [_P, _L, _P, _P, _I, _I, _I, _I, _I, _P],
              "dryft_gemm_wide_bf16": [_P, _L, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
-             "dryft_gemm_panel_swiglu_bf16": [_P, _L, _P, _P, _I, _I, _I, _P],
+             "dryft_gemm_panel_swiglu_bf16": [_P, _L, _P, _P, _I, _I, _I, _I, _P],
+             "dryft_gemm_panel_waves": [_I],
              "dryft_gemm_block_bf16": [_P, _L, _P, _P, _I, _I, _I, _I, _I, _I, _P],
              "dryft_gemm_block_f32": [_P, _L, _P, _P, _I, _I, _I, _I, _P],
              "dryft_gemm_rows_f32": [_P, _L, _P, _P, _I, _I, _I, _P],
@@ -488,12 +489,17 @@ def gemm_wide_bf16(x, w, out, partials=None, group_blocks: int = 2, splits: int 
 
 
 PANEL_GROUP = 128     # values of K the panel kernel moves at a time; K must be a multiple of it
-PANEL_OUTPUTS = 48    # gate/up outputs one of its workgroups owns
 
 
-def gemm_panel_swiglu_bf16(x, w_gate_up, out) -> torch.Tensor:
+def gemm_panel_waves(n_outputs: int) -> int:
+    """Waves per workgroup (8 outputs each) that the panel kernel chooses for this many outputs."""
+    return int(_fn("gemm", "dryft_gemm_panel_waves")(int(n_outputs)))
+
+
+def gemm_panel_swiglu_bf16(x, w_gate_up, out, waves: int = 0) -> torch.Tensor:
     """``silu(x @ Wg.T) * (x @ Wu.T)`` for ``w_gate_up = [Wg; Wu]``, at most 64 rows, by the kernel whose operands go
-    from memory straight into LDS. K must be a multiple of 128."""
+    from memory straight into LDS. K must be a multiple of 128. ``waves`` (4 to 8, 8 outputs each) per workgroup;
+    0 lets the library choose."""
     _gpu(x, "x", torch.bfloat16)
     _gpu(w_gate_up, "w_gate_up", torch.bfloat16)
     _gpu(out, "out", torch.bfloat16)
@@ -505,8 +511,9 @@ def gemm_panel_swiglu_bf16(x, w_gate_up, out) -> torch.Tensor:
              f"gemm_panel_swiglu: needs M <= 64 and K % {PANEL_GROUP} == 0, got M={m} K={k}")
     _require(x.data_ptr() % 16 == 0 and w_gate_up.data_ptr() % 16 == 0, "gemm_panel_swiglu: operands must be 16-byte aligned")
     _require(out.shape == (m, two_n // 2) and out.is_contiguous(), f"gemm_panel_swiglu: out must be [{m},{two_n // 2}]")
+    _require(waves == 0 or 4 <= waves <= 8, "gemm_panel_swiglu: waves 4 to 8, or 0")
     _check(_fn("gemm", "dryft_gemm_panel_swiglu_bf16")(_ptr(x), x.stride(0), _ptr(w_gate_up), _ptr(out), m, two_n // 2, k,
-                                                       _stream()), "gemm_panel_swiglu_bf16")
+                                                       int(waves), _stream()), "gemm_panel_swiglu_bf16")
     return out
 
 

@@ -10,8 +10,8 @@ engine/dryft_qwen3/model.py:153, 179-180, 237, 258-261). Here:
 * bfloat16, at most 16 rows (decoding at small batch): this library's weight-streaming
   matrix-core kernel, which stages whole cache lines through LDS and can leave its result
   as float32 partial sums over K for the consumer to add;
-* bfloat16, 17 to 64 rows, the fused gate/up product with its activation: this library's kernel that brings
-  its operands straight into LDS, where its workgroups all run at once (``panel_swiglu_ok``);
+* bfloat16, at most 64 rows, the fused gate/up product with its activation: this library's kernel that brings
+  its operands straight into LDS (``panel_swiglu_ok``; K a multiple of 128, else the two kernels below);
 * bfloat16, 17 to 64 rows: this library's shared-activation kernel where the consumer adds
   partial sums (the projections back to the hidden width, which give the vendor library too
   few tiles to fill the chip), where the result is wanted in float32 (the output head) and
@@ -73,14 +73,14 @@ def few_rows_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
 
 
 def panel_swiglu_ok(x: torch.Tensor, w_gate_up: torch.Tensor) -> bool:
-    """Does the fused gate/up product for 17 to 64 rows go to the kernel that brings its operands straight into LDS?
-    It keeps one workgroup on a compute unit, so it pays while all of them run at once: measured against the vendor
-    library plus the activation kernel, 26 against 31 us at 64 rows and 22 against 27 at 24 to 32 rows on Qwen3-4B's
-    sizes (203 workgroups), 39 to 40 against 46 to 52 on Qwen3-8B's (256), no gain on Qwen3-32B's (534)."""
+    """Does the fused gate/up product with its activation go to the kernel that brings its operands straight into
+    LDS? Up to 64 rows, K a multiple of its group. In-graph times on rotating cold weights, us, against the
+    line-staging kernel (up to 16 rows) or the vendor library plus the activation kernel (more): Qwen3-4B's sizes
+    20.3 against 21.5 at 8 rows, 20.3 against 22.4 at 16, 21.2 against 26.8 at 24, 24.9 against 30.7 at 64;
+    Qwen3-8B's 36.7 against 37.8, 36.8 against 38.0, 37.6 against 52.1, 39.9 against 52.7; Qwen3-32B's 96.9 against
+    98.4, 95.0 against 103.8, 97.6 against 100.9, 107.8 against 110.4."""
     m, k = x.shape
-    outputs = w_gate_up.shape[0] // 2
-    return (STREAM_ROWS < m <= WIDE_ROWS and k % ops.PANEL_GROUP == 0 and few_rows_ok(x, w_gate_up)
-            and -(-outputs // ops.PANEL_OUTPUTS) <= _COMPUTE_UNITS)
+    return m <= WIDE_ROWS and k % ops.PANEL_GROUP == 0 and few_rows_ok(x, w_gate_up)
 
 
 def linear(x: torch.Tensor, w: torch.Tensor, *, out_dtype: torch.dtype | None = None, allow_partials: bool = False):

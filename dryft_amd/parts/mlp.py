@@ -33,10 +33,10 @@ class SwiGLU(FeedForward):
 
     def forward(self, h, ctx):
         act = torch.empty((h.shape[0], self.inter), dtype=h.dtype, device=h.device)
-        if h.dtype == torch.bfloat16 and h.shape[0] <= STREAM_ROWS and few_rows_ok(h, self.w_gate_up):
-            ops.gemm_stream_swiglu_bf16(h, self.w_gate_up, act)       # product and activation in one kernel
-        elif h.dtype == torch.bfloat16 and panel_swiglu_ok(h, self.w_gate_up):
-            ops.gemm_panel_swiglu_bf16(h, self.w_gate_up, act)      # 17 to 64 rows: operands straight into LDS
+        if h.dtype == torch.bfloat16 and panel_swiglu_ok(h, self.w_gate_up):
+            ops.gemm_panel_swiglu_bf16(h, self.w_gate_up, act)        # product and activation in one kernel
+        elif h.dtype == torch.bfloat16 and h.shape[0] <= STREAM_ROWS and few_rows_ok(h, self.w_gate_up):
+            ops.gemm_stream_swiglu_bf16(h, self.w_gate_up, act)       # the same for any K that is a multiple of 8
         else:
             ops.silu_mul(linear(h, self.w_gate_up), act)
         return linear(act, self.w_down, allow_partials=True)
