@@ -543,7 +543,8 @@ DRYFT_API int dryft_gemm_wide_swiglu_bf16(const void* x, int64_t x_stride, const
 // per group, also past the end of K (the last group again, into a buffer nobody reads), so one constant says how
 // many may still be in flight when a group is needed. K must be a multiple of 128. The compiler does not know
 // that these loads write LDS; each wave waits for its own, then a barrier.
-// Measured beside it on Qwen3-4B's gate/up at 64 rows (26 us; the vendor library plus the activation kernel 31):
+// Measured beside it on Qwen3-4B's gate/up at 64 rows (26 us, 24.4 since the operand reads are ordered by hand; the
+// vendor library plus the activation kernel 30 to 31):
 // four waves and 32 outputs (304 workgroups, two rounds or shallow stages: 32 to 38 us), eight waves (28 to 34),
 // groups of 64 values (27 to 36), four or five stages (the same), weights and activations fetched by different waves
 // with depths of their own (26 at best). The plain product of the same form was no faster than what serves it now.
@@ -624,15 +625,38 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_panel_swiglu_kernel(const bf1
     fetch(group + STAGES - 1, stage == 0 ? STAGES - 1 : stage - 1);
     const unsigned char* ws = panel_lds + stage * STAGE_BYTES + (16 * wave + c) * RB;
     const unsigned char* xs = panel_lds + stage * STAGE_BYTES + W_BYTES + c * RB;
+    constexpr int US = PANEL_GROUP / 32;                   // 32 values of K at a time
+    bf16x8 a[US], b[US][MT];
 #pragma unroll
-    for (int u = 0; u < PANEL_GROUP / 32; ++u) {           // 32 values of K at a time
+    for (int u = 0; u < US; ++u) {
       const int place = ((4 * u + g) ^ c) << 4;            // row 16 t + c of any tile is swizzled like row c
-      const bf16x8 a = *(const bf16x8*)(ws + place);
+      a[u] = *(const bf16x8*)(ws + place);
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
-        const bf16x8 b = *(const bf16x8*)(xs + 16 * mt * RB + place);
-        acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[mt], 0, 0, 0);
+      for (int mt = 0; mt < MT; ++mt) b[u][mt] = *(const bf16x8*)(xs + 16 * mt * RB + place);
+    }
+#pragma unroll
+    for (int u = 0; u < US; ++u)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u], b[u][mt], acc[mt], 0, 0, 0);
+    // The order the scheduler is to keep (left alone it reads two operands, waits, multiplies, and so on, and every
+    // wait shows): the first quarter's reads; each quarter's matrix instructions with the next quarter's reads
+    // between them; the last quarter's matrix instructions. 0x100: LDS reads, 0x008: matrix instructions.
+    // With one or two tiles of rows all reads of the group go first.
+    if (MT <= 2) {
+      __builtin_amdgcn_sched_group_barrier(0x100, US * (MT + 1), 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, US * MT, 0);
+    } else {
+      __builtin_amdgcn_sched_group_barrier(0x100, MT + 1, 0);
+#pragma unroll
+      for (int u = 0; u + 1 < US; ++u) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
       }
+      __builtin_amdgcn_sched_group_barrier(0x008, MT, 0);
     }
     stage = stage + 1 == STAGES ? 0 : stage + 1;
   }
