@@ -673,6 +673,18 @@ def test_real_layer_sizes_against_plain(real_cases, dtype, sharp):
     check_against_plain(case, got, dtype, "real sizes, 24 sequences")
 
 
+@pytest.mark.parametrize("seed,max_batch", [(2000, 40), (2001, 8)])
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_random_batches_at_real_layer_sizes(real_cases, dtype, seed, max_batch):
+    """Batches drawn at random (up to 40 requests, so that the decoding steps take every product for 1 to 64 rows),
+    at the sizes at which the matrix-core kernels take their fast paths, with sharpened attention."""
+    case = real_cases[True]
+    records = random_trace(case, seed, max_batch=max_batch)
+    engine = case.engine(dtype, max_batch=40, max_len=512, max_tokens=40 * 320)
+    got = collect_positions(records, replay(engine, records))
+    check_against_plain(case, got, dtype, f"random batches at real sizes, seed {seed}")
+
+
 # --------------------------------------------------------------------------------- the command line
 def run_cli(*argv, timeout=600):
     proc = subprocess.run([sys.executable, "-m", "dryft_amd", *argv], capture_output=True, text=True, timeout=timeout,
