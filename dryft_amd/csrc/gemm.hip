@@ -531,7 +531,7 @@ DRYFT_API int dryft_gemm_wide_swiglu_bf16(const void* x, int64_t x_stride, const
 }
 
 // ------------------------------------------------------------------------------------------- panel
-// The fused gate/up product with its activation for 17 to 64 rows, with the operands going from memory straight
+// The fused gate/up product with its activation for steps of up to 64 rows, with the operands going from memory straight
 // into LDS (global_load_lds_dwordx4: 16 bytes a lane, no registers in between and nothing for the waves to store),
 // two groups of K ahead of the one that is multiplied. A workgroup of four to eight waves owns 8 outputs a wave
 // (each wave the gate rows and the up rows of its own) and all MT tiles of 16 rows of x. A group is
