@@ -70,7 +70,13 @@ def preload(modules) -> None:
     build.ensure(list(modules))
 
 
+# the current stream's handle without building a stream object per launch (hundreds of launches a step)
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream() -> int:
+    if _raw_stream is not None:
+        return _raw_stream(torch.cuda.current_device())
     return torch.cuda.current_stream().cuda_stream
 
 
@@ -87,13 +93,16 @@ def _require(cond: bool, msg: str) -> None:
 
 
 def _gpu(t: torch.Tensor, name: str, dtype=None) -> None:
-    _require(isinstance(t, torch.Tensor) and t.is_cuda, f"{name}: must be a GPU tensor (there is no CPU path)")
+    if not (isinstance(t, torch.Tensor) and t.is_cuda):
+        raise KernelError(f"{name}: must be a GPU tensor (there is no CPU path)")
     if dtype is not None:
-        _require(t.dtype == dtype, f"{name}: expected {dtype}, got {t.dtype}")
+        if not (t.dtype == dtype):
+            raise KernelError(f"{name}: expected {dtype}, got {t.dtype}")
 
 
 def _float_flag(t: torch.Tensor, name: str) -> int:
-    _require(t.dtype in (torch.float32, torch.bfloat16), f"{name}: expected float32 or bfloat16, got {t.dtype}")
+    if not (t.dtype in (torch.float32, torch.bfloat16)):
+        raise KernelError(f"{name}: expected float32 or bfloat16, got {t.dtype}")
     return 1 if t.dtype == torch.float32 else 0
 
 
@@ -117,7 +126,8 @@ def prepare_batch(seq_slot, q_len, lengths, n_seqs: int, n_rows: int, cu_rows, t
                        ("row_seq", row_seq, n_rows), ("row_slot", row_slot, n_rows), ("row_pos", row_pos, n_rows),
                        ("lengths", lengths, 1)):
         _gpu(t, name, torch.int32)
-        _require(t.is_contiguous() and t.numel() >= n, f"{name}: needs {n} contiguous entries, has {t.numel()}")
+        if not (t.is_contiguous() and t.numel() >= n):
+            raise KernelError(f"{name}: needs {n} contiguous entries, has {t.numel()}")
     _check(_fn("batch", "dryft_prepare_batch")(
         _ptr(seq_slot), _ptr(q_len), _ptr(lengths), n_seqs, n_rows, ROW_TILE, _ptr(cu_rows), _ptr(tile_cu), _ptr(kv_len),
         _ptr(seq_start), _ptr(row_seq), _ptr(row_slot), _ptr(row_pos), _stream()), "prepare_batch")
@@ -129,8 +139,10 @@ def embed_rows(tokens: torch.Tensor, table: torch.Tensor, out: torch.Tensor) -> 
     _gpu(table, "table")
     _gpu(out, "out", table.dtype)
     n, (vocab, hidden) = tokens.numel(), table.shape
-    _require(table.is_contiguous() and out.is_contiguous() and tokens.is_contiguous(), "embed_rows: contiguous operands")
-    _require(out.shape == (n, hidden), f"embed_rows: out is {tuple(out.shape)}, expected {(n, hidden)}")
+    if not (table.is_contiguous() and out.is_contiguous() and tokens.is_contiguous()):
+        raise KernelError("embed_rows: contiguous operands")
+    if not (out.shape == (n, hidden)):
+        raise KernelError(f"embed_rows: out is {tuple(out.shape)}, expected {(n, hidden)}")
     _check(_fn("embed", "dryft_embed_rows")(_ptr(tokens), _ptr(table), _ptr(out), n, hidden, vocab,
                                             _float_flag(table, "table"), _stream()), "embed_rows")
     return out
@@ -149,21 +161,26 @@ def add_rmsnorm(res: torch.Tensor, delta, weight: torch.Tensor, eps: float, res_
     is_f32 = _float_flag(res, "res")
     _gpu(weight, "weight")
     w_f32 = _float_flag(weight, "weight")
-    _require(weight.shape == (width,) and weight.is_contiguous(), f"add_rmsnorm: weight must be [{width}]")
+    if not (weight.shape == (width,) and weight.is_contiguous()):
+        raise KernelError(f"add_rmsnorm: weight must be [{width}]")
     _gpu(y, "y", res.dtype)
-    _require(res.is_contiguous() and y.is_contiguous() and y.shape == res.shape, "add_rmsnorm: res and y contiguous, same shape")
+    if not (res.is_contiguous() and y.is_contiguous() and y.shape == res.shape):
+        raise KernelError("add_rmsnorm: res and y contiguous, same shape")
     kind, stride = 0, 0
     if delta is not None:
         _gpu(delta, "delta")
         _gpu(res_out, "res_out", res.dtype)
-        _require(res_out.shape == res.shape and res_out.is_contiguous(), "add_rmsnorm: res_out like res")
-        _require(delta.is_contiguous(), "add_rmsnorm: delta contiguous")
+        if not (res_out.shape == res.shape and res_out.is_contiguous()):
+            raise KernelError("add_rmsnorm: res_out like res")
+        if not (delta.is_contiguous()):
+            raise KernelError("add_rmsnorm: delta contiguous")
         if delta.dim() == 3:
-            _require(delta.dtype == torch.float32 and delta.shape[1:] == res.shape and delta.shape[0] >= n_partials,
-                     "add_rmsnorm: partial sums must be float32 [n, rows, width]")
+            if not (delta.dtype == torch.float32 and delta.shape[1:] == res.shape and delta.shape[0] >= n_partials):
+                raise KernelError("add_rmsnorm: partial sums must be float32 [n, rows, width]")
             kind, stride = 2, rows * width
         else:
-            _require(delta.dtype == res.dtype and delta.shape == res.shape, "add_rmsnorm: delta like res")
+            if not (delta.dtype == res.dtype and delta.shape == res.shape):
+                raise KernelError("add_rmsnorm: delta like res")
             kind, n_partials, stride = 1, 1, rows * width
     else:
         n_partials = 0
@@ -176,8 +193,8 @@ def add_rows(a: torch.Tensor, b: torch.Tensor, out: torch.Tensor) -> torch.Tenso
     _gpu(a, "a")
     _gpu(b, "b", a.dtype)
     _gpu(out, "out", a.dtype)
-    _require(a.shape == b.shape == out.shape and a.is_contiguous() and b.is_contiguous() and out.is_contiguous(),
-             "add_rows: contiguous operands of one shape")
+    if not (a.shape == b.shape == out.shape and a.is_contiguous() and b.is_contiguous() and out.is_contiguous()):
+        raise KernelError("add_rows: contiguous operands of one shape")
     _check(_fn("norm", "dryft_add_rows")(_ptr(a), _ptr(b), _ptr(out), a.numel(), _float_flag(a, "a"), _stream()),
            "add_rows")
     return out
@@ -188,8 +205,10 @@ def silu_mul(gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     _gpu(gate_up, "gate_up")
     _gpu(out, "out", gate_up.dtype)
     rows, two_i = gate_up.shape
-    _require(two_i % 2 == 0 and out.shape == (rows, two_i // 2), "silu_mul: out must be [rows, width / 2]")
-    _require(gate_up.stride(1) == 1 and out.is_contiguous(), "silu_mul: unit stride along the width")
+    if not (two_i % 2 == 0 and out.shape == (rows, two_i // 2)):
+        raise KernelError("silu_mul: out must be [rows, width / 2]")
+    if not (gate_up.stride(1) == 1 and out.is_contiguous()):
+        raise KernelError("silu_mul: unit stride along the width")
     _check(_fn("activation", "dryft_silu_mul")(_ptr(gate_up), _ptr(out), rows, two_i // 2, gate_up.stride(0),
                                                _float_flag(gate_up, "gate_up"), _stream()), "silu_mul")
     return out
@@ -205,29 +224,36 @@ def qk_norm_rope_kv(qkv: torch.Tensor, q_weight, k_weight, eps: float, cos, sin,
     is_f32 = _float_flag(qkv, "qkv")
     rows = qkv.shape[0]
     need_cols = (n_heads + (2 * n_kv if write_kv else 0)) * head_dim
-    _require(qkv.dim() == 2 and qkv.stride(1) == 1 and qkv.shape[1] >= need_cols,
-             f"qk_norm_rope_kv: qkv needs {need_cols} columns, has {tuple(qkv.shape)}")
+    if not (qkv.dim() == 2 and qkv.stride(1) == 1 and qkv.shape[1] >= need_cols):
+        raise KernelError(f"qk_norm_rope_kv: qkv needs {need_cols} columns, has {tuple(qkv.shape)}")
     has_norm = q_weight is not None
     w_f32 = 0
     if has_norm:
         for name, w in (("q_weight", q_weight), ("k_weight", k_weight)):
             _gpu(w, name)
-            _require(w.shape == (head_dim,) and w.is_contiguous(), f"{name}: must be [{head_dim}]")
-        _require(q_weight.dtype == k_weight.dtype, "q_weight and k_weight must share a dtype")
+            if not (w.shape == (head_dim,) and w.is_contiguous()):
+                raise KernelError(f"{name}: must be [{head_dim}]")
+        if not (q_weight.dtype == k_weight.dtype):
+            raise KernelError("q_weight and k_weight must share a dtype")
         w_f32 = _float_flag(q_weight, "q_weight")
     if rot:
-        _require(rot % 2 == 0 and rot <= head_dim, f"rotary width {rot} must be even and at most {head_dim}")
+        if not (rot % 2 == 0 and rot <= head_dim):
+            raise KernelError(f"rotary width {rot} must be even and at most {head_dim}")
         for name, t in (("cos", cos), ("sin", sin)):
             _gpu(t, name, qkv.dtype)
-            _require(t.dim() == 2 and t.shape[1] == rot // 2 and t.is_contiguous(), f"{name}: must be [positions, {rot // 2}]")
+            if not (t.dim() == 2 and t.shape[1] == rot // 2 and t.is_contiguous()):
+                raise KernelError(f"{name}: must be [positions, {rot // 2}]")
     for name, t in (("row_slot", row_slot), ("row_pos", row_pos)):
         _gpu(t, name, torch.int32)
-        _require(t.numel() >= rows and t.is_contiguous(), f"{name}: needs {rows} entries")
+        if not (t.numel() >= rows and t.is_contiguous()):
+            raise KernelError(f"{name}: needs {rows} entries")
     if q_out is not None:
         _gpu(q_out, "q_out", qkv.dtype)
-        _require(q_out.is_contiguous() and q_out.numel() == rows * n_heads * head_dim, "q_out: must be [rows, heads, head_dim]")
+        if not (q_out.is_contiguous() and q_out.numel() == rows * n_heads * head_dim):
+            raise KernelError("q_out: must be [rows, heads, head_dim]")
     else:
-        _require(write_kv, "qk_norm_rope_kv: nothing to do without q_out and without a cache to write")
+        if not (write_kv):
+            raise KernelError("qk_norm_rope_kv: nothing to do without q_out and without a cache to write")
     max_pages = 0
     if write_kv:
         _check_pages(k_pages, v_pages, page_table, n_kv, head_dim, qkv.dtype)
@@ -242,10 +268,11 @@ def qk_norm_rope_kv(qkv: torch.Tensor, q_weight, k_weight, eps: float, cos, sin,
 def _check_pages(k_pages, v_pages, page_table, n_kv: int, head_dim: int, dtype) -> None:
     for name, t in (("k_pages", k_pages), ("v_pages", v_pages)):
         _gpu(t, name, dtype)
-        _require(t.dim() == 4 and t.shape[1] == n_kv and t.shape[2] * t.shape[3] == 64 * head_dim and t.is_contiguous(),
-                 f"{name}: must be contiguous [pages, {n_kv}, 64, {head_dim}], got {tuple(t.shape)}")
+        if not (t.dim() == 4 and t.shape[1] == n_kv and t.shape[2] * t.shape[3] == 64 * head_dim and t.is_contiguous()):
+            raise KernelError(f"{name}: must be contiguous [pages, {n_kv}, 64, {head_dim}], got {tuple(t.shape)}")
     _gpu(page_table, "page_table", torch.int32)
-    _require(page_table.dim() == 2 and page_table.is_contiguous(), "page_table: must be contiguous [slots, pages]")
+    if not (page_table.dim() == 2 and page_table.is_contiguous()):
+        raise KernelError("page_table: must be contiguous [slots, pages]")
 
 
 # --------------------------------------------------------------------------------------- attention
@@ -254,14 +281,18 @@ def attn_rows(q, k_pages, v_pages, page_table, row_slot, row_pos, out, n_heads: 
     _gpu(q, "q")
     is_f32 = _float_flag(q, "q")
     rows = q.numel() // (n_heads * head_dim)
-    _require(q.is_contiguous() and q.numel() == rows * n_heads * head_dim, "attn_rows: q must be [rows, heads, head_dim]")
+    if not (q.is_contiguous() and q.numel() == rows * n_heads * head_dim):
+        raise KernelError("attn_rows: q must be [rows, heads, head_dim]")
     _gpu(out, "out", q.dtype)
-    _require(out.is_contiguous() and out.numel() == q.numel(), "attn_rows: out like q")
+    if not (out.is_contiguous() and out.numel() == q.numel()):
+        raise KernelError("attn_rows: out like q")
     _check_pages(k_pages, v_pages, page_table, n_kv, head_dim, q.dtype)
     for name, t in (("row_slot", row_slot), ("row_pos", row_pos)):
         _gpu(t, name, torch.int32)
-        _require(t.numel() >= rows, f"{name}: needs {rows} entries")
-    _require(n_heads <= 65535, "attn_rows: too many heads")
+        if not (t.numel() >= rows):
+            raise KernelError(f"{name}: needs {rows} entries")
+    if not (n_heads <= 65535):
+        raise KernelError("attn_rows: too many heads")
     _check(_fn("attn_rows", "dryft_attn_rows")(
         _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(page_table), page_table.shape[1], _ptr(row_slot), _ptr(row_pos),
         _ptr(out), rows, n_heads, n_kv, head_dim, float(scale), int(window), is_f32, _stream()), "attn_rows")
@@ -276,13 +307,16 @@ def attn_causal_bf16(q, k_pages, v_pages, page_table, seq_slot, cu_rows, tile_cu
     other head size."""
     _gpu(q, "q", torch.bfloat16)
     _gpu(out, "out", torch.bfloat16)
-    _require(q.is_contiguous() and out.is_contiguous() and out.numel() == q.numel(), "attn_causal: q and out contiguous")
+    if not (q.is_contiguous() and out.is_contiguous() and out.numel() == q.numel()):
+        raise KernelError("attn_causal: q and out contiguous")
     _check_pages(k_pages, v_pages, page_table, n_kv, head_dim, torch.bfloat16)
     for name, t, n in (("seq_slot", seq_slot, n_seqs), ("cu_rows", cu_rows, n_seqs + 1),
                        ("tile_cu", tile_cu, n_seqs + 1), ("seq_start", seq_start, n_seqs)):
         _gpu(t, name, torch.int32)
-        _require(t.numel() >= n, f"{name}: needs {n} entries")
-    _require(n_heads <= 65535, "attn_causal: too many heads")
+        if not (t.numel() >= n):
+            raise KernelError(f"{name}: needs {n} entries")
+    if not (n_heads <= 65535):
+        raise KernelError("attn_causal: too many heads")
     _check(_fn("attn_mfma", "dryft_attn_causal_bf16")(
         _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(page_table), page_table.shape[1], _ptr(seq_slot), _ptr(cu_rows),
         _ptr(tile_cu), _ptr(seq_start), n_seqs, max_tiles, _ptr(out), n_heads, n_kv, head_dim, float(scale),
@@ -303,25 +337,32 @@ def attn_causal_projected_bf16(qkv, q_weight, eps: float, cos, sin, k_pages, v_p
     _gpu(qkv, "qkv", torch.bfloat16)
     _gpu(out, "out", torch.bfloat16)
     rows = qkv.shape[0]
-    _require(qkv.dim() == 2 and qkv.stride(1) == 1 and qkv.shape[1] >= n_heads * head_dim and qkv.stride(0) % 8 == 0,
-             "attn_causal_projected: qkv must be [rows, >= heads * head_dim] with rows 16 bytes apart or a multiple")
-    _require(out.is_contiguous() and out.numel() == rows * n_heads * head_dim, "attn_causal_projected: out [rows, heads, head_dim]")
-    _require(attn_causal_takes_projection(head_dim, 2 * cos.shape[1] if cos is not None else 0),
-             "attn_causal_projected: the kernel refuses these sizes")
+    if not (qkv.dim() == 2 and qkv.stride(1) == 1 and qkv.shape[1] >= n_heads * head_dim and qkv.stride(0) % 8 == 0):
+        raise KernelError(
+            "attn_causal_projected: qkv must be [rows, >= heads * head_dim] with rows 16 bytes apart or a multiple"
+        )
+    if not (out.is_contiguous() and out.numel() == rows * n_heads * head_dim):
+        raise KernelError("attn_causal_projected: out [rows, heads, head_dim]")
+    if not (attn_causal_takes_projection(head_dim, 2 * cos.shape[1] if cos is not None else 0)):
+        raise KernelError("attn_causal_projected: the kernel refuses these sizes")
     w_f32 = 0
     if q_weight is not None:
         _gpu(q_weight, "q_weight")
-        _require(q_weight.shape == (head_dim,) and q_weight.is_contiguous(), f"q_weight: must be [{head_dim}]")
+        if not (q_weight.shape == (head_dim,) and q_weight.is_contiguous()):
+            raise KernelError(f"q_weight: must be [{head_dim}]")
         w_f32 = _float_flag(q_weight, "q_weight")
     for name, t in (("cos", cos), ("sin", sin)):
         _gpu(t, name, torch.bfloat16)
-        _require(t.dim() == 2 and t.shape[1] == head_dim // 2 and t.is_contiguous(), f"{name}: must be [positions, {head_dim // 2}]")
+        if not (t.dim() == 2 and t.shape[1] == head_dim // 2 and t.is_contiguous()):
+            raise KernelError(f"{name}: must be [positions, {head_dim // 2}]")
     _check_pages(k_pages, v_pages, page_table, n_kv, head_dim, torch.bfloat16)
     for name, t, n in (("seq_slot", seq_slot, n_seqs), ("cu_rows", cu_rows, n_seqs + 1),
                        ("tile_cu", tile_cu, n_seqs + 1), ("seq_start", seq_start, n_seqs)):
         _gpu(t, name, torch.int32)
-        _require(t.numel() >= n, f"{name}: needs {n} entries")
-    _require(n_heads <= 65535, "attn_causal: too many heads")
+        if not (t.numel() >= n):
+            raise KernelError(f"{name}: needs {n} entries")
+    if not (n_heads <= 65535):
+        raise KernelError("attn_causal: too many heads")
     _check(_fn("attn_mfma", "dryft_attn_causal_projected_bf16")(
         _ptr(qkv), qkv.stride(0), _ptr(q_weight), w_f32, int(q_weight is not None), float(eps), _ptr(cos), _ptr(sin),
         _ptr(k_pages), _ptr(v_pages), _ptr(page_table), page_table.shape[1], _ptr(seq_slot), _ptr(cu_rows), _ptr(tile_cu),
@@ -333,16 +374,21 @@ def attn_split_bf16(q, k_pages, v_pages, page_table, seq_slot, cu_rows, kv_len, 
                     n_splits: int, out, n_heads: int, n_kv: int, head_dim: int, scale: float, window: int) -> None:
     _gpu(q, "q", torch.bfloat16)
     _gpu(out, "out", torch.bfloat16)
-    _require(q.is_contiguous() and out.is_contiguous() and out.numel() == q.numel(), "attn_split: q and out contiguous")
+    if not (q.is_contiguous() and out.is_contiguous() and out.numel() == q.numel()):
+        raise KernelError("attn_split: q and out contiguous")
     _check_pages(k_pages, v_pages, page_table, n_kv, head_dim, torch.bfloat16)
     for name, t, n in (("seq_slot", seq_slot, n_seqs), ("cu_rows", cu_rows, n_seqs + 1), ("kv_len", kv_len, n_seqs)):
         _gpu(t, name, torch.int32)
-        _require(t.numel() >= n, f"{name}: needs {n} entries")
+        if not (t.numel() >= n):
+            raise KernelError(f"{name}: needs {n} entries")
     _gpu(part_o, "part_o", torch.float32)
     _gpu(part_ml, "part_ml", torch.float32)
-    _require(part_o.numel() >= n_seqs * n_heads * n_splits * head_dim and part_ml.numel() >= n_seqs * n_heads * n_splits * 2,
-             "attn_split: partial buffers too small")
-    _require(n_splits <= 65535 and n_kv * ((n_heads // n_kv + 15) // 16) <= 65535, "attn_split: grid too large")
+    if not (
+            part_o.numel() >= n_seqs * n_heads * n_splits * head_dim and part_ml.numel() >= n_seqs * n_heads * n_splits * 2
+    ):
+        raise KernelError("attn_split: partial buffers too small")
+    if not (n_splits <= 65535 and n_kv * ((n_heads // n_kv + 15) // 16) <= 65535):
+        raise KernelError("attn_split: grid too large")
     _check(_fn("attn_mfma", "dryft_attn_split_bf16")(
         _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(page_table), page_table.shape[1], _ptr(seq_slot), _ptr(cu_rows),
         _ptr(kv_len), n_seqs, _ptr(part_o), _ptr(part_ml), n_splits, _ptr(out), n_heads, n_kv, head_dim, float(scale),
@@ -360,31 +406,40 @@ def attn_decode_fused_bf16(qkv, q_weight, k_weight, eps: float, cos, sin, rot: i
     _gpu(qkv, "qkv", torch.bfloat16)
     _gpu(out, "out", torch.bfloat16)
     need_cols = (n_heads + 2 * n_kv) * head_dim
-    _require(qkv.dim() == 2 and qkv.stride(1) == 1 and qkv.shape[1] >= need_cols and qkv.shape[0] >= n_seqs,
-             f"attn_decode_fused: qkv must be [rows >= {n_seqs}, >= {need_cols}]")
-    _require(out.is_contiguous() and out.numel() >= n_seqs * n_heads * head_dim, "attn_decode_fused: out too small")
-    _require(n_heads // n_kv <= 16, "attn_decode_fused: at most 16 query heads per kv head")
+    if not (qkv.dim() == 2 and qkv.stride(1) == 1 and qkv.shape[1] >= need_cols and qkv.shape[0] >= n_seqs):
+        raise KernelError(f"attn_decode_fused: qkv must be [rows >= {n_seqs}, >= {need_cols}]")
+    if not (out.is_contiguous() and out.numel() >= n_seqs * n_heads * head_dim):
+        raise KernelError("attn_decode_fused: out too small")
+    if not (n_heads // n_kv <= 16):
+        raise KernelError("attn_decode_fused: at most 16 query heads per kv head")
     _check_pages(k_pages, v_pages, page_table, n_kv, head_dim, torch.bfloat16)
     has_norm = q_weight is not None
     w_f32 = 0
     if has_norm:
         for name, w in (("q_weight", q_weight), ("k_weight", k_weight)):
             _gpu(w, name)
-            _require(w.shape == (head_dim,) and w.is_contiguous(), f"{name}: must be [{head_dim}]")
-        _require(q_weight.dtype == k_weight.dtype, "q_weight and k_weight must share a dtype")
+            if not (w.shape == (head_dim,) and w.is_contiguous()):
+                raise KernelError(f"{name}: must be [{head_dim}]")
+        if not (q_weight.dtype == k_weight.dtype):
+            raise KernelError("q_weight and k_weight must share a dtype")
         w_f32 = _float_flag(q_weight, "q_weight")
     if rot:
-        _require(rot % 2 == 0 and rot <= head_dim, f"rotary width {rot} must be even and at most {head_dim}")
+        if not (rot % 2 == 0 and rot <= head_dim):
+            raise KernelError(f"rotary width {rot} must be even and at most {head_dim}")
         for name, t in (("cos", cos), ("sin", sin)):
             _gpu(t, name, torch.bfloat16)
-            _require(t.dim() == 2 and t.shape[1] == rot // 2 and t.is_contiguous(), f"{name}: must be [positions, {rot // 2}]")
+            if not (t.dim() == 2 and t.shape[1] == rot // 2 and t.is_contiguous()):
+                raise KernelError(f"{name}: must be [positions, {rot // 2}]")
     for name, t, n in (("seq_slot", seq_slot, n_seqs), ("cu_rows", cu_rows, n_seqs + 1), ("kv_len", kv_len, n_seqs)):
         _gpu(t, name, torch.int32)
-        _require(t.numel() >= n, f"{name}: needs {n} entries")
+        if not (t.numel() >= n):
+            raise KernelError(f"{name}: needs {n} entries")
     _gpu(part_o, "part_o", torch.float32)
     _gpu(part_ml, "part_ml", torch.float32)
-    _require(part_o.numel() >= n_seqs * n_heads * n_splits * head_dim and part_ml.numel() >= n_seqs * n_heads * n_splits * 2,
-             "attn_decode_fused: partial buffers too small")
+    if not (
+            part_o.numel() >= n_seqs * n_heads * n_splits * head_dim and part_ml.numel() >= n_seqs * n_heads * n_splits * 2
+    ):
+        raise KernelError("attn_decode_fused: partial buffers too small")
     _check(_fn("attn_mfma", "dryft_attn_decode_fused_bf16")(
         _ptr(qkv), qkv.stride(0), _ptr(q_weight), _ptr(k_weight), w_f32, int(has_norm), float(eps), _ptr(cos), _ptr(sin),
         int(rot), int(write_kv), _ptr(k_pages), _ptr(v_pages), _ptr(page_table), page_table.shape[1], _ptr(seq_slot),
@@ -400,11 +455,12 @@ def gemm_tiled(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Ten
     is_f32 = _float_flag(x, "x")
     m, k = x.shape
     n = w.shape[0]
-    _require(w.shape == (n, k) and w.is_contiguous() and x.stride(1) == 1, "gemm_tiled: x [M,K] row-major, w [N,K] contiguous")
+    if not (w.shape == (n, k) and w.is_contiguous() and x.stride(1) == 1):
+        raise KernelError("gemm_tiled: x [M,K] row-major, w [N,K] contiguous")
     _gpu(out, "out")
     out_f32 = 1 if out.dtype == torch.float32 else 0
-    _require(out.shape == (m, n) and out.is_contiguous() and (out.dtype == x.dtype or out_f32),
-             f"gemm_tiled: out must be [{m},{n}] in the input dtype or float32")
+    if not (out.shape == (m, n) and out.is_contiguous() and (out.dtype == x.dtype or out_f32)):
+        raise KernelError(f"gemm_tiled: out must be [{m},{n}] in the input dtype or float32")
     for m0 in range(0, m, 65535 * 64):                      # the row tiles ride on grid.y
         m1 = min(m, m0 + 65535 * 64)
         _check(_fn("gemm", "dryft_gemm_tiled")(_ptr(x[m0:m1]), x.stride(0), _ptr(w), _ptr(out[m0:m1]), m1 - m0, n, k,
@@ -423,20 +479,24 @@ def gemm_stream_bf16(x, w, out, partials=None, group_blocks: int = 2, splits: in
     _gpu(w, "w", torch.bfloat16)
     m, k = x.shape
     n = w.shape[0]
-    _require(w.shape == (n, k) and w.is_contiguous() and x.stride(1) == 1, "gemm_stream: x [M,K] row-major, w [N,K] contiguous")
-    _require(m <= 16 and k % 8 == 0 and x.stride(0) % 8 == 0, f"gemm_stream: needs M <= 16 and K % 8 == 0, got M={m} K={k}")
-    _require(x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0, "gemm_stream: operands must be 16-byte aligned")
-    _require(group_blocks in (1, 2) and depth in (1, 2) and 1 <= splits <= 64,
-             "gemm_stream: group_blocks and depth in 1, 2 and splits in 1..64")
+    if not (w.shape == (n, k) and w.is_contiguous() and x.stride(1) == 1):
+        raise KernelError("gemm_stream: x [M,K] row-major, w [N,K] contiguous")
+    if not (m <= 16 and k % 8 == 0 and x.stride(0) % 8 == 0):
+        raise KernelError(f"gemm_stream: needs M <= 16 and K % 8 == 0, got M={m} K={k}")
+    if not (x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0):
+        raise KernelError("gemm_stream: operands must be 16-byte aligned")
+    if not (group_blocks in (1, 2) and depth in (1, 2) and 1 <= splits <= 64):
+        raise KernelError("gemm_stream: group_blocks and depth in 1, 2 and splits in 1..64")
     out_f32 = 0
     if splits > 1:
         _gpu(partials, "partials", torch.float32)
-        _require(partials.numel() >= splits * m * n and partials.is_contiguous(), "gemm_stream: partials too small")
+        if not (partials.numel() >= splits * m * n and partials.is_contiguous()):
+            raise KernelError("gemm_stream: partials too small")
     else:
         _gpu(out, "out")
         out_f32 = 1 if out.dtype == torch.float32 else 0
-        _require(out.shape == (m, n) and out.is_contiguous() and out.dtype in (torch.float32, torch.bfloat16),
-                 f"gemm_stream: out must be contiguous [{m},{n}]")
+        if not (out.shape == (m, n) and out.is_contiguous() and out.dtype in (torch.float32, torch.bfloat16)):
+            raise KernelError(f"gemm_stream: out must be contiguous [{m},{n}]")
     _check(_fn("gemm", "dryft_gemm_stream_bf16")(_ptr(x), x.stride(0), _ptr(w), _ptr(out), _ptr(partials), m, n, k,
                                                  int(group_blocks), int(depth), int(splits), out_f32, _stream()), "gemm_stream_bf16")
 
@@ -448,12 +508,16 @@ def gemm_stream_swiglu_bf16(x, w_gate_up, out, group_blocks: int = 2, depth: int
     _gpu(out, "out", torch.bfloat16)
     m, k = x.shape
     two_n = w_gate_up.shape[0]
-    _require(two_n % 2 == 0 and w_gate_up.shape == (two_n, k) and w_gate_up.is_contiguous() and x.stride(1) == 1,
-             "gemm_stream_swiglu: x [M,K] row-major, w [2N,K] contiguous")
-    _require(m <= 16 and k % 8 == 0 and x.stride(0) % 8 == 0, f"gemm_stream_swiglu: needs M <= 16 and K % 8 == 0, got M={m} K={k}")
-    _require(x.data_ptr() % 16 == 0 and w_gate_up.data_ptr() % 16 == 0, "gemm_stream_swiglu: operands must be 16-byte aligned")
-    _require(out.shape == (m, two_n // 2) and out.is_contiguous(), f"gemm_stream_swiglu: out must be [{m},{two_n // 2}]")
-    _require(group_blocks in (1, 2) and depth in (1, 2), "gemm_stream_swiglu: group_blocks and depth in 1, 2")
+    if not (two_n % 2 == 0 and w_gate_up.shape == (two_n, k) and w_gate_up.is_contiguous() and x.stride(1) == 1):
+        raise KernelError("gemm_stream_swiglu: x [M,K] row-major, w [2N,K] contiguous")
+    if not (m <= 16 and k % 8 == 0 and x.stride(0) % 8 == 0):
+        raise KernelError(f"gemm_stream_swiglu: needs M <= 16 and K % 8 == 0, got M={m} K={k}")
+    if not (x.data_ptr() % 16 == 0 and w_gate_up.data_ptr() % 16 == 0):
+        raise KernelError("gemm_stream_swiglu: operands must be 16-byte aligned")
+    if not (out.shape == (m, two_n // 2) and out.is_contiguous()):
+        raise KernelError(f"gemm_stream_swiglu: out must be [{m},{two_n // 2}]")
+    if not (group_blocks in (1, 2) and depth in (1, 2)):
+        raise KernelError("gemm_stream_swiglu: group_blocks and depth in 1, 2")
     _check(_fn("gemm", "dryft_gemm_stream_swiglu_bf16")(_ptr(x), x.stride(0), _ptr(w_gate_up), _ptr(out), m, two_n // 2, k,
                                                         int(group_blocks), int(depth), _stream()), "gemm_stream_swiglu_bf16")
     return out
@@ -470,20 +534,24 @@ def gemm_wide_bf16(x, w, out, partials=None, group_blocks: int = 2, splits: int 
     _gpu(w, "w", torch.bfloat16)
     m, k = x.shape
     n = w.shape[0]
-    _require(w.shape == (n, k) and w.is_contiguous() and x.stride(1) == 1, "gemm_wide: x [M,K] row-major, w [N,K] contiguous")
-    _require(m <= 64 and k % 8 == 0 and x.stride(0) % 8 == 0, f"gemm_wide: needs M <= 64 and K % 8 == 0, got M={m} K={k}")
-    _require(x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0, "gemm_wide: operands must be 16-byte aligned")
-    _require(group_blocks in (1, 2) and depth in (1, 2, 3) and 1 <= splits <= 64,
-             "gemm_wide: group_blocks in 1, 2, depth in 1..3 and splits in 1..64")
+    if not (w.shape == (n, k) and w.is_contiguous() and x.stride(1) == 1):
+        raise KernelError("gemm_wide: x [M,K] row-major, w [N,K] contiguous")
+    if not (m <= 64 and k % 8 == 0 and x.stride(0) % 8 == 0):
+        raise KernelError(f"gemm_wide: needs M <= 64 and K % 8 == 0, got M={m} K={k}")
+    if not (x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0):
+        raise KernelError("gemm_wide: operands must be 16-byte aligned")
+    if not (group_blocks in (1, 2) and depth in (1, 2, 3) and 1 <= splits <= 64):
+        raise KernelError("gemm_wide: group_blocks in 1, 2, depth in 1..3 and splits in 1..64")
     out_f32 = 0
     if splits > 1:
         _gpu(partials, "partials", torch.float32)
-        _require(partials.numel() >= splits * m * n and partials.is_contiguous(), "gemm_wide: partials too small")
+        if not (partials.numel() >= splits * m * n and partials.is_contiguous()):
+            raise KernelError("gemm_wide: partials too small")
     else:
         _gpu(out, "out")
         out_f32 = 1 if out.dtype == torch.float32 else 0
-        _require(out.shape == (m, n) and out.is_contiguous() and out.dtype in (torch.float32, torch.bfloat16),
-                 f"gemm_wide: out must be contiguous [{m},{n}]")
+        if not (out.shape == (m, n) and out.is_contiguous() and out.dtype in (torch.float32, torch.bfloat16)):
+            raise KernelError(f"gemm_wide: out must be contiguous [{m},{n}]")
     _check(_fn("gemm", "dryft_gemm_wide_bf16")(_ptr(x), x.stride(0), _ptr(w), _ptr(out), _ptr(partials), m, n, k,
                                                int(group_blocks), int(depth), int(splits), out_f32, _stream()), "gemm_wide_bf16")
 
@@ -505,13 +573,16 @@ def gemm_panel_swiglu_bf16(x, w_gate_up, out, waves: int = 0) -> torch.Tensor:
     _gpu(out, "out", torch.bfloat16)
     m, k = x.shape
     two_n = w_gate_up.shape[0]
-    _require(two_n % 2 == 0 and w_gate_up.shape == (two_n, k) and w_gate_up.is_contiguous() and x.stride(1) == 1,
-             "gemm_panel_swiglu: x [M,K] row-major, w [2N,K] contiguous")
-    _require(m <= 64 and k % PANEL_GROUP == 0 and x.stride(0) % 8 == 0,
-             f"gemm_panel_swiglu: needs M <= 64 and K % {PANEL_GROUP} == 0, got M={m} K={k}")
-    _require(x.data_ptr() % 16 == 0 and w_gate_up.data_ptr() % 16 == 0, "gemm_panel_swiglu: operands must be 16-byte aligned")
-    _require(out.shape == (m, two_n // 2) and out.is_contiguous(), f"gemm_panel_swiglu: out must be [{m},{two_n // 2}]")
-    _require(waves == 0 or 4 <= waves <= 8, "gemm_panel_swiglu: waves 4 to 8, or 0")
+    if not (two_n % 2 == 0 and w_gate_up.shape == (two_n, k) and w_gate_up.is_contiguous() and x.stride(1) == 1):
+        raise KernelError("gemm_panel_swiglu: x [M,K] row-major, w [2N,K] contiguous")
+    if not (m <= 64 and k % PANEL_GROUP == 0 and x.stride(0) % 8 == 0):
+        raise KernelError(f"gemm_panel_swiglu: needs M <= 64 and K % {PANEL_GROUP} == 0, got M={m} K={k}")
+    if not (x.data_ptr() % 16 == 0 and w_gate_up.data_ptr() % 16 == 0):
+        raise KernelError("gemm_panel_swiglu: operands must be 16-byte aligned")
+    if not (out.shape == (m, two_n // 2) and out.is_contiguous()):
+        raise KernelError(f"gemm_panel_swiglu: out must be [{m},{two_n // 2}]")
+    if not (waves == 0 or 4 <= waves <= 8):
+        raise KernelError("gemm_panel_swiglu: waves 4 to 8, or 0")
     _check(_fn("gemm", "dryft_gemm_panel_swiglu_bf16")(_ptr(x), x.stride(0), _ptr(w_gate_up), _ptr(out), m, two_n // 2, k,
                                                        int(waves), _stream()), "gemm_panel_swiglu_bf16")
     return out
@@ -524,12 +595,16 @@ def gemm_wide_swiglu_bf16(x, w_gate_up, out, group_blocks: int = 2, depth: int =
     _gpu(out, "out", torch.bfloat16)
     m, k = x.shape
     two_n = w_gate_up.shape[0]
-    _require(two_n % 2 == 0 and w_gate_up.shape == (two_n, k) and w_gate_up.is_contiguous() and x.stride(1) == 1,
-             "gemm_wide_swiglu: x [M,K] row-major, w [2N,K] contiguous")
-    _require(m <= 64 and k % 8 == 0 and x.stride(0) % 8 == 0, f"gemm_wide_swiglu: needs M <= 64 and K % 8 == 0, got M={m} K={k}")
-    _require(x.data_ptr() % 16 == 0 and w_gate_up.data_ptr() % 16 == 0, "gemm_wide_swiglu: operands must be 16-byte aligned")
-    _require(out.shape == (m, two_n // 2) and out.is_contiguous(), f"gemm_wide_swiglu: out must be [{m},{two_n // 2}]")
-    _require(group_blocks in (1, 2) and depth in (1, 2, 3), "gemm_wide_swiglu: group_blocks in 1, 2 and depth in 1..3")
+    if not (two_n % 2 == 0 and w_gate_up.shape == (two_n, k) and w_gate_up.is_contiguous() and x.stride(1) == 1):
+        raise KernelError("gemm_wide_swiglu: x [M,K] row-major, w [2N,K] contiguous")
+    if not (m <= 64 and k % 8 == 0 and x.stride(0) % 8 == 0):
+        raise KernelError(f"gemm_wide_swiglu: needs M <= 64 and K % 8 == 0, got M={m} K={k}")
+    if not (x.data_ptr() % 16 == 0 and w_gate_up.data_ptr() % 16 == 0):
+        raise KernelError("gemm_wide_swiglu: operands must be 16-byte aligned")
+    if not (out.shape == (m, two_n // 2) and out.is_contiguous()):
+        raise KernelError(f"gemm_wide_swiglu: out must be [{m},{two_n // 2}]")
+    if not (group_blocks in (1, 2) and depth in (1, 2, 3)):
+        raise KernelError("gemm_wide_swiglu: group_blocks in 1, 2 and depth in 1..3")
     _check(_fn("gemm", "dryft_gemm_wide_swiglu_bf16")(_ptr(x), x.stride(0), _ptr(w_gate_up), _ptr(out), m, two_n // 2, k,
                                                       int(group_blocks), int(depth), _stream()), "gemm_wide_swiglu_bf16")
     return out
@@ -545,15 +620,23 @@ def gemm_block_bf16(x, w, out, swiglu: bool = False, shape: int | None = None) -
     _gpu(out, "out")
     m, k = x.shape
     n = w.shape[0] // 2 if swiglu else w.shape[0]
-    _require(w.dim() == 2 and w.shape[1] == k and w.is_contiguous() and x.stride(1) == 1 and (not swiglu or w.shape[0] % 2 == 0),
-             "gemm_block: x [M,K] row-major, w [N,K] (or [2N,K]) contiguous")
-    _require(k % 8 == 0 and x.stride(0) % 8 == 0, f"gemm_block: needs K % 8 == 0, got K={k}")
-    _require(x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0, "gemm_block: operands must be 16-byte aligned")
-    _require(out.shape == (m, n) and out.is_contiguous() and out.dtype in (torch.float32, torch.bfloat16) and
-             not (swiglu and out.dtype != torch.bfloat16), f"gemm_block: out must be contiguous [{m},{n}]")
+    if not (
+            w.dim() == 2 and w.shape[1] == k and w.is_contiguous() and x.stride(1) == 1 and (not swiglu or w.shape[0] % 2 == 0)
+    ):
+        raise KernelError("gemm_block: x [M,K] row-major, w [N,K] (or [2N,K]) contiguous")
+    if not (k % 8 == 0 and x.stride(0) % 8 == 0):
+        raise KernelError(f"gemm_block: needs K % 8 == 0, got K={k}")
+    if not (x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0):
+        raise KernelError("gemm_block: operands must be 16-byte aligned")
+    if not (
+            out.shape == (m, n) and out.is_contiguous() and out.dtype in (torch.float32, torch.bfloat16) and
+            not (swiglu and out.dtype != torch.bfloat16)
+    ):
+        raise KernelError(f"gemm_block: out must be contiguous [{m},{n}]")
     if shape is None:
         shape = 1 if -(-m // 256) * -(-(2 * n if swiglu else n) // 256) >= 256 else 0
-    _require(shape in (0, 1), "gemm_block: shape 0 or 1")
+    if not (shape in (0, 1)):
+        raise KernelError("gemm_block: shape 0 or 1")
     _check(_fn("gemm", "dryft_gemm_block_bf16")(_ptr(x), x.stride(0), _ptr(w), _ptr(out), m, n, k, 1 if swiglu else 0,
                                                 1 if out.dtype == torch.float32 else 0, int(shape), _stream()), "gemm_block_bf16")
     return out
@@ -567,13 +650,18 @@ def gemm_block_f32(x, w, out, shape: int | None = None) -> torch.Tensor:
     _gpu(out, "out", torch.float32)
     m, k = x.shape
     n = w.shape[0]
-    _require(w.shape == (n, k) and w.is_contiguous() and x.stride(1) == 1, "gemm_block_f32: x [M,K] row-major, w [N,K] contiguous")
-    _require(k % 4 == 0 and x.stride(0) % 4 == 0, f"gemm_block_f32: needs K % 4 == 0, got K={k}")
-    _require(x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0, "gemm_block_f32: operands must be 16-byte aligned")
-    _require(out.shape == (m, n) and out.is_contiguous(), f"gemm_block_f32: out must be contiguous [{m},{n}]")
+    if not (w.shape == (n, k) and w.is_contiguous() and x.stride(1) == 1):
+        raise KernelError("gemm_block_f32: x [M,K] row-major, w [N,K] contiguous")
+    if not (k % 4 == 0 and x.stride(0) % 4 == 0):
+        raise KernelError(f"gemm_block_f32: needs K % 4 == 0, got K={k}")
+    if not (x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0):
+        raise KernelError("gemm_block_f32: operands must be 16-byte aligned")
+    if not (out.shape == (m, n) and out.is_contiguous()):
+        raise KernelError(f"gemm_block_f32: out must be contiguous [{m},{n}]")
     if shape is None:
         shape = 1 if -(-m // 256) * -(-n // 256) >= 256 else 0
-    _require(shape in (0, 1), "gemm_block_f32: shape 0 or 1")
+    if not (shape in (0, 1)):
+        raise KernelError("gemm_block_f32: shape 0 or 1")
     _check(_fn("gemm", "dryft_gemm_block_f32")(_ptr(x), x.stride(0), _ptr(w), _ptr(out), m, n, k, int(shape), _stream()),
            "gemm_block_f32")
     return out
@@ -587,9 +675,12 @@ def gemm_rows_f32(x, w, out) -> torch.Tensor:
     _gpu(out, "out", torch.float32)
     m, k = x.shape
     n = w.shape[0]
-    _require(w.shape == (n, k) and w.is_contiguous() and x.stride(1) == 1, "gemm_rows_f32: x [M,K] row-major, w [N,K] contiguous")
-    _require(m <= 16 and k % 4 == 0 and w.data_ptr() % 16 == 0, f"gemm_rows_f32: needs M <= 16, K % 4 == 0, aligned w; got M={m} K={k}")
-    _require(out.shape == (m, n) and out.is_contiguous(), f"gemm_rows_f32: out must be contiguous [{m},{n}]")
+    if not (w.shape == (n, k) and w.is_contiguous() and x.stride(1) == 1):
+        raise KernelError("gemm_rows_f32: x [M,K] row-major, w [N,K] contiguous")
+    if not (m <= 16 and k % 4 == 0 and w.data_ptr() % 16 == 0):
+        raise KernelError(f"gemm_rows_f32: needs M <= 16, K % 4 == 0, aligned w; got M={m} K={k}")
+    if not (out.shape == (m, n) and out.is_contiguous()):
+        raise KernelError(f"gemm_rows_f32: out must be contiguous [{m},{n}]")
     _check(_fn("gemm", "dryft_gemm_rows_f32")(_ptr(x), x.stride(0), _ptr(w), _ptr(out), m, n, k, _stream()), "gemm_rows_f32")
     return out
 
@@ -597,9 +688,10 @@ def gemm_rows_f32(x, w, out) -> torch.Tensor:
 def sum_partials(partials: torch.Tensor, out: torch.Tensor, splits: int) -> torch.Tensor:
     _gpu(partials, "partials", torch.float32)
     _gpu(out, "out")
-    _require(out.is_contiguous() and partials.is_contiguous() and partials.numel() >= splits * out.numel(),
-             "sum_partials: partials must hold splits * out.numel() values")
-    _require(out.dtype in (torch.float32, torch.bfloat16), "sum_partials: out must be float32 or bfloat16")
+    if not (out.is_contiguous() and partials.is_contiguous() and partials.numel() >= splits * out.numel()):
+        raise KernelError("sum_partials: partials must hold splits * out.numel() values")
+    if not (out.dtype in (torch.float32, torch.bfloat16)):
+        raise KernelError("sum_partials: out must be float32 or bfloat16")
     _check(_fn("gemm", "dryft_sum_partials")(_ptr(partials), _ptr(out), out.numel(), splits,
                                              1 if out.dtype == torch.float32 else 0, _stream()), "sum_partials")
     return out
@@ -610,7 +702,8 @@ def argmax_rows(logits: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     _gpu(logits, "logits", torch.float32)
     _gpu(out, "out", torch.int32)
     rows, vocab = logits.shape
-    _require(logits.stride(1) == 1 and out.numel() >= rows and out.is_contiguous(), "argmax_rows: bad operands")
+    if not (logits.stride(1) == 1 and out.numel() >= rows and out.is_contiguous()):
+        raise KernelError("argmax_rows: bad operands")
     chunks = 1 if vocab < 8192 else min(64, vocab // 2048)
     scratch_v = scratch_i = None
     if chunks > 1:
@@ -626,8 +719,10 @@ def sample_rows(logits: torch.Tensor, temperature: float, uniforms: torch.Tensor
     _gpu(uniforms, "uniforms", torch.float32)
     _gpu(out, "out", torch.int32)
     rows, vocab = logits.shape
-    _require(temperature > 0, "sample_rows: temperature must be positive (use argmax_rows for greedy)")
-    _require(logits.stride(1) == 1 and out.numel() >= rows and uniforms.numel() >= rows, "sample_rows: bad operands")
+    if not (temperature > 0):
+        raise KernelError("sample_rows: temperature must be positive (use argmax_rows for greedy)")
+    if not (logits.stride(1) == 1 and out.numel() >= rows and uniforms.numel() >= rows):
+        raise KernelError("sample_rows: bad operands")
     chunks = 1 if vocab < 8192 else min(64, vocab // 2048)
     chunk_max = chunk_sum = None
     if chunks > 1:
