@@ -6,7 +6,8 @@
 //    sizes the matrix-core kernel refuses.
 //  * gemm_stream (M <= 16) and gemm_wide (M <= 64): bfloat16, few rows (decoding, output head): every
 //    weight is read once and multiplied on the matrix cores; K may be split across workgroups into
-//    float partial sums that the consumer adds in a fixed order.
+//    float partial sums that the consumer adds in a fixed order. gemm_panel (M <= 64) is the fused gate/up
+//    product, gemm_mid (M <= 256) the projections back to the hidden width for short prompts.
 #include "common.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
@@ -740,6 +741,152 @@ DRYFT_API int dryft_gemm_panel_swiglu_bf16(const void* x, int64_t x_stride, cons
     case 3: return panel_waves<3>(x, x_stride, w, y, M, N, K, waves, stream);
     default: return panel_waves<4>(x, x_stride, w, y, M, N, K, waves, stream);
   }
+}
+
+// --------------------------------------------------------------------------------------------- mid
+// The projections back to the hidden width (few outputs, a long K) for short prompts, 65 to 256 rows: there the
+// vendor library takes 20 to 50 us for matrices that stream in 4 to 10 (Qwen3-4B: o 20 to 25 us, down 27 to 53),
+// because its tiles are too few for the chip. Here a workgroup of four waves owns 64 outputs (16 rows of W a wave)
+// and all rows of x, K is split over workgroups into float partial sums that the consumer adds in a fixed order,
+// and the operands go from memory straight into LDS as in the panel product (groups of 64 values of K: rows of
+// 128 bytes, piece p of row r at place p ^ ((r / 2) % 8); three groups in LDS; a wave fetches its own 16 rows of W
+// and its share of the rows of x; every workgroup walks its part of K from a starting group of its own). Every
+// workgroup reads all of x (from L2), which is why this form stops paying at about 250 rows and never pays for the
+// products with many outputs (q/k/v, gate/up). Measured, weights from memory, us at 80 / 128 / 192 rows against the
+// vendor library: Qwen3-4B's o 10.9 / 12.8 / 17.3 (21 / 25 / 19), down 19.1 / 21.0 / 28.5 (27 / 53 / 34); Qwen3-8B's o
+// 13.5 / 15.4 / 20.6 (21 / 25 / 34), down 29 / 38 / 53 (38 / 67 / 90); Qwen3-32B's o 26 / 29 / 39 (30 / 45 / 61), down
+// 72 / 88 / 111 (173 / 181 / 209).
+#define MID_GROUP 64
+#define MID_STAGES 3
+#define MID_WAVES 4
+
+template <int MT>
+__global__ __launch_bounds__(64 * MID_WAVES) void gemm_mid_kernel(const bf16_t* __restrict__ x, int64_t x_stride,
+                                                                  const bf16_t* __restrict__ w,
+                                                                  float* __restrict__ partials, int M, int N, int K,
+                                                                  int groups_per_split) {
+  extern __shared__ __align__(16) unsigned char mid_lds[];
+  constexpr int STAGES = MID_STAGES, WAVES = MID_WAVES;
+  constexpr int RB = 2 * MID_GROUP;                        // bytes of a row in a group
+  constexpr int X_ALL = 2 * MT;                            // 1 KB pieces (8 rows) of x in a group
+  constexpr int X_LOADS = (X_ALL + WAVES - 1) / WAVES;     // every wave issues this many
+  constexpr int LOADS = 2 + X_LOADS;
+  constexpr int W_BYTES = 16 * WAVES * RB, X_BYTES = 16 * MT * RB, STAGE_BYTES = W_BYTES + X_BYTES;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
+  const int lane = threadIdx.x % WAVE, c = lane % 16, g = lane / 16;
+  const int n0 = (blockIdx.x * WAVES + wave) * 16;         // first output of this wave
+  const int group0 = blockIdx.y * groups_per_split;
+  const int groups = min(groups_per_split, K / MID_GROUP - group0);
+  uint32_t w_from[2], x_from[X_LOADS];
+  int x_piece[X_LOADS];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int r = 8 * i + lane / 8;                        // row within the wave's 16
+    w_from[i] = (uint32_t)min(n0 + r, N - 1) * (uint32_t)K * 2u + (((lane % 8) ^ ((r >> 1) & 7)) << 4);
+  }
+#pragma unroll
+  for (int i = 0; i < X_LOADS; ++i) {
+    x_piece[i] = min(wave + WAVES * i, X_ALL - 1);
+    const int r = 8 * x_piece[i] + lane / 8;               // row of x
+    x_from[i] = (uint32_t)min(r, M - 1) * (uint32_t)x_stride * 2u + (((lane % 8) ^ ((r >> 1) & 7)) << 4);
+  }
+  const uint32_t lds0 = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)mid_lds);
+  const int first_group = (int)((blockIdx.x * 5u) % (unsigned)groups);
+  auto fetch = [&](int group, int stage) {
+    int gk = min(group, groups - 1) + first_group;         // past the end: the last group again, into a free buffer
+    gk = (gk >= groups ? gk - groups : gk) + group0;
+    const unsigned char* wb = (const unsigned char*)w + (int64_t)gk * RB;
+    const unsigned char* xb = (const unsigned char*)x + (int64_t)gk * RB;
+    const uint32_t at = lds0 + stage * STAGE_BYTES;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) panel_load16(wb, w_from[i], at + (16 * wave + 8 * i) * RB);
+#pragma unroll
+    for (int i = 0; i < X_LOADS; ++i) panel_load16(xb, x_from[i], at + W_BYTES + x_piece[i] * 1024);
+  };
+  f32x4 acc[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int s = 0; s < STAGES - 1; ++s) fetch(s, s);
+  int stage = 0;
+  const int sw = (c >> 1) & 7;                             // row 16 t + c of any tile is swizzled like row c
+  for (int group = 0; group < groups; ++group) {
+    panel_wait<(STAGES - 2) * LOADS>();                    // this group has arrived; the later ones may be on their way
+    __syncthreads();                                       // everybody's part of it too; the group before is done with
+    fetch(group + STAGES - 1, stage == 0 ? STAGES - 1 : stage - 1);
+    const unsigned char* ws = mid_lds + stage * STAGE_BYTES + (16 * wave + c) * RB;
+    const unsigned char* xs = mid_lds + stage * STAGE_BYTES + W_BYTES + c * RB;
+    bf16x8 a[2], b[2][MT];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {                          // 32 values of K at a time
+      const int place = ((4 * u + g) ^ sw) << 4;
+      a[u] = *(const bf16x8*)(ws + place);
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) b[u][mt] = *(const bf16x8*)(xs + 16 * mt * RB + place);
+    }
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u], b[u][mt], acc[mt], 0, 0, 0);
+    // the order the scheduler is to keep: the first half's reads; its matrix instructions with one read of the
+    // second half after each; the second half's matrix instructions (0x100: LDS reads, 0x008: matrix instructions)
+    __builtin_amdgcn_sched_group_barrier(0x100, MT + 1, 0);
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    __builtin_amdgcn_sched_group_barrier(0x008, MT, 0);
+    stage = stage + 1 == STAGES ? 0 : stage + 1;
+  }
+  panel_wait<0>();                                         // the loads past the end have landed before the waves leave
+  // acc[mt][i] is output n0 + 4g + i of activation row 16 mt + c
+  float* out = partials + (int64_t)blockIdx.y * M * N;
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int m = 16 * mt + c, n = n0 + 4 * g;
+    if (m >= M) continue;
+    if (n + 3 < N && (N & 3) == 0) {
+      *(f32x4*)(out + (int64_t)m * N + n) = acc[mt];
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (n + i < N) out[(int64_t)m * N + n + i] = acc[mt][i];
+    }
+  }
+}
+
+template <int MT>
+static int launch_mid(const void* x, int64_t x_stride, const void* w, float* partials, int M, int N, int K, int splits,
+                      int groups_per_split, hipStream_t stream) {
+  constexpr int lds = MID_STAGES * (16 * MID_WAVES + 16 * MT) * 2 * MID_GROUP;
+  static_assert(lds <= 160 * 1024, "the stages must fit a compute unit's LDS");
+  static bool raised = false;                              // more dynamic LDS than the default limit allows
+  auto kernel = gemm_mid_kernel<MT>;
+  if (lds > 64 * 1024 && !raised) {
+    if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess) return -2;
+    raised = true;
+  }
+  dim3 grid((N + 16 * MID_WAVES - 1) / (16 * MID_WAVES), splits), block(64 * MID_WAVES);
+  hipLaunchKernelGGL(kernel, grid, block, lds, stream, (const bf16_t*)x, x_stride, (const bf16_t*)w, partials, M, N, K,
+                     groups_per_split);
+  return DRYFT_LAUNCH_CHECK();
+}
+
+// M <= 256. partials[splits, M, N] = float partial sums of x . W^T over `splits` equal runs of groups of 64 values of K
+// (the last run may be shorter, none may be empty); K a multiple of 64; x and W within reach of 32-bit byte offsets.
+DRYFT_API int dryft_gemm_mid_bf16(const void* x, int64_t x_stride, const void* w, float* partials, int M, int N, int K,
+                                  int splits, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (M > 256 || K <= 0 || K % MID_GROUP || splits < 1 || x_stride % 8 || (((uintptr_t)x | (uintptr_t)w) & 15) ||
+      ((uintptr_t)partials & 15) || (int64_t)N * K * 2 >= (int64_t)4 << 30 || (int64_t)M * x_stride * 2 >= (int64_t)4 << 30)
+    return -1;
+  const int groups = K / MID_GROUP, per = (groups + splits - 1) / splits;
+  if ((groups + per - 1) / per != splits) return -1;       // a run would be empty
+  if (M <= 128) return launch_mid<8>(x, x_stride, w, partials, M, N, K, splits, per, stream);
+  if (M <= 192) return launch_mid<12>(x, x_stride, w, partials, M, N, K, splits, per, stream);
+  return launch_mid<16>(x, x_stride, w, partials, M, N, K, splits, per, stream);
 }
 
 // ------------------------------------------------------------------------------------------- block

@@ -40,6 +40,7 @@ _SIGNATURES = {
              "dryft_gemm_wide_bf16": [_P, _L, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
              "dryft_gemm_panel_swiglu_bf16": [_P, _L, _P, _P, _I, _I, _I, _I, _P],
              "dryft_gemm_panel_waves": [_I],
+             "dryft_gemm_mid_bf16": [_P, _L, _P, _P, _I, _I, _I, _I, _P],
              "dryft_gemm_block_bf16": [_P, _L, _P, _P, _I, _I, _I, _I, _I, _I, _P],
              "dryft_gemm_block_f32": [_P, _L, _P, _P, _I, _I, _I, _I, _P],
              "dryft_gemm_rows_f32": [_P, _L, _P, _P, _I, _I, _I, _P],
@@ -586,6 +587,43 @@ def gemm_panel_swiglu_bf16(x, w_gate_up, out, waves: int = 0) -> torch.Tensor:
     _check(_fn("gemm", "dryft_gemm_panel_swiglu_bf16")(_ptr(x), x.stride(0), _ptr(w_gate_up), _ptr(out), m, two_n // 2, k,
                                                        int(waves), _stream()), "gemm_panel_swiglu_bf16")
     return out
+
+
+MID_ROWS = 256      # the most rows gemm_mid takes
+MID_GROUP = 64      # values of K it walks at a time; K must be a multiple, and the splits are runs of such groups
+
+
+def gemm_mid_splits(k: int, splits: int) -> int:
+    """The number of splits closest below ``splits`` that cuts ``k`` into runs of groups none of which is empty."""
+    groups = k // MID_GROUP
+    splits = max(1, min(splits, groups))
+    while splits > 1 and -(-groups // -(-groups // splits)) != splits:
+        splits -= 1
+    return splits
+
+
+def gemm_mid_bf16(x, w, partials, splits: int) -> torch.Tensor:
+    """Float partial sums ``partials[splits, M, N]`` of ``x @ w.T`` over ``splits`` runs of K, for 1 to 256 rows, by the
+    kernel whose operands go from memory straight into LDS. K must be a multiple of 64 and ``splits`` one that
+    ``gemm_mid_splits`` returns."""
+    _gpu(x, "x", torch.bfloat16)
+    _gpu(w, "w", torch.bfloat16)
+    _gpu(partials, "partials", torch.float32)
+    m, k = x.shape
+    n = w.shape[0]
+    if not (w.shape == (n, k) and w.is_contiguous() and x.stride(1) == 1):
+        raise KernelError("gemm_mid: x [M,K] row-major, w [N,K] contiguous")
+    if not (m <= MID_ROWS and k % MID_GROUP == 0 and x.stride(0) % 8 == 0):
+        raise KernelError(f"gemm_mid: needs M <= {MID_ROWS} and K % {MID_GROUP} == 0, got M={m} K={k}")
+    if not (x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0 and partials.data_ptr() % 16 == 0):
+        raise KernelError("gemm_mid: operands must be 16-byte aligned")
+    if not (splits >= 1 and gemm_mid_splits(k, splits) == splits):
+        raise KernelError(f"gemm_mid: {splits} splits would leave a run of K = {k} empty")
+    if not (partials.shape == (splits, m, n) and partials.is_contiguous()):
+        raise KernelError(f"gemm_mid: partials must be [{splits},{m},{n}]")
+    _check(_fn("gemm", "dryft_gemm_mid_bf16")(_ptr(x), x.stride(0), _ptr(w), _ptr(partials), m, n, k, int(splits),
+                                              _stream()), "gemm_mid_bf16")
+    return partials
 
 
 def gemm_wide_swiglu_bf16(x, w_gate_up, out, group_blocks: int = 2, depth: int = 1) -> torch.Tensor:

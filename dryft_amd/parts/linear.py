@@ -16,6 +16,8 @@ engine/dryft_qwen3/model.py:153, 179-180, 237, 258-261). Here:
   partial sums (the projections back to the hidden width, which give the vendor library too
   few tiles to fill the chip), where the result is wanted in float32 (the output head) and
   for sizes the vendor library does not take;
+* bfloat16, 65 to 256 rows (short prompts), the projections back to the hidden width where the consumer adds
+  partial sums: this library's kernel that splits K and brings its operands straight into LDS (``mid_plan``);
 * bfloat16, otherwise (prompts, decoding at large batch): the vendor library through
   ``torch.mm``, as in the reference; float32 results of many rows and output sizes the
   library does not take are this library's block kernel (128 x 128 or 256 x 256 outputs
@@ -65,6 +67,19 @@ def wide_plan(n: int, k: int, may_split: bool) -> tuple[int, int, int]:
     k_blocks = (k + 63) // 64
     splits = max(1, min(_COMPUTE_UNITS // tiles, k_blocks // 4, 16)) if may_split else 1
     return (splits, 1, 3) if splits > 1 else (1, 2, 1)
+
+
+def mid_plan(n: int, k: int) -> int:
+    """Splits of K across workgroups for the kernel that takes the projections back to the hidden width at 65 to 256
+    rows (64 outputs a workgroup): as many as give every compute unit one workgroup, twice that where a split would
+    still walk more than 64 groups of K; 1 (not worth it) where the outputs alone fill the chip. Measured on the o
+    and down shapes of 4B, 8B and 32B models at 80, 128 and 192 rows."""
+    blocks = (n + 63) // 64
+    groups = k // ops.MID_GROUP
+    splits = _COMPUTE_UNITS // blocks
+    if splits >= 1 and groups // max(splits, 1) > 64:
+        splits *= 2
+    return ops.gemm_mid_splits(k, min(splits, 16)) if splits > 1 else 1
 
 
 def few_rows_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
@@ -117,6 +132,12 @@ def linear(x: torch.Tensor, w: torch.Tensor, *, out_dtype: torch.dtype | None = 
             out = torch.empty((m, n), dtype=out_dtype, device=x.device)
             ops.gemm_wide_bf16(x, w, out, None, group, 1, depth)
             return out
+    if m <= ops.MID_ROWS and allow_partials and few_ok and k % ops.MID_GROUP == 0:
+        splits = mid_plan(n, k)
+        if splits > 1:
+            partials = torch.empty((splits, m, n), dtype=torch.float32, device=x.device)
+            ops.gemm_mid_bf16(x, w, partials, splits)
+            return Partials(partials, splits)
     if library_ok:
         return torch.mm(x, w.t())
     out = torch.empty((m, n), dtype=out_dtype, device=x.device)

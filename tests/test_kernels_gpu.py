@@ -631,6 +631,47 @@ def test_gemm_panel_swiglu(m, inter, k):
         ops().gemm_panel_swiglu_bf16(x.to(DEV)[:, :64].contiguous(), w.to(DEV)[:, :64].contiguous(), out)
 
 
+@pytest.mark.parametrize("m", [1, 65, 128, 129, 192, 193, 256])
+@pytest.mark.parametrize("n,k,splits", [(2560, 4096, 6), (77, 64, 1), (100, 192, 3), (136, 640, 4), (64, 1024, 16),
+                                         (130, 9728, 6)])
+def test_gemm_mid(m, n, k, splits):
+    """Float partial sums over runs of K, operands straight into LDS: row counts around the kernel's three tile
+    counts, output counts that are no multiple of 4 or of the 64 a workgroup owns, one group of K and many, runs of
+    unequal length; every split against the product over its own run; a row of x strided wider than K."""
+    torch.manual_seed(m + n + k)
+    o = ops()
+    assert o.gemm_mid_splits(k, splits) == splits
+    x, w = torch.randn(m, k).to(torch.bfloat16), (torch.randn(n, k) / math.sqrt(k)).to(torch.bfloat16)
+    parts = torch.full((splits, m, n), float("nan"), dtype=torch.float32, device=DEV)
+    o.gemm_mid_bf16(x.to(DEV), w.to(DEV), parts, splits)
+    groups = k // 64
+    per = -(-groups // splits)
+    for s in range(splits):
+        a, b = 64 * per * s, min(k, 64 * per * (s + 1))
+        close(parts[s], x[:, a:b].double() @ w[:, a:b].double().T, torch.float32, what=f"mid, split {s}")
+    close(parts.sum(0), x.double() @ w.double().T, torch.float32, what="mid, sum")
+    wide = torch.zeros(m, k + 8, dtype=torch.bfloat16, device=DEV)
+    wide[:, :k] = x.to(DEV)
+    parts2 = torch.full((splits, m, n), float("nan"), dtype=torch.float32, device=DEV)
+    o.gemm_mid_bf16(wide[:, :k], w.to(DEV), parts2, splits)
+    assert torch.equal(parts, parts2)
+
+
+def test_gemm_mid_refuses():
+    o = ops()
+    x, w = torch.zeros(257, 128, dtype=torch.bfloat16, device=DEV), torch.zeros(64, 128, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(Exception, match="M <= 256"):
+        o.gemm_mid_bf16(x, w, torch.empty(1, 257, 64, device=DEV), 1)
+    with pytest.raises(Exception, match="K % 64"):
+        o.gemm_mid_bf16(x[:100, :96].contiguous(), w[:, :96].contiguous(), torch.empty(1, 100, 64, device=DEV), 1)
+    assert o.gemm_mid_splits(5 * 64, 4) == 3                  # four runs of two groups would leave the last one empty
+    with pytest.raises(Exception, match="empty"):
+        o.gemm_mid_bf16(x[:100, :64].contiguous().repeat(1, 5), w[:, :64].contiguous().repeat(1, 5),
+                        torch.empty(4, 100, 64, device=DEV), 4)
+    with pytest.raises(Exception, match="partials must be"):
+        o.gemm_mid_bf16(x[:100], w, torch.empty(1, 100, 64, device=DEV), 2)
+
+
 @pytest.mark.parametrize("m,n,k", [(130, 331, 72), (1, 17, 8), (257, 128, 64), (300, 100, 1000), (128, 129, 136),
                                    (513, 2560, 2560), (64, 64, 9728)])
 @pytest.mark.parametrize("shape", [0, 1])
@@ -693,14 +734,14 @@ def test_linear_dispatch_matches_everywhere():
     torch.manual_seed(5)
     for n, k in ((384, 96), (100, 2560), (331, 72)):           # 331 outputs: no size the vendor library takes
         w = (torch.randn(n, k) / math.sqrt(k)).to(torch.bfloat16).to(DEV)
-        for m in (1, 7, 16, 17, 64, 65, 300):
+        for m in (1, 7, 16, 17, 64, 65, 130, 256, 257, 300):
             x = torch.randn(m, k).to(torch.bfloat16).to(DEV)
             want = x.double().cpu() @ w.double().cpu().T
             close(linear(x, w), want, torch.bfloat16, ulps=1.0, what=f"linear m={m}")
             close(linear(x, w, out_dtype=torch.float32), want, torch.float32, what=f"linear m={m} float32 out")
             got = linear(x, w, allow_partials=True)
             if isinstance(got, Partials):
-                assert got.count > 1 and m <= 64
+                assert got.count > 1 and (m <= 64 or (m <= 256 and k % 64 == 0))
                 got = got.data[: got.count].sum(0)
             close(got, want, torch.bfloat16, ulps=1.0, what=f"linear partials m={m}")
             close(linear(x.float(), w.float()), want, torch.float32, what=f"linear float32 m={m}")
