@@ -522,6 +522,22 @@ def test_decoding_across_context_ranges(cases, dtype):
     assert list(engine.generate(prompts, 12)) == ours
 
 
+@pytest.mark.parametrize("name,n_seqs", [("A_sharp", 70), ("B", 130), ("C_sharp", 200)])
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_many_sequences_decode_through_the_graph(cases, dtype, name, n_seqs):
+    """More sequences than the few-row products take (64): the decoding steps of 70 and 130 sequences, captured, give
+    the plain loop's tokens, and the same with fewer requests than slots in the next batch."""
+    case = cases[name]
+    engine = case.engine(dtype, max_batch=n_seqs, max_len=128, use_graph=True)
+    rng = np.random.default_rng(n_seqs)
+    prompts = [random_tokens(int(rng.integers(1, 40)), case.vocab, seed=9000 + i) for i in range(n_seqs)]
+    ours = list(engine.generate(prompts, 4))
+    check_generation(case, prompts, ours, 4, dtype)
+    fewer = prompts[: n_seqs - 3]
+    check_generation(case, fewer, list(engine.generate(fewer, 3)), 3, dtype)
+    assert engine.cache.slots.free_count == n_seqs
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_graph_replay_equals_eager(cases, dtype):
     """A captured decoding step gives bit-identical logits to the same step run eagerly."""
