@@ -88,21 +88,15 @@ def _check(rc: int, what: str) -> None:
         raise KernelError(f"{what}: launch failed with HIP error {rc}")
 
 
-def _require(cond: bool, msg: str) -> None:
-    if not cond:
-        raise KernelError(msg)
-
-
 def _gpu(t: torch.Tensor, name: str, dtype=None) -> None:
     if not (isinstance(t, torch.Tensor) and t.is_cuda):
         raise KernelError(f"{name}: must be a GPU tensor (there is no CPU path)")
-    if dtype is not None:
-        if not (t.dtype == dtype):
-            raise KernelError(f"{name}: expected {dtype}, got {t.dtype}")
+    if dtype is not None and t.dtype != dtype:
+        raise KernelError(f"{name}: expected {dtype}, got {t.dtype}")
 
 
 def _float_flag(t: torch.Tensor, name: str) -> int:
-    if not (t.dtype in (torch.float32, torch.bfloat16)):
+    if t.dtype not in (torch.float32, torch.bfloat16):
         raise KernelError(f"{name}: expected float32 or bfloat16, got {t.dtype}")
     return 1 if t.dtype == torch.float32 else 0
 
@@ -384,9 +378,8 @@ def attn_split_bf16(q, k_pages, v_pages, page_table, seq_slot, cu_rows, kv_len, 
             raise KernelError(f"{name}: needs {n} entries")
     _gpu(part_o, "part_o", torch.float32)
     _gpu(part_ml, "part_ml", torch.float32)
-    if not (
-            part_o.numel() >= n_seqs * n_heads * n_splits * head_dim and part_ml.numel() >= n_seqs * n_heads * n_splits * 2
-    ):
+    entries = n_seqs * n_heads * n_splits
+    if part_o.numel() < entries * head_dim or part_ml.numel() < entries * 2:
         raise KernelError("attn_split: partial buffers too small")
     if not (n_splits <= 65535 and n_kv * ((n_heads // n_kv + 15) // 16) <= 65535):
         raise KernelError("attn_split: grid too large")
@@ -437,9 +430,8 @@ def attn_decode_fused_bf16(qkv, q_weight, k_weight, eps: float, cos, sin, rot: i
             raise KernelError(f"{name}: needs {n} entries")
     _gpu(part_o, "part_o", torch.float32)
     _gpu(part_ml, "part_ml", torch.float32)
-    if not (
-            part_o.numel() >= n_seqs * n_heads * n_splits * head_dim and part_ml.numel() >= n_seqs * n_heads * n_splits * 2
-    ):
+    entries = n_seqs * n_heads * n_splits
+    if part_o.numel() < entries * head_dim or part_ml.numel() < entries * 2:
         raise KernelError("attn_decode_fused: partial buffers too small")
     _check(_fn("attn_mfma", "dryft_attn_decode_fused_bf16")(
         _ptr(qkv), qkv.stride(0), _ptr(q_weight), _ptr(k_weight), w_f32, int(has_norm), float(eps), _ptr(cos), _ptr(sin),
@@ -658,18 +650,14 @@ def gemm_block_bf16(x, w, out, swiglu: bool = False, shape: int | None = None) -
     _gpu(out, "out")
     m, k = x.shape
     n = w.shape[0] // 2 if swiglu else w.shape[0]
-    if not (
-            w.dim() == 2 and w.shape[1] == k and w.is_contiguous() and x.stride(1) == 1 and (not swiglu or w.shape[0] % 2 == 0)
-    ):
+    if not (w.dim() == 2 and w.shape[1] == k and w.is_contiguous() and x.stride(1) == 1) or (swiglu and w.shape[0] % 2):
         raise KernelError("gemm_block: x [M,K] row-major, w [N,K] (or [2N,K]) contiguous")
     if not (k % 8 == 0 and x.stride(0) % 8 == 0):
         raise KernelError(f"gemm_block: needs K % 8 == 0, got K={k}")
     if not (x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0):
         raise KernelError("gemm_block: operands must be 16-byte aligned")
-    if not (
-            out.shape == (m, n) and out.is_contiguous() and out.dtype in (torch.float32, torch.bfloat16) and
-            not (swiglu and out.dtype != torch.bfloat16)
-    ):
+    out_dtypes = (torch.bfloat16,) if swiglu else (torch.float32, torch.bfloat16)
+    if not (out.shape == (m, n) and out.is_contiguous() and out.dtype in out_dtypes):
         raise KernelError(f"gemm_block: out must be contiguous [{m},{n}]")
     if shape is None:
         shape = 1 if -(-m // 256) * -(-(2 * n if swiglu else n) // 256) >= 256 else 0
