@@ -617,6 +617,40 @@ def test_layer_sizes_of_a_real_model_bfloat16_agrees_with_float32():
     assert engines["bfloat16"].cache.slots.free_count == 40
 
 
+def test_a_sequence_longer_than_65536_tokens():
+    """One layer with Qwen3-4B's head geometry and one sequence of 66,001 tokens (positions and page counts past 16
+    bits): the bfloat16 engine against the float32 engine, which shares no attention or matrix kernel with it, at the
+    prompt's last positions and three decoded tokens; and the same prompt cut into two portions and two single
+    tokens, which must give the same logits within rounding."""
+    from dryft_amd import Engine
+    from dryft_amd.engine.step import SeqStep
+    from dryft_amd.models import load_preset
+    raw = dict(load_preset("qwen3-4b"))
+    raw.update(num_hidden_layers=1, vocab_size=4096)
+    n = 66_001
+    tokens = random_tokens(n + 3, 4096, seed=5)
+    got = {}
+    for dtype in ("bfloat16", "float32"):
+        engine = Engine(config=raw, seed=3, dtype=dtype, max_batch=1, max_len=n + 64, max_tokens=n + 128)
+        for mode in (("whole", "cut") if dtype == "bfloat16" else ("whole",)):
+            slot = engine.acquire(1)[0]
+            if mode == "whole":
+                rows = [engine.step([SeqStep(slot, tokens[:n], [n - 2, n - 1])]).float().cpu()]
+            else:
+                engine.step([SeqStep(slot, tokens[:40_000], [])])
+                engine.step([SeqStep(slot, tokens[40_000:n - 2], [])])
+                rows = [engine.step([SeqStep(slot, [tokens[i]], [0])]).float().cpu() for i in (n - 2, n - 1)]
+            rows += [engine.step([SeqStep(slot, [tokens[n + t]], [0])]).float().cpu() for t in range(3)]
+            engine.release([slot])
+            got[(dtype, mode)] = torch.cat(rows)
+        del engine
+    ref = got[("float32", "whole")]
+    assert torch.isfinite(ref).all()
+    for key in (("bfloat16", "whole"), ("bfloat16", "cut")):
+        err = float((got[key] - ref).abs().max()) / float(ref.abs().max())
+        assert err <= TOL["bfloat16"], (key, err)
+
+
 REAL_LENGTHS = [78, 308, 1108] + list(range(20, 44))
 
 
