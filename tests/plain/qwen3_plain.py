@@ -1,10 +1,11 @@
 """A plain, slow Qwen3 dense decoder: whole sequences, no cache, one function per part.
 
 Written from the reference's formulas (cited per function as file:line under the
-reference's root); it shares no code with ``dryft_amd``. Everything runs on the CPU in
-one floating dtype (float32 by default, float64 to bound its own rounding), with library
-routines (``torch.softmax``, ``F.silu``, ``@``). Inputs are the raw ``config.json``
-dictionary and a dictionary of checkpoint tensors by name.
+reference's root); it shares no code with ``dryft_amd``. Everything runs in one floating
+dtype (float32 by default, float64 to bound its own rounding) with library routines
+(``torch.softmax``, ``F.silu``, ``@``), on the CPU unless the weights it is handed sit on
+another device (layers of a real model's sizes take minutes in float64 on a CPU). Inputs are
+the raw ``config.json`` dictionary and a dictionary of checkpoint tensors by name.
 """
 
 from __future__ import annotations
@@ -53,8 +54,8 @@ def causal_gqa_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scal
     k = k.repeat_interleave(group, dim=1)      # [T, nH, d]
     v = v.repeat_interleave(group, dim=1)
     scores = torch.einsum("ihd,jhd->hij", q, k) * scale
-    i = torch.arange(T)[:, None]
-    j = torch.arange(T)[None, :]
+    i = torch.arange(T, device=q.device)[:, None]
+    j = torch.arange(T, device=q.device)[None, :]
     visible = j <= i
     if window is not None:
         visible = visible & (i - j < window)
@@ -104,10 +105,11 @@ def forward(cfg: dict, weights: dict, tokens, dtype=torch.float32) -> torch.Tens
     engine/dryft_qwen3/model.py:132 (embedding gather), 152 (layers in order), 185-186 (final norm, head);
     weights.py:47-49 (a tied head is the embedding)."""
     w = {k: v.to(dtype) for k, v in weights.items()}
-    ids = torch.as_tensor(tokens, dtype=torch.long)
+    device = w["model.embed_tokens.weight"].device
+    ids = torch.as_tensor(tokens, dtype=torch.long).to(device)
     n_heads = cfg["num_attention_heads"]
     d = cfg.get("head_dim") or cfg["hidden_size"] // n_heads
-    cos, sin = rope_tables(d, cfg["rope_theta"], len(ids), dtype)
+    cos, sin = (t.to(device) for t in rope_tables(d, cfg["rope_theta"], len(ids), dtype))
     x = w["model.embed_tokens.weight"][ids]
     for i in range(cfg["num_hidden_layers"]):
         x = decoder_layer(x, w, i, cfg, cos, sin)

@@ -244,6 +244,13 @@ CASES = [  # n_heads, n_kv, D, lengths (cached tokens incl. the rows'), q rows p
     (8, 2, 32, [31, 13, 6, 1], 31),
     (6, 3, 48, [129, 90], 64),
     (4, 2, 16, [300], 300),
+    # head size 128 with eight, five and two query heads to a kv head (the architecture allows any whole number)
+    (64, 8, 128, [1, 513, 300, 64], 1),
+    (40, 8, 128, [257, 64, 1, 130], 1),
+    (16, 8, 128, [700, 65], 1),
+    (64, 8, 128, [150, 64, 209], 70),
+    (40, 8, 128, [150, 64, 209], 70),
+    (16, 8, 128, [150, 64, 209], 70),
 ]
 
 
@@ -330,6 +337,9 @@ CAUSAL_CASES = CASES + [      # many rows: several tiles per sequence, sequences
     (32, 8, 128, [260], 260),
     (32, 8, 128, [700, 330], 290),      # rows that continue after 410 and 40 cached tokens
     (9, 3, 32, [200, 150, 1, 65], 200),   # three heads to a kv head: no pairs of heads
+    (64, 8, 128, [260, 70], 260),
+    (40, 8, 128, [330, 129], 200),
+    (16, 8, 128, [700, 330], 290),
 ]
 
 
@@ -372,7 +382,8 @@ def test_attn_split_bf16(case, splits):
 
 # The reference's own lengths for its split-KV kernel (kernels/attn_decode.py:204-215) at Qwen3-4B's heads: a
 # split here walks up to 128 pages, four waves taking them in turn.
-LONG_DECODE = [(32, 8, 128, [2047], 1), (32, 8, 128, [8191, 4096], 1), (32, 8, 128, list(range(3, 3 + 16 * 31, 31)), 1)]
+LONG_DECODE = [(32, 8, 128, [2047], 1), (32, 8, 128, [8191, 4096], 1), (32, 8, 128, list(range(3, 3 + 16 * 31, 31)), 1),
+               (64, 8, 128, [2047, 4100], 1), (40, 8, 128, [8191, 2049], 1), (16, 8, 128, [2047, 4096], 1)]
 
 
 @pytest.mark.parametrize("splits", [1, 8, 32])
@@ -384,7 +395,9 @@ def test_attn_split_bf16_long_sequences(case, splits):
 
 
 @pytest.mark.parametrize("n_heads,n_kv,D,splits,window", [(32, 8, 128, 3, 0), (6, 3, 48, 1, 0), (4, 2, 16, 2, 0),
-                                                          (16, 1, 64, 4, 0), (8, 2, 32, 2, 50)])
+                                                          (16, 1, 64, 4, 0), (8, 2, 32, 2, 50),
+                                                          (64, 8, 128, 3, 0), (40, 8, 128, 2, 0), (16, 8, 128, 4, 0),
+                                                          (10, 2, 128, 1, 70)])
 def test_attn_decode_fused_equals_the_two_kernels(n_heads, n_kv, D, splits, window):
     """Norm + rotation + append + attention in one kernel gives what the separate kernels give, bit for bit,
     in the output and in the cache."""
@@ -433,16 +446,17 @@ def test_attn_decode_fused_equals_the_two_kernels(n_heads, n_kv, D, splits, wind
     assert torch.equal(k3, k1) and torch.equal(v3, v1) and torch.equal(out3, out2)
 
 
+@pytest.mark.parametrize("heads", [(8, 2), (16, 2), (10, 2), (4, 2), (3, 3)])       # 4, 8, 5, 2 and 1 to a kv head
 @pytest.mark.parametrize("mode,few_rows,w_f32,window", [(1, False, False, 0), (3, False, True, 0), (0, True, False, 0),
                                                       (1, False, False, 100)])
-def test_prompt_attention_that_takes_the_queries_from_the_projection(mode, few_rows, w_f32, window):
+def test_prompt_attention_that_takes_the_queries_from_the_projection(mode, few_rows, w_f32, window, heads):
     """At head size 128 the prompt kernel norms and rotates the queries itself. It gives what the stand-alone
     kernel plus the prompt kernel give (the sum of squares is added up in another order, so a value may land on the
     neighbouring bfloat16 now and then), and the cache gets the same keys and values whether or not the queries are
     written out. Sequences continue cached tokens, one sits out, one has a single row."""
     torch.manual_seed(7 + mode)
     o = ops()
-    n_heads, n_kv, D = 8, 2, 128
+    (n_heads, n_kv), D = heads, 128
     assert o.attn_causal_takes_projection(D, D) and not o.attn_causal_takes_projection(64, 64)
     assert not o.attn_causal_takes_projection(D, 64)
     q_lens = [3, 1, 5, 2] if few_rows else [150, 1, 70, 260]        # few rows: the append goes through the other kernels

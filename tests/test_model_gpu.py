@@ -31,7 +31,9 @@ LENGTHS = [1, 5, 9, 17, 33, 64, 65, 70, 128, 129, 131, 200]     # 64-token cache
 class Case:
     """A tiny model folder, its plain logits and engines on it."""
 
-    def __init__(self, name, tmp, sharp=False, raw=None, kw=None, lengths=LENGTHS, sharpness=4.0):
+    def __init__(self, name, tmp, sharp=False, raw=None, kw=None, lengths=LENGTHS, sharpness=4.0, plain_device="cpu"):
+        """``plain_device``: where the plain implementation computes (the GPU's float64 library routines for layers of
+        a real model's sizes, which would take minutes on the CPU)."""
         if raw is None:
             raw, kw = TINY[name]
         self.name = name
@@ -39,6 +41,8 @@ class Case:
         if sharp:
             self._sharpen(sharpness)
         self.raw, self.weights = read_model_dir(self.dir)
+        if plain_device != "cpu":
+            self.weights = {k: v.to(plain_device) for k, v in self.weights.items()}
         self.vocab = raw["vocab_size"]
         self.requests = {f"r{n}": random_tokens(n, self.vocab, seed=1000 + n) for n in lengths}
         self._plain = {}
@@ -57,7 +61,7 @@ class Case:
     def plain_logits(self, rid):
         rid = rid.split("#")[0]          # "r70#2" is request r70 replayed a second time
         if rid not in self._plain:
-            self._plain[rid] = plain.forward(self.raw, self.weights, self.requests[rid], torch.float64).float()
+            self._plain[rid] = plain.forward(self.raw, self.weights, self.requests[rid], torch.float64).float().cpu()
         return self._plain[rid]
 
     def tolerance(self, rid, dtype):
@@ -68,7 +72,7 @@ class Case:
         key = ("noise", rid)
         if key not in self._plain:
             ref = self.plain_logits(rid)
-            low = plain.forward(self.raw, self.weights, self.requests[rid], torch.bfloat16).float()
+            low = plain.forward(self.raw, self.weights, self.requests[rid], torch.bfloat16).float().cpu()
             self._plain[key] = float((low - ref).abs().max()) / float(ref.abs().max())
         return max(TOL[dtype], 2.0 * self._plain[key])
 
@@ -652,31 +656,50 @@ def test_a_sequence_longer_than_65536_tokens():
 
 
 REAL_LENGTHS = [78, 308, 1108] + list(range(20, 44))
+# Presets whose layer sizes the tests run at, two layers each and a vocabulary of 2,048: four, eight, five and two
+# query heads to a kv head at head size 128; widths 2560 to 5120; tied and untied heads.
+REAL_SIZES = {"4b": "qwen3-4b", "8b": "qwen3-8b", "32b": "qwen3-32b", "14b": "qwen3-14b", "0.6b": "qwen3-0.6b"}
+
+
+class RealCases:
+    """Cases at real layer sizes, made when first asked for; the plain implementation computes on the GPU in float64."""
+
+    def __init__(self, tmp):
+        self.tmp, self.made = tmp, {}
+
+    def get(self, size, sharp):
+        from dryft_amd.models import load_preset
+        if (size, sharp) not in self.made:
+            raw = dict(load_preset(REAL_SIZES[size]))
+            raw.update(num_hidden_layers=2, vocab_size=2048)
+            self.made[(size, sharp)] = Case("real" + size, self.tmp, sharp=sharp, raw=raw, lengths=REAL_LENGTHS,
+                                            kw=dict(seed=77, norm_std=0.1, std=0.02), sharpness=3.0,
+                                            plain_device="cuda:0")
+        return self.made[(size, sharp)]
+
+    def drop(self, size, sharp):
+        """Forgets a case with its engines and weights (the larger ones hold gigabytes of device memory)."""
+        self.made.pop((size, sharp), None)
+        torch.cuda.empty_cache()
 
 
 @pytest.fixture(scope="module")
 def real_cases(tmp_path_factory):
-    """Two layers with Qwen3-4B's layer sizes (head size 128, four query heads to a kv head, widths 2560 / 9728) and a
-    vocabulary of 2,048, small enough for the plain implementation in float64; once as drawn and once with
-    sharpened attention."""
-    from dryft_amd.models import load_preset
-    raw = dict(load_preset("qwen3-4b"))
-    raw.update(num_hidden_layers=2, vocab_size=2048)
-    tmp = str(tmp_path_factory.mktemp("real"))
-    kw = dict(seed=77, norm_std=0.1, std=0.02)
-    return {False: Case("real", tmp, raw=raw, kw=kw, lengths=REAL_LENGTHS),
-            True: Case("real", tmp, sharp=True, raw=raw, kw=kw, lengths=REAL_LENGTHS, sharpness=3.0)}
+    return RealCases(str(tmp_path_factory.mktemp("real")))
 
 
-@pytest.mark.parametrize("sharp", [False, True])
+REAL_RUNS = [("4b", False)] + [(size, True) for size in REAL_SIZES]
+
+
+@pytest.mark.parametrize("size,sharp", REAL_RUNS)
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_real_layer_sizes_against_plain(real_cases, dtype, sharp):
+def test_real_layer_sizes_against_plain(real_cases, dtype, size, sharp):
     """The sizes at which the matrix-core kernels take their fast paths, against the plain implementation (not
     against the other precision of the engine): prompts of 70, 300 and 1,100 tokens in one step with logits
     everywhere, then 8 given tokens each through the captured decoding graph; then 24 short sequences, whose
     decoding steps take the products of 17 to 64 rows."""
     from dryft_amd.engine.step import SeqStep
-    case = real_cases[sharp]
+    case = real_cases.get(size, sharp)
     engine = case.engine(dtype, max_batch=24, max_len=1280, max_tokens=3 * 1280 + 24 * 64, use_graph=True)
     names = ["r78", "r308", "r1108"]
     got = {}
@@ -723,12 +746,13 @@ def test_real_layer_sizes_against_plain(real_cases, dtype, sharp):
     check_against_plain(case, got, dtype, "real sizes, 24 sequences")
 
 
-@pytest.mark.parametrize("seed,max_batch", [(2000, 40), (2001, 8)])
+@pytest.mark.parametrize("size,seed,max_batch", [("4b", 2000, 40), ("4b", 2001, 8)] +
+                         [(size, 2002, 40) for size in REAL_SIZES if size != "4b"])
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_random_batches_at_real_layer_sizes(real_cases, dtype, seed, max_batch):
+def test_random_batches_at_real_layer_sizes(real_cases, dtype, size, seed, max_batch):
     """Batches drawn at random (up to 40 requests, so that the decoding steps take every product for 1 to 64 rows),
     at the sizes at which the matrix-core kernels take their fast paths, with sharpened attention."""
-    case = real_cases[True]
+    case = real_cases.get(size, True)
     records = random_trace(case, seed, max_batch=max_batch)
     engine = case.engine(dtype, max_batch=40, max_len=512, max_tokens=40 * 320)
     got = collect_positions(records, replay(engine, records))
