@@ -86,8 +86,10 @@ class CacheStore:
     sequence's count rounded up to whole pages; ``max_len`` bounds one sequence.
     """
 
-    def __init__(self, needs: dict[int, KVNeed | StateNeed | None], *, max_tokens: int, n_slots: int,
+    def __init__(self, needs: dict[int, KVNeed | StateNeed | dict | None], *, max_tokens: int, n_slots: int,
                  max_len: int, dtype: torch.dtype, device):
+        """``needs``: per cache line what it keeps: one need, or a dictionary from names to needs for a line that keeps
+        several things; ``line()`` then returns a dictionary of storage under the same names."""
         self.device = torch.device(device)
         self.dtype = dtype
         self.n_pages = max(1, pages_for(max_tokens))
@@ -98,10 +100,16 @@ class CacheStore:
         self.lengths_dev = torch.zeros(self.n_slots, dtype=torch.int32, device=self.device)
         self.kv_groups: list[KVGroup] = []
         self.state_groups: list[StateGroup] = []
-        self._line: dict[int, tuple[object, int]] = {}
-        by_need: dict[object, list[int]] = {}
+        self._line: dict[object, tuple[object, int]] = {}
+        self._named: dict[object, list[str]] = {}      # lines that keep several things: the names of those
+        by_need: dict[object, list[object]] = {}
         for line, need in needs.items():
-            if need is not None:
+            if isinstance(need, dict):
+                self._named[line] = list(need)
+                for name, one in need.items():
+                    if one is not None:
+                        by_need.setdefault(one, []).append((line, name))
+            elif need is not None:
                 by_need.setdefault(need, []).append(line)
         for need, lines in by_need.items():
             if isinstance(need, KVNeed):
@@ -116,7 +124,14 @@ class CacheStore:
                 self._line[line] = (g, i)
 
     # ---- what mixers see
-    def line(self, line: int) -> KVLine | StateLine | None:
+    def line(self, line):
+        """The storage of a cache line: a ``KVLine``, a ``StateLine``, None for a line that keeps nothing, or a
+        dictionary of those for a line that asked for several things by name."""
+        if line in self._named:
+            return {name: self._storage((line, name)) for name in self._named[line]}
+        return self._storage(line)
+
+    def _storage(self, line) -> KVLine | StateLine | None:
         entry = self._line.get(line)
         if entry is None:
             return None

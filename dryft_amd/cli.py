@@ -152,8 +152,9 @@ def cmd_bench(args) -> int:
 
 
 def cmd_profile(args) -> int:
-    """Per-kernel table of decoding steps or of one prompt step, from ``torch.profiler`` device events: calls and
-    microseconds per step, share, and for decoding the bandwidth the step's bytes imply (agent/profiler.py:58-89).
+    """Where the time of decoding steps or of one prompt step goes, from ``torch.profiler``'s averages per kernel
+    name: share, running share, microseconds and calls per step, and for decoding the bandwidth the step's bytes
+    imply (what agent/profiler.py:58-89 reports).
     Decoding steps run without graph capture so that every kernel is visible by name (profiler.py:47-48)."""
     import torch
     from torch.profiler import ProfilerActivity, profile
@@ -191,23 +192,23 @@ def cmd_profile(args) -> int:
             steps, what = args.steps, f"{args.steps} decoding steps of {args.batch} sequences at {args.prompt_len} tokens"
     finally:
         engine.release(slots)
-    rows: dict[str, list[float]] = {}
-    for ev in prof.events():
-        if getattr(ev, "device_type", None) is not None and "cuda" in str(ev.device_type).lower():
-            us = float(getattr(ev, "device_time", 0.0) or getattr(ev, "cuda_time", 0.0) or 0.0)
-            entry = rows.setdefault(ev.name, [0, 0.0])
-            entry[0] += 1
-            entry[1] += us
-    total = sum(v[1] for v in rows.values())
-    print(f"{what}: {total / steps:.1f} us of kernels per step")
-    print(f"{'kernel':72s} {'calls/step':>10s} {'us/step':>10s} {'share':>6s}")
-    for name, (count, us) in sorted(rows.items(), key=lambda kv: -kv[1][1])[: args.rows]:
-        print(f"{name[:72]:72s} {count / steps:10.1f} {us / steps:10.1f} {100 * us / max(total, 1e-9):5.1f}%")
+    # the profiler's own per-name averages, device kernels only, longest first, with the share that has run up so far
+    kernels = [(float(avg.self_device_time_total), int(avg.count), str(avg.key)) for avg in prof.key_averages()
+               if "cuda" in str(avg.device_type).lower() and avg.self_device_time_total > 0]
+    kernels.sort(reverse=True)
+    total = sum(us for us, _, _ in kernels)
+    launches = sum(n for _, n, _ in kernels)
+    print(f"{what}")
+    print(f"  {total / steps:.1f} us in {launches / steps:.0f} kernels a step")
+    so_far = 0.0
+    for us, n, name in kernels[: args.rows]:
+        so_far += us
+        print(f"  {us / total:6.1%} (to here {so_far / total:6.1%})  {us / steps:9.1f} us  x{n / steps:<6.1f} {name[:90]}")
     if not args.prefill and total > 0:
         weights = engine.model.streamed_weight_bytes()
         cache = args.batch * engine.cache.bytes_read(args.prompt_len + 2 + args.steps / 2)
-        print(f"implied bandwidth: {(weights + cache) / (total / steps * 1e-6) / 1e9:.0f} GB/s "
-              f"(weights read once, cache of the live sequences)")
+        print(f"  the weights once and the cache of the live sequences in that time: "
+              f"{(weights + cache) / (total / steps * 1e-6) / 1e9:.0f} GB/s")
     return 0
 
 
@@ -236,14 +237,14 @@ def cmd_attention(args) -> int:
         table = torch.arange(n_seqs * pages, dtype=torch.int32, device=dev).view(n_seqs, pages)
         seq_slot, seq_start = ints(list(range(n_seqs))), ints([0] * n_seqs)
         cu_rows = ints([length * i for i in range(n_seqs + 1)])
-        tile_cu = ints([ops.row_tiles(length) * i for i in range(n_seqs + 1)])
+        tile_cu = ints([(-(-length // ops.ATTN_ROW_TILE)) * i for i in range(n_seqs + 1)])
         flops = 2.0 * n_seqs * length * length * heads * dim
         calls = max(3, int(2e-3 * 0.8e15 / flops))
         best = {m: float("inf") for m in modes}
         for _ in range(4):
             for m in modes:
                 run = lambda: ops.attn_causal_bf16(q, k, v, table, seq_slot, cu_rows, tile_cu, seq_start, n_seqs,
-                                                   n_seqs * ops.row_tiles(length), out, heads, kv, dim, dim ** -0.5, 0, m)
+                                                   n_seqs * (-(-length // ops.ATTN_ROW_TILE)), out, heads, kv, dim, dim ** -0.5, 0, m)
                 run()
                 torch.cuda.synchronize()
                 begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)

@@ -498,7 +498,7 @@ __global__ __launch_bounds__(256, (GP * RP * KB <= 8 && KB <= 4) ? (GP * RP == 1
 
 // 16 bytes from base + offset (a base the whole wave shares, an offset per lane) to LDS byte lds_base + 16 * lane
 __device__ __forceinline__ void load_to_lds16(const void* base, uint32_t offset, uint32_t lds_base) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_base), "v"(offset), "s"(base) : "memory");
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_base), "v"(offset), "s"(base) : "memory", "m0");
 }
 
 // s_waitcnt vmcnt(0), leaving the other counters alone (vmcnt in bits 3:0 and 15:14, expcnt 6:4, lgkmcnt 11:8). As a

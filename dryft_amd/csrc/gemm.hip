@@ -552,7 +552,7 @@ DRYFT_API int dryft_gemm_wide_swiglu_bf16(const void* x, int64_t x_stride, const
 // Walking K from a different starting group in every workgroup took Qwen3-8B's gate/up (rows 8,192 bytes apart)
 // from 44 to 38 us at 8 to 40 rows; at Qwen3-4B's 5,120 bytes it changes nothing.
 __device__ __forceinline__ void panel_load16(const void* base, uint32_t offset, uint32_t lds_base) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_base), "v"(offset), "s"(base) : "memory");
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_base), "v"(offset), "s"(base) : "memory", "m0");
 }
 
 // s_waitcnt vmcnt(N) alone (vmcnt sits in bits 3:0 and 15:14 of the immediate, the other counters stay at their

@@ -18,7 +18,8 @@ from . import build
 
 _P, _I, _L, _F = c_void_p, c_int, c_int64, c_float
 _SIGNATURES = {
-    "batch": {"dryft_prepare_batch": [_P, _P, _P, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _P]},
+    "batch": {"dryft_prepare_batch": [_P, _P, _P, _I, _I, _P, _P, _P, _P, _P, _P, _P],
+              "dryft_tile_prefix": [_P, _P, _I, _I, _P, _P]},
     "embed": {"dryft_embed_rows": [_P, _P, _P, _I, _I, _I, _I, _P]},
     "norm": {"dryft_add_rmsnorm": [_P, _P, _I, _I, _L, _P, _I, _P, _P, _I, _I, _F, _I, _P],
              "dryft_add_rows": [_P, _P, _P, _L, _I, _P]},
@@ -106,26 +107,31 @@ def _ptr(t) -> int:
 
 
 # ------------------------------------------------------------------------------------------- batch
-ROW_TILE = 64      # rows of a sequence that one workgroup of the prompt-attention kernel takes (its smallest tile)
-
-
-def row_tiles(q_len: int) -> int:
-    """Tiles of ``ROW_TILE`` rows that a sequence bringing ``q_len`` rows occupies."""
-    return (q_len + ROW_TILE - 1) // ROW_TILE
-
-
-def prepare_batch(seq_slot, q_len, lengths, n_seqs: int, n_rows: int, cu_rows, tile_cu, kv_len, seq_start,
+def prepare_batch(seq_slot, q_len, lengths, n_seqs: int, n_rows: int, cu_rows, kv_len, seq_start,
                   row_seq, row_slot, row_pos) -> None:
     for name, t, n in (("seq_slot", seq_slot, n_seqs), ("q_len", q_len, n_seqs), ("cu_rows", cu_rows, n_seqs + 1),
-                       ("tile_cu", tile_cu, n_seqs + 1), ("kv_len", kv_len, n_seqs), ("seq_start", seq_start, n_seqs),
+                       ("kv_len", kv_len, n_seqs), ("seq_start", seq_start, n_seqs),
                        ("row_seq", row_seq, n_rows), ("row_slot", row_slot, n_rows), ("row_pos", row_pos, n_rows),
                        ("lengths", lengths, 1)):
         _gpu(t, name, torch.int32)
         if not (t.is_contiguous() and t.numel() >= n):
             raise KernelError(f"{name}: needs {n} contiguous entries, has {t.numel()}")
     _check(_fn("batch", "dryft_prepare_batch")(
-        _ptr(seq_slot), _ptr(q_len), _ptr(lengths), n_seqs, n_rows, ROW_TILE, _ptr(cu_rows), _ptr(tile_cu), _ptr(kv_len),
+        _ptr(seq_slot), _ptr(q_len), _ptr(lengths), n_seqs, n_rows, _ptr(cu_rows), _ptr(kv_len),
         _ptr(seq_start), _ptr(row_seq), _ptr(row_slot), _ptr(row_pos), _stream()), "prepare_batch")
+
+
+def tile_prefix(seq_slot, q_len, n_seqs: int, tile_rows: int, tile_cu) -> None:
+    """``tile_cu[s]``: how many tiles of ``tile_rows`` rows the sequences before ``s`` fill with their rows of this
+    step (a sequence that sits out, slot -1, fills none); ``tile_cu[n_seqs]``: the step's tiles."""
+    for name, t, n in (("seq_slot", seq_slot, n_seqs), ("q_len", q_len, n_seqs), ("tile_cu", tile_cu, n_seqs + 1)):
+        _gpu(t, name, torch.int32)
+        if not (t.is_contiguous() and t.numel() >= n):
+            raise KernelError(f"{name}: needs {n} contiguous entries, has {t.numel()}")
+    if tile_rows <= 0:
+        raise KernelError(f"tile_prefix: tiles of {tile_rows} rows")
+    _check(_fn("batch", "dryft_tile_prefix")(_ptr(seq_slot), _ptr(q_len), n_seqs, int(tile_rows), _ptr(tile_cu),
+                                             _stream()), "tile_prefix")
 
 
 # ------------------------------------------------------------------------------------------- embed
@@ -291,6 +297,9 @@ def attn_rows(q, k_pages, v_pages, page_table, row_slot, row_pos, out, n_heads: 
     _check(_fn("attn_rows", "dryft_attn_rows")(
         _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(page_table), page_table.shape[1], _ptr(row_slot), _ptr(row_pos),
         _ptr(out), rows, n_heads, n_kv, head_dim, float(scale), int(window), is_f32, _stream()), "attn_rows")
+
+
+ATTN_ROW_TILE = 64      # rows of a sequence that one workgroup of the prompt-attention kernels takes (``tile_cu``)
 
 
 def attn_causal_bf16(q, k_pages, v_pages, page_table, seq_slot, cu_rows, tile_cu, seq_start, n_seqs: int,
@@ -550,6 +559,7 @@ def gemm_wide_bf16(x, w, out, partials=None, group_blocks: int = 2, splits: int 
 
 
 PANEL_GROUP = 128     # values of K the panel kernel moves at a time; K must be a multiple of it
+DIRECT_REACH = 1 << 32    # bytes: the kernels that bring operands straight into LDS address them by 32-bit offsets
 
 
 def gemm_panel_waves(n_outputs: int) -> int:

@@ -14,6 +14,7 @@ from __future__ import annotations
 
 import sys
 import time
+from collections import OrderedDict
 from typing import Any, Iterator, Sequence
 
 import torch
@@ -40,6 +41,25 @@ def log(*parts: object) -> None:
     print("[engine]", *parts, file=sys.stderr, flush=True)
 
 
+def default_batch_buckets(max_batch: int) -> tuple[int, ...]:
+    """Batch sizes that captured decoding steps come in: every size up to 8, then four to an octave (10, 12, 14, 16,
+    20, 24, ...), the largest batch last. A step of another size runs in the next bucket with dead rows to fill it, at
+    most a quarter more rows than it has."""
+    sizes, n = [], 1
+    while n < max_batch:
+        sizes.append(n)
+        n += max(1, 1 << max(0, n.bit_length() - 3))
+    return tuple(sizes) + (int(max_batch),)
+
+
+def pick_bucket(buckets: Sequence[int], need: int) -> int:
+    """The smallest bucket that holds ``need`` (the reference's rule, engine/dryft_qwen3/config.py:203-207)."""
+    for b in buckets:
+        if b >= need:
+            return b
+    raise ValueError(f"{need} exceeds the largest bucket ({buckets[-1] if buckets else None})")
+
+
 def require_gpu(device) -> torch.device:
     device = torch.device(device)
     if device.type != "cuda" or not torch.cuda.is_available():
@@ -51,6 +71,7 @@ class PendingStep:
     """A launched decoding step: where its chosen tokens will be, and when."""
 
     def __init__(self, n: int, device: torch.device):
+        self.n = n                                            # how many of the entries are the batch's own
         self.chosen = torch.empty(n, dtype=torch.int32, device=device)
         self.host = torch.empty(n, dtype=torch.int32).pin_memory()
         self.done = torch.cuda.Event()
@@ -61,7 +82,12 @@ class Engine:
     def __init__(self, model_path: str | None = None, *, config: dict[str, Any] | None = None,
                  seed: int | None = None, norm_std: float = 0.0, dtype: str = "bfloat16", max_batch: int = 32,
                  max_len: int | None = None, max_tokens: int | None = None, use_graph: bool = True,
+                 batch_buckets: Sequence[int] | None = None, max_graphs: int | None = None,
                  device: str = "cuda:0", verbose: bool = False):
+        """``batch_buckets``: the batch sizes captured decoding steps are made for (default: see
+        ``default_batch_buckets``; the reference's are 1, 2, 4, ... 32, engine/dryft_qwen3/config.py:169); the largest
+        must be ``max_batch``. ``max_graphs``: how many captured steps are kept at most, the one used longest ago going
+        first (default: one per bucket and range of context lengths, so none ever goes)."""
         t0 = time.time()
         self.device = require_gpu(device)
         torch.cuda.set_device(self.device)
@@ -97,7 +123,18 @@ class Engine:
                                 max_len=self.max_len, dtype=self.dtype, device=self.device)
         self.stepper = Stepper(self.model, self.cache)
         self.use_graph = bool(use_graph)
-        self._graphs: dict[tuple[int, int], DecodeGraph] = {}     # (batch size, context range) -> captured step
+        buckets = sorted(set(int(b) for b in batch_buckets)) if batch_buckets is not None else \
+            list(default_batch_buckets(self.max_batch))
+        if not buckets or buckets[0] < 1 or buckets[-1] != self.max_batch:
+            raise ValueError(f"batch_buckets must be positive and end at max_batch ({self.max_batch}), got {buckets}")
+        self.batch_buckets = tuple(buckets)
+        self.max_graphs = int(max_graphs) if max_graphs is not None else len(buckets) * len(self.context_ranges())
+        if self.max_graphs < 1:
+            raise ValueError("max_graphs must be at least 1")
+        # (batch bucket, context range) -> captured step, least recently used first; one memory pool for all of them,
+        # since only one runs at a time
+        self._graphs: OrderedDict[tuple[int, int], DecodeGraph] = OrderedDict()
+        self._graph_pool = None
         self._sampler = Sampler()
         self._last_choice: torch.Tensor | None = None
         if verbose:
@@ -163,17 +200,22 @@ class Engine:
         live = [s for s in slots if s >= 0]
         lengths = self.cache.slots.lengths
         graph = self._graph_for(n, max((int(lengths[s]) + 1 for s in live), default=1))
+        width = graph.batch                                   # the bucket: rows beyond ``n`` are dead
+        slots = list(slots) + [-1] * (width - n)
         self.cache.begin_step(live, [1] * len(live))
         if tokens is None:
-            if self._last_choice is None or self._last_choice.numel() != n:
+            if self._last_choice is None or self._last_choice.numel() != width:
                 raise RuntimeError("no previous step of this batch to take the tokens from")
             logits = graph.replay(slots, self._last_choice)
         else:
-            logits = graph.replay(slots, tokens)
+            logits = graph.replay(slots, list(tokens) + [0] * (width - n))
         self.cache.end_step(live, [1] * len(live))
-        pending = PendingStep(n, self.device)
+        pending = PendingStep(width, self.device)
+        pending.n = n
         pending.sampler_state = self._sampler.state()
-        uniforms = None if self._sampler.greedy else self._sampler.draw(n)
+        uniforms = None
+        if not self._sampler.greedy:                          # the dead rows of the bucket draw nothing
+            uniforms = torch.cat([self._sampler.draw(n), torch.zeros(width - n)]) if width > n else self._sampler.draw(n)
         self._sampler.choose(logits, uniforms, out=pending.chosen)
         pending.host.copy_(pending.chosen, non_blocking=True)
         pending.done.record()
@@ -183,7 +225,7 @@ class Engine:
     def advance_end(self, pending: "PendingStep") -> list[int]:
         """The tokens a launched step chose (waits for that step only)."""
         pending.done.synchronize()
-        return pending.host.tolist()
+        return pending.host[:pending.n].tolist()
 
     def advance_drop(self, pending: "PendingStep") -> None:
         """Forgets the step launched last: its random numbers count as not drawn."""
@@ -205,23 +247,63 @@ class Engine:
         uniforms = None if self._sampler.greedy else self._sampler.draw(n)
         return self._sampler.choose(logits, uniforms).tolist()
 
+    def context_ranges(self) -> list[int]:
+        """The context lengths captured steps are sized for: 256, 512, 1,024, ... and the slot length last."""
+        ranges, reach = [], SHORTEST_GRAPH_CONTEXT
+        while reach < self.max_len:
+            ranges.append(reach)
+            reach *= 2
+        return ranges + [self.max_len]
+
     def _graph_for(self, batch: int, context: int | None = None) -> DecodeGraph | None:
         """The captured step for ``batch`` sequences whose longest will hold ``context`` tokens after the step
-        (default: as long as the cache allows): one graph per batch size and power-of-two range of contexts."""
+        (default: as long as the cache allows): one graph per batch bucket and power-of-two range of contexts,
+        captured when first asked for and kept until ``max_graphs`` others have been used since."""
         if not self.use_graph:
             return None
-        reach = self.max_len
-        if context is not None:
-            reach = SHORTEST_GRAPH_CONTEXT
-            while reach < context:
-                reach *= 2
-            reach = min(reach, self.max_len)
-        g = self._graphs.get((batch, reach))
+        bucket = pick_bucket(self.batch_buckets, batch)
+        reach = self.max_len if context is None else next((r for r in self.context_ranges() if r >= context), self.max_len)
+        key = (bucket, reach)
+        g = self._graphs.get(key)
         if g is None:
-            g = DecodeGraph(self.stepper, batch, reach)
+            while len(self._graphs) >= self.max_graphs:
+                self._graphs.popitem(last=False)
+            if self._graph_pool is None:
+                self._graph_pool = torch.cuda.graph_pool_handle()
+            g = DecodeGraph(self.stepper, bucket, reach, pool=self._graph_pool)
             g.capture()
-            self._graphs[(batch, reach)] = g
+            self._graphs[key] = g
+        self._graphs.move_to_end(key)
         return g
+
+    def warm(self, batch_sizes: Sequence[int] | None = None, contexts: Sequence[int] | None = None) -> int:
+        """Captures decoding steps before the first request needs them, as the reference does when it is built
+        (engine/dryft_qwen3/graphs.py:39-59): for the buckets of ``batch_sizes`` (default: every bucket) and the ranges
+        of the context lengths ``contexts`` (default: every range). Returns how many captured steps are held then."""
+        if not self.use_graph:
+            return 0
+        buckets = sorted(set(pick_bucket(self.batch_buckets, int(b)) for b in batch_sizes)) \
+            if batch_sizes is not None else list(self.batch_buckets)
+        ranges = self.context_ranges()
+        reaches = sorted(set(next((r for r in ranges if r >= int(c)), self.max_len) for c in contexts)) \
+            if contexts is not None else ranges
+        if len(buckets) * len(reaches) > self.max_graphs:
+            raise ValueError(f"{len(buckets)} x {len(reaches)} captured steps asked for, max_graphs is {self.max_graphs}")
+        for reach in reaches:
+            for bucket in buckets:
+                self._graph_for(bucket, reach)
+        return len(self._graphs)
+
+    def prepare(self, n: int, shortest_context: int, longest_context: int) -> None:
+        """What the generation loop says before a batch's first step: ``n`` sequences will decode at contexts between
+        these two. Captures what is missing now, so that no capture falls between two decoding steps."""
+        if self.use_graph:
+            ranges = self.context_ranges()
+            lo = next((r for r in ranges if r >= shortest_context), self.max_len)
+            hi = next((r for r in ranges if r >= longest_context), self.max_len)
+            wanted = [r for r in ranges if lo <= r <= hi]
+            for reach in wanted[-self.max_graphs:]:
+                self._graph_for(n, reach)
 
     # ------------------------------------------------------------------ generation
     def generate(self, input_ids: Sequence[Sequence[int]], max_new_tokens: int, *, temperature: float = 0.0,

@@ -36,6 +36,8 @@ class StepBackend(Protocol):
     #                                                                  before this one chose, kept on the device)
     #   advance_end(handle) -> list[int]
     #   advance_drop(handle)                                           (a launched step whose result nobody wants)
+    # A backend may also have ``prepare(n, shortest_context, longest_context)``: told before a batch's first step how
+    # many sequences will decode and between which context lengths, it can get ready what those steps need.
 
 
 def check_request(prompts: Sequence[Sequence[int]], max_new_tokens: int, max_len: int) -> None:
@@ -61,6 +63,9 @@ def generate_batch(backend: StepBackend, prompts: list[list[int]], max_new_token
     try:
         # a sequence needs room for its prompt and for every token that is fed back (all but the last)
         backend.reserve(slots, [len(p) + max_new_tokens - 1 for p in prompts])
+        if max_new_tokens > 1 and hasattr(backend, "prepare"):
+            # decoding steps will see contexts from the shortest prompt plus one to the longest sequence's end
+            backend.prepare(n, min(len(p) for p in prompts) + 1, max(len(p) for p in prompts) + max_new_tokens - 1)
         running = [True] * n
         tokens = backend.start(slots, [list(p) for p in prompts], 0)
         if getattr(backend, "chains", False):

@@ -21,17 +21,19 @@ from .step import BatchBuffers, Stepper, make_context
 
 
 class DecodeGraph:
-    def __init__(self, stepper: Stepper, batch_size: int, max_kv_len: int | None = None):
+    def __init__(self, stepper: Stepper, batch_size: int, max_kv_len: int | None = None, pool=None):
         """``max_kv_len``: the longest sequence the graph is meant for (default: the longest the cache holds). Parts
         size their launches by it (attention: into how many runs a sequence's keys are cut); a replay on longer
-        sequences is still right, only sized for shorter ones."""
+        sequences is still right, only sized for shorter ones. ``pool``: a graph memory pool to share with other
+        captured steps (only one of them may run at a time; what each returns stays its own)."""
+        self.pool = pool
         self.stepper, self.batch = stepper, int(batch_size)
         dev = stepper.device
         self.buf = BatchBuffers(self.batch, self.batch, dev)
         self.buf.q_len.fill_(1)
         self.max_kv_len = min(int(max_kv_len), stepper.cache.max_len) if max_kv_len else stepper.cache.max_len
         self.ctx: StepContext = make_context(self.buf, self.batch, self.batch, stepper.model.dtype, max_q_len=1,
-                                             max_tiles=self.batch, max_kv_len=self.max_kv_len, host=None)
+                                             max_kv_len=self.max_kv_len, host=None)
         self.logits: torch.Tensor | None = None
         self.graph: torch.cuda.CUDAGraph | None = None
         # Host-side staging for tokens and slots. Steps may be launched one ahead of the host reading their
@@ -54,7 +56,7 @@ class DecodeGraph:
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
+        with torch.cuda.graph(graph, pool=self.pool):
             self.logits = self._body()
         self.graph = graph
 

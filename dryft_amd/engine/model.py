@@ -64,13 +64,26 @@ class DecoderModel:
         return set(self.plan.optional_tensors)
 
     def load(self, tensors: dict[str, torch.Tensor]) -> None:
-        """Hands every part its tensors. Parts whose plans name the same checkpoint tensor share it."""
+        """Hands every part its tensors. Parts whose plans name the same checkpoint tensor share it. ``tensors`` is
+        emptied on the way: a tensor leaves it once the last part that reads it has loaded, so that a part which fuses
+        several tensors into one of its own (and so no longer holds them) frees them there and then, and loading never
+        holds much more than the weights themselves."""
         for extra, same_as in self.plan.optional_tensors.items():
             if extra in tensors and not torch.equal(tensors[extra], tensors[same_as]):
                 # the reference's check of a tied head's copy (engine/dryft_qwen3/weights.py:86-87)
                 raise ValueError(f"{extra} is present and differs from {same_as}, which the model reads in its place")
+            tensors.pop(extra, None)
+        readers: dict[str, int] = {}
         for part, names in self._bindings:
+            for logical in part.tensor_specs():
+                readers[names[logical]] = readers.get(names[logical], 0) + 1
+        for part, names in self._bindings:
+            wanted = [names[logical] for logical in part.tensor_specs()]
             part.load({logical: tensors[names[logical]] for logical in part.tensor_specs()})
+            for name in wanted:
+                readers[name] -= 1
+                if readers[name] == 0:
+                    tensors.pop(name, None)
 
     def kernel_modules(self) -> list[str]:
         mods = {"batch", "embed"}
@@ -122,21 +135,39 @@ class DecoderModel:
             part.prepare(n_positions, self.dtype, self.device)
 
     # ---- compute
-    def forward(self, tokens: torch.Tensor, ctx: StepContext, cache) -> torch.Tensor:
-        """Hidden states after the final norm, ``[rows, hidden]``."""
+    def forward(self, tokens: torch.Tensor, ctx: StepContext, cache, rows: torch.Tensor | None = None) -> torch.Tensor:
+        """Hidden states after the final norm, ``[rows, hidden]``: of every row of the step, or of ``rows`` alone
+        (int32 indices into the step's rows, on the device), which are picked before the final norm so that it runs
+        over nothing else."""
         ctx.positions = self.positions
         x = self.embedding.forward(tokens)
         pending = None
         for run in self.plan.schedule:
             x, pending = self.blocks[run.layer].forward(x, pending, ctx, cache.line(run.cache_line), run.writes_cache)
+        if rows is not None:
+            if rows.numel() == 0:                              # nothing is wanted: the layers have run, that is all
+                return x[:0]
+            x, pending = _pick_rows(x, rows), _pick_rows(pending, rows)
         if pending is None:
             return self.final_norm.forward(x)
         _, h = self.final_norm.add_forward(x, pending)
         return h
 
-    def logits(self, hidden: torch.Tensor, rows: torch.Tensor | None) -> torch.Tensor:
-        """Float32 logits at ``rows`` (int32 indices into the step's rows; None: all rows)."""
-        if rows is not None:
-            picked = torch.empty((rows.numel(), hidden.shape[1]), dtype=hidden.dtype, device=hidden.device)
-            hidden = ops.embed_rows(rows, hidden, picked)       # a row gather is a row gather
-        return self.head.forward(hidden)
+    def logits(self, hidden: torch.Tensor, rows: torch.Tensor | None = None) -> torch.Tensor:
+        """Float32 logits of hidden states that have been through the final norm (at ``rows`` of them; None: all)."""
+        return self.head.forward(hidden if rows is None else _pick_rows(hidden, rows))
+
+
+def _pick_rows(x, rows: torch.Tensor):
+    """Rows ``rows`` of a tensor ``[n, width]`` or of partial sums ``[count, n, width]`` (a row gather is what the
+    embedding kernel does)."""
+    if x is None:
+        return None
+    if isinstance(x, Partials):
+        count, n, width = x.count, x.data.shape[1], x.data.shape[2]
+        table = x.data[:count].reshape(count * n, width)
+        index = (rows[None, :] + n * torch.arange(count, dtype=torch.int32, device=rows.device)[:, None]).reshape(-1)
+        picked = torch.empty((count * rows.numel(), width), dtype=table.dtype, device=table.device)
+        return Partials(ops.embed_rows(index.contiguous(), table, picked).view(count, rows.numel(), width), count)
+    picked = torch.empty((rows.numel(), x.shape[1]), dtype=x.dtype, device=x.device)
+    return ops.embed_rows(rows, x, picked)

@@ -46,7 +46,6 @@ class BatchBuffers:
         self.seq_slot = torch.full((max_seqs,), -1, **i32)
         self.q_len = torch.zeros(max_seqs, **i32)
         self.cu_rows = torch.zeros(max_seqs + 1, **i32)
-        self.tile_cu = torch.zeros(max_seqs + 1, **i32)
         self.kv_len = torch.zeros(max_seqs, **i32)
         self.seq_start = torch.zeros(max_seqs, **i32)
 
@@ -77,26 +76,25 @@ def stage_batch(cache: CacheStore, buf: BatchBuffers, slots: list[int], q_lens: 
     buf.seq_slot[:n_seqs].copy_(stage[n_rows:n_rows + n_seqs])
     buf.q_len[:n_seqs].copy_(stage[n_rows + n_seqs:])
     ctx = make_context(buf, n_rows, n_seqs, dtype, max_q_len=max(q_lens),
-                       max_tiles=sum(ops.row_tiles(q) for q in live_q),
                        max_kv_len=max([st + q for st, q in zip(starts_live, live_q)], default=0),
                        host=HostBatch(list(slots), list(q_lens), starts))
     derive_rows(cache, buf, ctx)
     return ctx
 
 
-def make_context(buf: BatchBuffers, n_rows: int, n_seqs: int, dtype: torch.dtype, *, max_q_len: int, max_tiles: int,
+def make_context(buf: BatchBuffers, n_rows: int, n_seqs: int, dtype: torch.dtype, *, max_q_len: int,
                  max_kv_len: int, host: HostBatch | None) -> StepContext:
     return StepContext(n_rows=n_rows, n_seqs=n_seqs, dtype=dtype, device=buf.tokens.device,
                        row_seq=buf.row_seq, row_slot=buf.row_slot, row_pos=buf.row_pos, cu_rows=buf.cu_rows,
-                       tile_cu=buf.tile_cu, seq_slot=buf.seq_slot, q_len=buf.q_len, kv_len=buf.kv_len,
-                       seq_start=buf.seq_start, max_q_len=max_q_len, max_tiles=max_tiles, max_kv_len=max_kv_len,
+                       seq_slot=buf.seq_slot, q_len=buf.q_len, kv_len=buf.kv_len,
+                       seq_start=buf.seq_start, max_q_len=max_q_len, max_kv_len=max_kv_len,
                        host=host)
 
 
 def derive_rows(cache: CacheStore, buf: BatchBuffers, ctx: StepContext) -> None:
     """Per-row facts from per-sequence facts, on the device; advances the device's lengths."""
     ops.prepare_batch(buf.seq_slot, buf.q_len, cache.lengths_dev, ctx.n_seqs, ctx.n_rows, buf.cu_rows,
-                      buf.tile_cu, buf.kv_len, buf.seq_start, buf.row_seq, buf.row_slot, buf.row_pos)
+                      buf.kv_len, buf.seq_start, buf.row_seq, buf.row_slot, buf.row_pos)
 
 
 class Stepper:
@@ -139,12 +137,13 @@ class Stepper:
         q_lens = [len(s.tokens) for s in seqs]
         buf = self._buffers_for(len(tokens), len(seqs))
         ctx = stage_batch(self.cache, buf, slots, q_lens, tok, self.model.dtype)
-        hidden = self.model.forward(buf.tokens[:ctx.n_rows], ctx, self.cache)
+        # the wanted rows are picked before the final norm; when every row is wanted in order, nothing is picked
+        rows = None if wanted == list(range(ctx.n_rows)) else torch.tensor(wanted, dtype=torch.int32, device=self.device)
+        hidden = self.model.forward(buf.tokens[:ctx.n_rows], ctx, self.cache, rows)
         self.cache.end_step([s for s in slots if s >= 0], [q for s, q in zip(slots, q_lens) if s >= 0])
         if not wanted:
             return torch.empty((0, self.vocab), dtype=torch.float32, device=self.device)
-        rows = torch.tensor(wanted, dtype=torch.int32, device=self.device)
-        return self.model.logits(hidden, rows)
+        return self.model.logits(hidden)
 
     def run(self, buf: BatchBuffers, ctx: StepContext) -> torch.Tensor:
         """The device work of a step whose facts already sit in ``buf`` (what a captured graph holds)."""

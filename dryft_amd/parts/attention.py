@@ -82,10 +82,9 @@ class GQAAttention(Mixer):
             if ctx.max_kv_len > table.n_positions:
                 raise ValueError(f"position tables cover {table.n_positions} positions, the step reaches {ctx.max_kv_len}")
         window = self.window or 0
-        # Every kernel leaves the rows of sequences that sit out at zero; the tiled prompt kernel never visits them,
-        # so for it they are cleared beforehand.
-        sitting_out = ctx.host is not None and any(s < 0 for s in ctx.host.slots)
-        make = torch.zeros if sitting_out and ctx.max_q_len > 1 else torch.empty
+        # Every kernel leaves the rows of sequences that sit out at zero; the tiled prompt kernels never visit them,
+        # so for those the rows are cleared beforehand wherever the step may hold such sequences.
+        make = torch.zeros if ctx.max_q_len > 1 and ctx.some_sit_out() else torch.empty
         out = make((rows, self.n_heads, self.head_dim), dtype=h.dtype, device=h.device)
         # bfloat16 on the matrix cores where they take the head size; float32 and the other head sizes on the plain kernel
         matrix_cores = h.dtype == torch.bfloat16 and self.head_dim % MATRIX_CORE_HEAD_STEP == 0
@@ -108,9 +107,10 @@ class GQAAttention(Mixer):
                 ops.qk_norm_rope_kv(qkv, self.q_norm, self.k_norm, self.qk_norm_eps or 0.0, cos, sin, self.rotary_dim,
                                     ctx.row_slot, ctx.row_pos, None, line.k, line.v, line.page_table, True,
                                     self.n_heads, self.n_kv, self.head_dim)
+            tile_cu, max_tiles = ctx.tiles(ops.ATTN_ROW_TILE)
             ops.attn_causal_projected_bf16(qkv, self.q_norm, self.qk_norm_eps or 0.0, cos, sin, line.k, line.v,
-                                           line.page_table, ctx.seq_slot, ctx.cu_rows, ctx.tile_cu, ctx.seq_start,
-                                           ctx.n_seqs, ctx.max_tiles, out, self.n_heads, self.n_kv, self.head_dim,
+                                           line.page_table, ctx.seq_slot, ctx.cu_rows, tile_cu, ctx.seq_start,
+                                           ctx.n_seqs, max_tiles, out, self.n_heads, self.n_kv, self.head_dim,
                                            self.scale, window)
             return linear(out.view(rows, self.q_dim), self.w_o, allow_partials=True)
         q = torch.empty((rows, self.n_heads, self.head_dim), dtype=h.dtype, device=h.device)
@@ -122,8 +122,9 @@ class GQAAttention(Mixer):
                                 ctx.n_seqs, part_o, part_ml, splits, out, self.n_heads, self.n_kv, self.head_dim,
                                 self.scale, window)
         elif matrix_cores:
-            ops.attn_causal_bf16(q, line.k, line.v, line.page_table, ctx.seq_slot, ctx.cu_rows, ctx.tile_cu,
-                                 ctx.seq_start, ctx.n_seqs, ctx.max_tiles, out, self.n_heads, self.n_kv,
+            tile_cu, max_tiles = ctx.tiles(ops.ATTN_ROW_TILE)
+            ops.attn_causal_bf16(q, line.k, line.v, line.page_table, ctx.seq_slot, ctx.cu_rows, tile_cu,
+                                 ctx.seq_start, ctx.n_seqs, max_tiles, out, self.n_heads, self.n_kv,
                                  self.head_dim, self.scale, window)
         else:
             ops.attn_rows(q, line.k, line.v, line.page_table, ctx.row_slot, ctx.row_pos, out, self.n_heads, self.n_kv,

@@ -31,10 +31,14 @@ class StepContext:
 
     Rows are the step's tokens, packed sequence after sequence. Row ``r`` belongs to
     sequence ``row_seq[r]`` in cache slot ``row_slot[r]`` (-1: takes no part) at
-    position ``row_pos[r]``. ``cu_rows``/``tile_cu`` are prefix sums over sequences of
-    rows and of row tiles (``csrc.ops.ROW_TILE`` rows, for kernels that walk a step tile
-    by tile); ``kv_len`` is each sequence's cached length after this step, ``seq_start``
-    before it.
+    position ``row_pos[r]``. ``cu_rows`` are prefix sums over sequences of rows;
+    ``kv_len`` is each sequence's cached length after this step, ``seq_start`` before it.
+    A part whose kernel walks the step in tiles of some number of rows asks ``tiles()``
+    for the prefix sums of those.
+
+    ``host`` is the step as the host knows it, or None while a captured step is replayed.
+    A part must not let what it computes depend on whether ``host`` is there; it may only
+    use it to do less (skip clearing rows that no sequence sitting out owns).
     """
 
     n_rows: int
@@ -45,16 +49,36 @@ class StepContext:
     row_slot: torch.Tensor
     row_pos: torch.Tensor
     cu_rows: torch.Tensor
-    tile_cu: torch.Tensor
     seq_slot: torch.Tensor
     q_len: torch.Tensor
     kv_len: torch.Tensor
     seq_start: torch.Tensor
     max_q_len: int                      # host bound on rows per sequence; 1 means a decoding step
-    max_tiles: int                      # host bound on row tiles in the step
     max_kv_len: int                     # host bound on any sequence's cached length after the step
     host: HostBatch | None = None
     positions: dict[str, Any] = field(default_factory=dict)   # name -> position encoding, tables ready
+    _tiles: dict[int, tuple[torch.Tensor, int]] = field(default_factory=dict, repr=False)
+
+    def tiles(self, rows_per_tile: int) -> tuple[torch.Tensor, int]:
+        """For kernels that walk the step tile by tile: ``(tile_cu, bound)``. ``tile_cu`` (int32, device,
+        ``n_seqs + 1`` entries) holds the prefix sums over the sequences of the tiles of ``rows_per_tile`` rows that
+        their rows of this step fill (a sequence that sits out fills none); ``bound`` is what the host knows the
+        total not to exceed (a grid size). Computed when first asked for, once per tile size and step."""
+        from ..csrc import ops
+        found = self._tiles.get(rows_per_tile)
+        if found is None:
+            tile_cu = torch.empty(self.n_seqs + 1, dtype=torch.int32, device=self.device)
+            ops.tile_prefix(self.seq_slot, self.q_len, self.n_seqs, rows_per_tile, tile_cu)
+            if self.host is not None:
+                bound = sum(-(-q // rows_per_tile) for s, q in zip(self.host.slots, self.host.q_lens) if s >= 0)
+            else:
+                bound = self.n_seqs * -(-self.max_q_len // rows_per_tile)
+            found = self._tiles[rows_per_tile] = (tile_cu, bound)
+        return found
+
+    def some_sit_out(self) -> bool:
+        """May the step hold sequences that sit out (slot -1)? Without the host's view: yes."""
+        return self.host is None or any(s < 0 for s in self.host.slots)
 
 
 @dataclass
@@ -108,14 +132,17 @@ class Norm(Part):
 
 
 class Mixer(Part):
-    """Mixes information across positions of a sequence; owns one cache line per run."""
+    """Mixes information across positions of a sequence; owns the cache line of each of its runs."""
 
     def cache_need(self):
-        """A ``KVNeed``, a ``StateNeed`` or None."""
+        """What a run of this mixer keeps per sequence: a ``KVNeed``, a ``StateNeed``, None, or a dictionary from
+        names of its own choosing to needs when it keeps several things (keys and values beside fixed-size state,
+        two sets of keys with different windows)."""
         return None
 
     def forward(self, h: torch.Tensor, ctx: StepContext, line, writes_cache: bool):
-        """``h`` is ``[rows, hidden]``; returns a tensor of the same shape or ``Partials``."""
+        """``h`` is ``[rows, hidden]``; returns a tensor of the same shape or ``Partials``. ``line`` is the storage
+        ``cache_need`` asked for: a ``KVLine``, a ``StateLine``, None, or a dictionary of those under the same names."""
         raise NotImplementedError
 
 

@@ -95,7 +95,14 @@ def panel_swiglu_ok(x: torch.Tensor, w_gate_up: torch.Tensor) -> bool:
     Qwen3-8B's 36.7 against 37.8, 36.8 against 38.0, 37.6 against 52.1, 39.9 against 52.7; Qwen3-32B's 96.9 against
     98.4, 95.0 against 103.8, 97.6 against 100.9, 107.8 against 110.4."""
     m, k = x.shape
-    return m <= WIDE_ROWS and k % ops.PANEL_GROUP == 0 and few_rows_ok(x, w_gate_up)
+    return m <= WIDE_ROWS and k % ops.PANEL_GROUP == 0 and few_rows_ok(x, w_gate_up) and within_direct_reach(x, w_gate_up)
+
+
+def within_direct_reach(x: torch.Tensor, w: torch.Tensor) -> bool:
+    """Do both operands lie within what the kernels that bring them straight into LDS can address (32-bit byte
+    offsets from the operand's start)? Larger ones go to the kernels that hold 64-bit addresses."""
+    return w.numel() * w.element_size() < ops.DIRECT_REACH and \
+        x.shape[0] * x.stride(0) * x.element_size() < ops.DIRECT_REACH
 
 
 def linear(x: torch.Tensor, w: torch.Tensor, *, out_dtype: torch.dtype | None = None, allow_partials: bool = False):
@@ -132,7 +139,7 @@ def linear(x: torch.Tensor, w: torch.Tensor, *, out_dtype: torch.dtype | None = 
             out = torch.empty((m, n), dtype=out_dtype, device=x.device)
             ops.gemm_wide_bf16(x, w, out, None, group, 1, depth)
             return out
-    if m <= ops.MID_ROWS and allow_partials and few_ok and k % ops.MID_GROUP == 0:
+    if m <= ops.MID_ROWS and allow_partials and few_ok and k % ops.MID_GROUP == 0 and within_direct_reach(x, w):
         splits = mid_plan(n, k)
         if splits > 1:
             partials = torch.empty((splits, m, n), dtype=torch.float32, device=x.device)

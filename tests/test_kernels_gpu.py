@@ -394,6 +394,49 @@ def test_attn_split_bf16_long_sequences(case, splits):
         run_attention_case(splits, torch.bfloat16, *case, dead=(0,) if len(case[3]) > 1 else ())
 
 
+@pytest.mark.parametrize("kind", ["causal0", "causal1", "causal7", 16])
+def test_attention_past_65536_positions(kind):
+    """One sequence of 66,001 positions (positions, row numbers and page counts past 16 bits) against float64
+    arithmetic at sampled rows: the first, both sides of a page's edge, 65,535 and 65,536, and the last. The key that
+    stands out for each sampled row lies at a third of its distance, far from where a wrapped index would look. With
+    this many rows the kernel's own choice (mode 0) is 32 rows a wave."""
+    torch.manual_seed(9)
+    n, n_heads, n_kv, D = 66_001, 8, 2, 128
+    group = n_heads // n_kv
+    sampled = [0, 63, 64, 40_000, 65_535, 65_536, 65_999, 66_000]
+    k = torch.randn(1, n, n_kv, D).to(torch.bfloat16)
+    v = torch.randn(1, n, n_kv, D).to(torch.bfloat16)
+    decoding = not str(kind).startswith("causal")
+    rows = [n - 1] if decoding else list(range(n))
+    q = torch.randn(len(rows), n_heads, D).to(torch.bfloat16)
+    for r in ([n - 1] if decoding else sampled):
+        k[0, r // 3] = (3.0 * q[0 if decoding else r].float().view(n_kv, group, D).mean(1)).to(torch.bfloat16)
+    scale = D ** -0.5
+    k_pages, v_pages, table, slots = build_pages(k, v, [n], (n + 63) // 64 + 2, 3, seed=4, poison=1e4)
+    d = lambda t: t.to(DEV)
+    out = torch.zeros(len(rows), n_heads, D, dtype=torch.bfloat16, device=DEV)
+    o = ops()
+    seq_slot = d(torch.tensor(slots, dtype=torch.int32))
+    if decoding:
+        splits = kind
+        part_o = torch.empty(n_heads * splits * D, dtype=torch.float32, device=DEV)
+        part_ml = torch.empty(n_heads * splits * 2, dtype=torch.float32, device=DEV)
+        o.attn_split_bf16(d(q), d(k_pages), d(v_pages), d(table), seq_slot, d(torch.tensor([0, 1], dtype=torch.int32)),
+                          d(torch.tensor([n], dtype=torch.int32)), 1, part_o, part_ml, splits, out, n_heads, n_kv, D,
+                          scale, 0)
+    else:
+        tiles = (n + 63) // 64
+        o.attn_causal_bf16(d(q), d(k_pages), d(v_pages), d(table), seq_slot, d(torch.tensor([0, n], dtype=torch.int32)),
+                           d(torch.tensor([0, tiles], dtype=torch.int32)), d(torch.tensor([0], dtype=torch.int32)), 1,
+                           tiles, out, n_heads, n_kv, D, scale, 0, int(kind[6:]))
+    kk, vv = k[0].double().repeat_interleave(group, dim=1), v[0].double().repeat_interleave(group, dim=1)
+    for r in ([n - 1] if decoding else sampled):
+        i = 0 if decoding else r
+        s = torch.einsum("hd,jhd->hj", q[i].double(), kk[: r + 1]) * scale
+        want = torch.einsum("hj,jhd->hd", torch.softmax(s, -1), vv[: r + 1]).float()
+        close(out[i], want, torch.bfloat16, ulps=4.0, floor=1e-3, what=f"{kind}: row {r} of {n}")
+
+
 @pytest.mark.parametrize("n_heads,n_kv,D,splits,window", [(32, 8, 128, 3, 0), (6, 3, 48, 1, 0), (4, 2, 16, 2, 0),
                                                           (16, 1, 64, 4, 0), (8, 2, 32, 2, 50),
                                                           (64, 8, 128, 3, 0), (40, 8, 128, 2, 0), (16, 8, 128, 4, 0),
@@ -816,9 +859,12 @@ def test_prepare_batch():
     n_seqs, n_rows = 4, 202
     z = lambda n: torch.full((n,), -7, dtype=torch.int32, device=DEV)
     cu, tiles, kv, start, rseq, rslot, rpos = z(5), z(5), z(4), z(4), z(n_rows), z(n_rows), z(n_rows)
-    o.prepare_batch(seq_slot, q_len, lengths, n_seqs, n_rows, cu, tiles, kv, start, rseq, rslot, rpos)
+    o.prepare_batch(seq_slot, q_len, lengths, n_seqs, n_rows, cu, kv, start, rseq, rslot, rpos)
     assert cu.tolist() == [0, 70, 71, 72, 202]
+    o.tile_prefix(seq_slot, q_len, n_seqs, 64, tiles)
     assert tiles.tolist() == [0, 2, 2, 3, 6]
+    o.tile_prefix(seq_slot, q_len, n_seqs, 16, tiles)
+    assert tiles.tolist() == [0, 5, 5, 6, 15]
     assert kv.tolist() == [77, 0, 11, 133]
     assert start.tolist() == [7, 0, 10, 3]
     assert lengths.tolist() == [0, 11, 64, 77, 0, 133]
@@ -843,11 +889,13 @@ def test_prepare_batch_many_sequences(n_seqs):
     z = lambda n: torch.full((n,), -7, dtype=torch.int32, device=DEV)
     cu, tiles, kv, start = z(n_seqs + 1), z(n_seqs + 1), z(n_seqs), z(n_seqs)
     rseq, rslot, rpos = z(n_rows), z(n_rows), z(n_rows)
-    o.prepare_batch(seq_slot, q_len, lengths, n_seqs, n_rows, cu, tiles, kv, start, rseq, rslot, rpos)
+    o.prepare_batch(seq_slot, q_len, lengths, n_seqs, n_rows, cu, kv, start, rseq, rslot, rpos)
     live = slots >= 0
     want_start = np.where(live, past[np.maximum(slots, 0)], 0)
     assert cu.tolist() == [0] + np.cumsum(q).tolist()
-    assert tiles.tolist() == [0] + np.cumsum(np.where(live, (q + 63) // 64, 0)).tolist()
+    for tile_rows in (64, 48):
+        o.tile_prefix(seq_slot, q_len, n_seqs, tile_rows, tiles)
+        assert tiles.tolist() == [0] + np.cumsum(np.where(live, (q + tile_rows - 1) // tile_rows, 0)).tolist()
     assert start.tolist() == want_start.tolist()
     assert kv.tolist() == (want_start + np.where(live, q, 0)).tolist()
     new_len = past.copy()

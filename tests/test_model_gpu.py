@@ -526,6 +526,45 @@ def test_decoding_across_context_ranges(cases, dtype):
     assert list(engine.generate(prompts, 12)) == ours
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_batch_buckets_bound_the_captured_steps(cases, dtype):
+    """One engine generates at every batch size from 1 to 40 through captured steps that come in buckets of batch
+    sizes, the rows beyond a batch dead: the tokens are those of an engine with a captured step per exact size, greedy
+    and sampled; the number of captured steps stays within buckets x ranges; warmed beforehand, nothing is captured
+    and no device memory is taken during generation; a cap on their number drops the one used longest ago."""
+    from dryft_amd.engine.engine import default_batch_buckets, pick_bucket
+    case = cases["B"]
+    buckets = default_batch_buckets(40)
+    assert buckets == (1, 2, 3, 4, 5, 6, 7, 8, 10, 12, 14, 16, 20, 24, 28, 32, 40)
+    assert [pick_bucket(buckets, n) for n in (1, 8, 9, 17, 33, 40)] == [1, 8, 10, 20, 40, 40]
+    bucketed = case.engine(dtype, max_batch=40, max_len=256, use_graph=True)
+    exact = case.engine(dtype, max_batch=40, max_len=256, use_graph=True, batch_buckets=tuple(range(1, 41)))
+    assert bucketed.batch_buckets == buckets and bucketed.context_ranges() == [256]
+    assert bucketed.warm() == len(buckets) == len(bucketed._graphs)
+    rng = np.random.default_rng(5)
+    prompts = [random_tokens(int(rng.integers(1, 30)), case.vocab, seed=600 + i) for i in range(40)]
+    how = {n: dict(temperature=0.8, sample_seed=n) if n % 3 == 0 else {} for n in range(1, 41)}
+    want = {n: exact.generate_all(prompts[:n], 4, **how[n]) for n in range(1, 41)}
+    bucketed.generate_all(prompts, 2)                          # what a step itself holds on to (staging) exists now
+    torch.cuda.synchronize()
+    held = torch.cuda.memory_allocated()
+    for n in range(1, 41):
+        assert bucketed.generate_all(prompts[:n], 4, **how[n]) == want[n], f"batch of {n}"
+    assert len(bucketed._graphs) == len(buckets), "a step was captured although every bucket was warm"
+    torch.cuda.synchronize()
+    assert torch.cuda.memory_allocated() == held, "generation kept device memory although every bucket was warm"
+    assert len(exact._graphs) == 40
+    check_generation(case, prompts[:9], [list(col) for col in zip(*bucketed.generate_all(prompts[:9], 4))], 4, dtype)
+    # a cap: the captured step used longest ago goes, and comes back when asked for
+    capped = case.engine(dtype, max_batch=40, max_len=256, use_graph=True, max_graphs=2)
+    for n in (3, 9, 3, 17):
+        assert capped.generate_all(prompts[:n], 3) == exact.generate_all(prompts[:n], 3)
+    assert list(capped._graphs) == [(3, 256), (20, 256)]
+    with pytest.raises(ValueError, match="max_graphs"):
+        capped.warm()
+    assert bucketed.cache.slots.free_count == exact.cache.slots.free_count == 40
+
+
 @pytest.mark.parametrize("name,n_seqs", [("A_sharp", 70), ("B", 130), ("C_sharp", 200)])
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_many_sequences_decode_through_the_graph(cases, dtype, name, n_seqs):
@@ -653,6 +692,30 @@ def test_a_sequence_longer_than_65536_tokens():
     for key in (("bfloat16", "whole"), ("bfloat16", "cut")):
         err = float((got[key] - ref).abs().max()) / float(ref.abs().max())
         assert err <= TOL["bfloat16"], (key, err)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_a_long_prompt_beside_a_short_one_against_plain(tmp_path, dtype):
+    """One layer with Qwen3-4B's sizes, a prompt of 4,200 tokens beside one of 70 in one step: enough rows for the prompt
+    attention to take 32 rows a wave by its own choice. Logits at 16 places of the long prompt (its first and last
+    rows, both sides of page and tile edges) and at the short one's end, against the plain implementation in float64."""
+    from dryft_amd.engine.step import SeqStep
+    from dryft_amd.models import load_preset
+    raw = dict(load_preset("qwen3-4b"))
+    raw.update(num_hidden_layers=1, vocab_size=2048)
+    case = Case("long", str(tmp_path), sharp=True, raw=raw, kw=dict(seed=31, norm_std=0.1, std=0.02),
+                lengths=[4200, 70], sharpness=3.0, plain_device="cuda:0")
+    engine = case.engine(dtype, max_batch=2, max_len=4224)
+    places = [0, 1, 63, 64, 127, 128, 2047, 2048, 3000, 4095, 4096, 4159, 4160, 4197, 4198, 4199]
+    slots = engine.acquire(2)
+    try:
+        logits = engine.step([SeqStep(slots[0], case.requests["r4200"], places),
+                              SeqStep(slots[1], case.requests["r70"], [69])]).float().cpu()
+    finally:
+        engine.release(slots)
+    got = {("r4200", p): logits[i] for i, p in enumerate(places)}
+    got[("r70", 69)] = logits[len(places)]
+    check_against_plain(case, got, dtype, "long prompt beside a short one")
 
 
 REAL_LENGTHS = [78, 308, 1108] + list(range(20, 44))
@@ -797,7 +860,7 @@ def test_command_line_bench_and_profile():
     for r in lines:
         assert r["tok_s"] > 0 and r["total_ms"] >= r["ttft_ms"] > 0 and r["tpot_ms"] > 0
     out = run_cli("profile", "--tiny", "--batch", "2", "--prompt-len", "16", "--steps", "2")
-    assert "2 decoding steps of 2 sequences" in out and "implied bandwidth" in out
+    assert "2 decoding steps of 2 sequences" in out and "kernels a step" in out and "GB/s" in out
     table = out.splitlines()
     assert any("attn_split_kernel" in row for row in table) and any("add_rmsnorm" in row for row in table)
     out = run_cli("profile", "--tiny", "--batch", "2", "--prompt-len", "70", "--prefill")

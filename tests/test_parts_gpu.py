@@ -221,10 +221,11 @@ class ToyConfig:
     vocab_size: int
     decay: float
     intermediate_size: int
+    both: bool = False        # layer 0's mixer also attends: it keeps keys and values beside its state
 
     @classmethod
     def from_dict(cls, raw):
-        return cls(raw["hidden_size"], raw["vocab_size"], raw["decay"], raw["intermediate_size"])
+        return cls(raw["hidden_size"], raw["vocab_size"], raw["decay"], raw["intermediate_size"], raw.get("both", False))
 
 
 def toy_plan(cfg):
@@ -238,13 +239,15 @@ def toy_plan(cfg):
         return PartSpec("swiglu", dict(hidden_size=H, intermediate_size=cfg.intermediate_size),
                         {"gate_proj": f"l{i}.gate", "up_proj": f"l{i}.up", "down_proj": f"l{i}.down"})
 
+    attends = dict(hidden_size=H, num_heads=4, num_kv_heads=2, head_dim=16, positions="rotary")
+    first = PartSpec("toy_decay_mixer", dict(hidden_size=H, decay=cfg.decay), {"w_in": "l0.w_in", "w_out": "l0.w_out"})
+    if cfg.both:
+        first = PartSpec("toy_decay_attention", dict(decay=cfg.decay, **attends),
+                         {k: f"l0.{k}" for k in ("w_in", "w_out", "q_proj", "k_proj", "v_proj", "o_proj")})
     layers = (
-        LayerSpec("prenorm", {"mixer_norm": norm("l0.n1"), "ffn_norm": norm("l0.n2"), "ffn": ffn(0),
-                              "mixer": PartSpec("toy_decay_mixer", dict(hidden_size=H, decay=cfg.decay),
-                                                {"w_in": "l0.w_in", "w_out": "l0.w_out"})}),
+        LayerSpec("prenorm", {"mixer_norm": norm("l0.n1"), "ffn_norm": norm("l0.n2"), "ffn": ffn(0), "mixer": first}),
         LayerSpec("prenorm", {"mixer_norm": norm("l1.n1"), "ffn_norm": norm("l1.n2"), "ffn": ffn(1),
-                              "mixer": PartSpec("gqa_attention", dict(hidden_size=H, num_heads=4, num_kv_heads=2,
-                                                                      head_dim=16, positions="rotary"),
+                              "mixer": PartSpec("gqa_attention", attends,
                                                 {k: f"l1.{k}" for k in ("q_proj", "k_proj", "v_proj", "o_proj")})}),
     )
     return ModelPlan(vocab_size=cfg.vocab_size, hidden_size=H,
@@ -258,7 +261,7 @@ def register_toy():
     from dryft_amd import register_architecture, register_part
     from dryft_amd.cache import StateNeed
     from dryft_amd.models import known_architectures
-    from dryft_amd.parts.base import Mixer, matrix
+    from dryft_amd.parts.base import Mixer, Partials, matrix
 
     class DecayMixer(Mixer):
         """out_t = s_t @ w_out with s_t = decay * s_{t-1} + h_t @ w_in; s lives in the cache, one per sequence."""
@@ -289,8 +292,37 @@ def register_toy():
                 row += n
             return (out @ self.w_out.T).to(h.dtype)
 
+    class DecayAttention(Mixer):
+        """The decaying sum and attention side by side, their outputs added: one run keeps two things per sequence,
+        state of fixed size and keys and values, and is handed both by the names it gave them."""
+
+        def __init__(self, decay, **attention):
+            from dryft_amd.parts.attention import GQAAttention
+            self.sum = DecayMixer(attention["hidden_size"], decay)
+            self.attention = GQAAttention(**attention)
+
+        def tensor_specs(self):
+            return {**self.sum.tensor_specs(), **self.attention.tensor_specs()}
+
+        def load(self, tensors):
+            self.sum.load(tensors)
+            self.attention.load(tensors)
+
+        def kernel_modules(self, dtype):
+            return self.attention.kernel_modules(dtype)
+
+        def cache_need(self):
+            return {"sum": self.sum.cache_need(), "keys": self.attention.cache_need()}
+
+        def forward(self, h, ctx, line, writes_cache):
+            attended = self.attention.forward(h, ctx, line["keys"], writes_cache)
+            if isinstance(attended, Partials):
+                attended = attended.summed(h.dtype)
+            return (attended.float() + self.sum.forward(h, ctx, line["sum"], writes_cache).float()).to(h.dtype)
+
     if "ToyDecayLM" not in known_architectures():
         register_part("toy_decay_mixer", DecayMixer)
+        register_part("toy_decay_attention", DecayAttention)
         register_architecture("ToyDecayLM", ToyConfig, toy_plan)
 
 
@@ -306,35 +338,46 @@ def toy_plain(cfg, w, tokens):
     for t in range(T):
         s = cfg["decay"] * s + u[t]
         mixed.append(s)
+    cos, sin = P.rope_tables(16, 1e4, T, torch.float64)
+    x_in = x
     x = x + torch.stack(mixed) @ w["l0.w_out"].T
+    if cfg.get("both"):
+        q, k, v = ((h @ w[f"l0.{n}_proj"].T).view(T, heads, 16) for n, heads in (("q", 4), ("k", 2), ("v", 2)))
+        o = P.causal_gqa_attention(P.apply_rope(q, cos, sin), P.apply_rope(k, cos, sin), v, 0.25)
+        x = x_in + (torch.stack(mixed) @ w["l0.w_out"].T + o.reshape(T, 64) @ w["l0.o_proj"].T)
     x = x + P.swiglu(P.rms_norm(x, w["l0.n2"], 1e-5), {f"mlp.{k}_proj.weight": w[f"l0.{k}"] for k in ("gate", "up", "down")}, "")
     h = P.rms_norm(x, w["l1.n1"], 1e-5)
     q = (h @ w["l1.q_proj"].T).view(T, 4, 16)
     k = (h @ w["l1.k_proj"].T).view(T, 2, 16)
     v = (h @ w["l1.v_proj"].T).view(T, 2, 16)
-    cos, sin = P.rope_tables(16, 1e4, T, torch.float64)
     o = P.causal_gqa_attention(P.apply_rope(q, cos, sin), P.apply_rope(k, cos, sin), v, 0.25)
     x = x + o.reshape(T, 64) @ w["l1.o_proj"].T
     x = x + P.swiglu(P.rms_norm(x, w["l1.n2"], 1e-5), {f"mlp.{k}_proj.weight": w[f"l1.{k}"] for k in ("gate", "up", "down")}, "")
     return P.rms_norm(x, w["final"], 1e-5) @ w["emb"].T
 
 
+@pytest.mark.parametrize("both", [False, True])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_toy_mixer_with_state_is_registered_built_and_stepped(dtype, tmp_path):
+def test_toy_mixer_with_state_is_registered_built_and_stepped(dtype, tmp_path, both):
+    """``both``: the toy mixer also attends, so one run keeps fixed-size state and keys and values."""
     from dryft_amd import Engine
     from dryft_amd.engine.replay import Replayer
     from helpers import collect_positions, read_model_dir, trace_batches, trace_whole
     register_toy()
-    raw = {"architectures": ["ToyDecayLM"], "hidden_size": 64, "vocab_size": 97, "decay": 0.8, "intermediate_size": 72}
+    raw = {"architectures": ["ToyDecayLM"], "hidden_size": 64, "vocab_size": 97, "decay": 0.8, "intermediate_size": 72,
+           "both": both}
     # random weights written to a folder by the library, read back by name
     from dryft_amd.engine.model import DecoderModel
     from dryft_amd.weights import random_tensors, write_model_dir
     model = DecoderModel(toy_plan(ToyConfig.from_dict(raw)), torch.float32, "cpu")
-    assert any(isinstance(n, __import__("dryft_amd").cache.StateNeed) for n in model.cache_needs().values())
+    needs = model.cache_needs()
+    assert isinstance(needs[0], dict) == both
+    assert any(isinstance(n, __import__("dryft_amd").cache.StateNeed) for n in (needs[0].values() if both else needs.values()))
     path = write_model_dir(str(tmp_path / "toy"), raw, random_tensors(model.tensor_specs(), 5, torch.bfloat16, std=0.08))
     _, weights = read_model_dir(path)
     engine = Engine(path, dtype=dtype, max_batch=4, max_len=256, use_graph=False)
     assert len(engine.cache.state_groups) == 1 and len(engine.cache.kv_groups) == 1
+    assert len(engine.cache.kv_groups[0].lines) == (2 if both else 1)      # equal needs share a group, named or not
     reqs = {f"t{n}": random_tokens(n, 97, seed=n) for n in (3, 40, 90)}
     want = {rid: toy_plain(raw, weights, toks).float() for rid, toks in reqs.items()}
     limit = 1e-4 if dtype == "float32" else 3e-2

@@ -152,7 +152,9 @@ def test_fused_rows_equal_their_parts(tmp_path):
     path = make_model_dir(str(tmp_path / "m"), TINY_B, seed=3)
     model = model_for(TINY_B)
     tensors = load_tensors(path, model.tensor_specs(), torch.float32)
-    model.load(tensors)
+    handed = dict(tensors)
+    model.load(handed)
+    assert not handed, "loading hands every tensor on and keeps none in the dictionary it was given"
     att, ffn = model.blocks[1].mixer, model.blocks[1].ffn
     p = "model.layers.1."
     assert torch.equal(att.w_qkv[:256], tensors[p + "self_attn.q_proj.weight"])
