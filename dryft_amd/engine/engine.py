@@ -27,12 +27,13 @@ from ..sampling import Sampler
 from ..weights.loader import load_tensors
 from ..weights.random_init import random_tensors
 from . import generate as loop
-from .graph import DecodeGraph
+from .graph import DecodeGraph, PromptGraph
 from .model import DecoderModel
 from .step import SeqStep, Stepper
 
 DEFAULT_MAX_LEN = 8192
 SHORTEST_GRAPH_CONTEXT = 256       # captured decoding steps come in context ranges of 256, 512, 1,024, ... tokens
+PROMPT_GRAPH_ROWS = (16, 32, 64, 96, 128, 192, 256, 384, 512)   # captured prompts' steps come in these many rows
 DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32}
 
 
@@ -83,11 +84,13 @@ class Engine:
                  seed: int | None = None, norm_std: float = 0.0, dtype: str = "bfloat16", max_batch: int = 32,
                  max_len: int | None = None, max_tokens: int | None = None, use_graph: bool = True,
                  batch_buckets: Sequence[int] | None = None, max_graphs: int | None = None,
-                 device: str = "cuda:0", verbose: bool = False):
+                 prompt_graph_rows: int = 256, device: str = "cuda:0", verbose: bool = False):
         """``batch_buckets``: the batch sizes captured decoding steps are made for (default: see
         ``default_batch_buckets``; the reference's are 1, 2, 4, ... 32, engine/dryft_qwen3/config.py:169); the largest
         must be ``max_batch``. ``max_graphs``: how many captured steps are kept at most, the one used longest ago going
-        first (default: one per bucket and range of context lengths, so none ever goes)."""
+        first (default: one per bucket and range of context lengths, so none ever goes). ``prompt_graph_rows``: the
+        prompts of a batch that together have at most this many tokens run as a captured step too (0: never); such
+        steps are bound by the host's launches otherwise."""
         t0 = time.time()
         self.device = require_gpu(device)
         torch.cuda.set_device(self.device)
@@ -135,6 +138,8 @@ class Engine:
         # since only one runs at a time
         self._graphs: OrderedDict[tuple[int, int], DecodeGraph] = OrderedDict()
         self._graph_pool = None
+        self.prompt_graph_rows = int(prompt_graph_rows) if self.use_graph else 0
+        self._prompt_graphs: OrderedDict[tuple[int, int], PromptGraph] = OrderedDict()   # (sequences, rows) -> step
         self._sampler = Sampler()
         self._last_choice: torch.Tensor | None = None
         if verbose:
@@ -168,6 +173,7 @@ class Engine:
                 finally:
                     self.release(slots)
         self._graphs.clear()            # graphs captured before would keep the kernels chosen then
+        self._prompt_graphs.clear()
 
     # ------------------------------------------------------------------ StepBackend
     def acquire(self, n: int) -> list[int]:
@@ -180,8 +186,46 @@ class Engine:
         self.cache.reserve(slots, lengths)
 
     def start(self, slots: list[int], prompts: list[list[int]], step_index: int) -> list[int]:
-        logits = self.stepper.step([SeqStep(s, p, [len(p) - 1]) for s, p in zip(slots, prompts)])
-        return self._choose(logits, len(slots))
+        graph = self._prompt_graph_for(len(slots), sum(len(p) for p in prompts))
+        if graph is None:
+            logits = self.stepper.step([SeqStep(s, p, [len(p) - 1]) for s, p in zip(slots, prompts)])
+            return self._choose(logits, len(slots))
+        vocab = self.stepper.vocab
+        for p in prompts:
+            if not p:
+                raise ValueError("a sequence in a step must bring at least one token")
+            if min(p) < 0 or max(p) >= vocab:
+                raise ValueError(f"token ids must lie in [0, {vocab}); got {min(p)}..{max(p)}")
+        q_lens = [len(p) for p in prompts]
+        self.cache.begin_step(slots, q_lens)
+        logits = graph.replay(slots, prompts)
+        self.cache.end_step(slots, q_lens)
+        return self._choose(logits[:len(slots)], len(slots))
+
+    def _prompt_graph_for(self, n_seqs: int, rows: int) -> PromptGraph | None:
+        """The captured step for ``n_seqs`` sequences that start with ``rows`` tokens in all, or None where such steps
+        run launch by launch: one per number of rows in ``PROMPT_GRAPH_ROWS`` (up to ``prompt_graph_rows``; they keep
+        to the row counts at which the matrix products change kernels) and per power-of-two number of sequences (at
+        least one more than the batch has, so that the rows left over have a sequence to belong to), captured when
+        first asked for; they share the decoding steps' memory pool and their cap."""
+        n_rows = next((r for r in PROMPT_GRAPH_ROWS if r >= rows), None)
+        if n_rows is None or n_rows > self.prompt_graph_rows:
+            return None
+        seqs = 2
+        while seqs < n_seqs + 1:
+            seqs *= 2
+        key = (seqs, n_rows)
+        g = self._prompt_graphs.get(key)
+        if g is None:
+            while len(self._prompt_graphs) >= self.max_graphs:
+                self._prompt_graphs.popitem(last=False)
+            if self._graph_pool is None:
+                self._graph_pool = torch.cuda.graph_pool_handle()
+            g = PromptGraph(self.stepper, seqs, n_rows, pool=self._graph_pool)
+            g.capture()
+            self._prompt_graphs[key] = g
+        self._prompt_graphs.move_to_end(key)
+        return g
 
     def advance(self, slots: list[int], tokens: list[int], step_index: int) -> list[int]:
         if self.use_graph:
@@ -276,12 +320,16 @@ class Engine:
         self._graphs.move_to_end(key)
         return g
 
-    def warm(self, batch_sizes: Sequence[int] | None = None, contexts: Sequence[int] | None = None) -> int:
+    def warm(self, batch_sizes: Sequence[int] | None = None, contexts: Sequence[int] | None = None,
+             prompts: Sequence[tuple[int, int]] = ()) -> int:
         """Captures decoding steps before the first request needs them, as the reference does when it is built
         (engine/dryft_qwen3/graphs.py:39-59): for the buckets of ``batch_sizes`` (default: every bucket) and the ranges
-        of the context lengths ``contexts`` (default: every range). Returns how many captured steps are held then."""
+        of the context lengths ``contexts`` (default: every range); and the prompts' steps for ``prompts``, pairs of
+        (sequences, tokens in all). Returns how many captured decoding steps are held then."""
         if not self.use_graph:
             return 0
+        for n_seqs, rows in prompts:
+            self._prompt_graph_for(int(n_seqs), int(rows))
         buckets = sorted(set(pick_bucket(self.batch_buckets, int(b)) for b in batch_sizes)) \
             if batch_sizes is not None else list(self.batch_buckets)
         ranges = self.context_ranges()

@@ -145,7 +145,9 @@ class Stepper:
             return torch.empty((0, self.vocab), dtype=torch.float32, device=self.device)
         return self.model.logits(hidden)
 
-    def run(self, buf: BatchBuffers, ctx: StepContext) -> torch.Tensor:
-        """The device work of a step whose facts already sit in ``buf`` (what a captured graph holds)."""
+    def run(self, buf: BatchBuffers, ctx: StepContext, rows: torch.Tensor | None = None) -> torch.Tensor:
+        """The device work of a step whose facts already sit in ``buf`` (what a captured graph holds); the hidden
+        states after the final norm, of every row or of ``rows``."""
+        ctx.forget_derived()
         derive_rows(self.cache, buf, ctx)
-        return self.model.forward(buf.tokens[:ctx.n_rows], ctx, self.cache)
+        return self.model.forward(buf.tokens[:ctx.n_rows], ctx, self.cache, rows)

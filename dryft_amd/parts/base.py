@@ -76,6 +76,11 @@ class StepContext:
             found = self._tiles[rows_per_tile] = (tile_cu, bound)
         return found
 
+    def forget_derived(self) -> None:
+        """For a context that is used for more than one step: what ``tiles()`` has computed belongs to the step
+        before."""
+        self._tiles.clear()
+
     def some_sit_out(self) -> bool:
         """May the step hold sequences that sit out (slot -1)? Without the host's view: yes."""
         return self.host is None or any(s < 0 for s in self.host.slots)

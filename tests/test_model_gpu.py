@@ -545,11 +545,14 @@ def test_batch_buckets_bound_the_captured_steps(cases, dtype):
     prompts = [random_tokens(int(rng.integers(1, 30)), case.vocab, seed=600 + i) for i in range(40)]
     how = {n: dict(temperature=0.8, sample_seed=n) if n % 3 == 0 else {} for n in range(1, 41)}
     want = {n: exact.generate_all(prompts[:n], 4, **how[n]) for n in range(1, 41)}
-    bucketed.generate_all(prompts, 2)                          # what a step itself holds on to (staging) exists now
-    torch.cuda.synchronize()
-    held = torch.cuda.memory_allocated()
     for n in range(1, 41):
         assert bucketed.generate_all(prompts[:n], 4, **how[n]) == want[n], f"batch of {n}"
+    # again: the prompts' captured steps exist now too, and nothing more may be captured or kept
+    torch.cuda.synchronize()
+    held, prompt_steps = torch.cuda.memory_allocated(), len(bucketed._prompt_graphs)
+    for n in range(1, 41):
+        assert bucketed.generate_all(prompts[:n], 4, **how[n]) == want[n], f"batch of {n}, second time"
+    assert len(bucketed._prompt_graphs) == prompt_steps
     assert len(bucketed._graphs) == len(buckets), "a step was captured although every bucket was warm"
     torch.cuda.synchronize()
     assert torch.cuda.memory_allocated() == held, "generation kept device memory although every bucket was warm"
@@ -563,6 +566,47 @@ def test_batch_buckets_bound_the_captured_steps(cases, dtype):
     with pytest.raises(ValueError, match="max_graphs"):
         capped.warm()
     assert bucketed.cache.slots.free_count == exact.cache.slots.free_count == 40
+
+
+@pytest.mark.parametrize("name", ["B", "C_sharp", "A_sharp"])
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_short_prompts_start_through_a_captured_step(cases, dtype, name):
+    """Batches whose prompts have at most 256 tokens in all start in a captured step, filled up with sequences that
+    sit out: the logits at each prompt's end against the plain implementation, on slots that are used again, batch
+    shapes taking turns so that every captured step is replayed several times with other work in between; then
+    generation, whose tokens are those of an engine that starts launch by launch."""
+    case = cases[name]
+    engine = case.engine(dtype, max_batch=9, max_len=512, use_graph=True)
+    eager = case.engine(dtype, max_batch=9, max_len=512, use_graph=True, prompt_graph_rows=0)
+    shapes = [[1], [5, 9, 17], [64], [70, 1, 33], [129, 65, 9, 17, 5, 1, 1, 1, 1], [200, 33], [17], [131, 70, 33, 17, 5],
+              [9, 5], [200, 33, 17, 5, 1], [128, 128], [65, 17, 9]]
+    assert engine._prompt_graph_for(3, 300) is None and eager._prompt_graph_for(1, 5) is None
+    for turn in range(3):
+        for lengths in shapes:
+            names = [f"r{n}" for n in lengths]
+            prompts = [case.requests[r] for r in names]
+            graph = engine._prompt_graph_for(len(prompts), sum(lengths))
+            assert graph.n_seqs > len(prompts) and sum(lengths) <= graph.n_rows <= max(32, 1.6 * sum(lengths))
+            slots = engine.acquire(len(prompts))
+            try:
+                engine.cache.begin_step(slots, lengths)
+                logits = graph.replay(slots, prompts)[:len(prompts)].float().cpu()
+                engine.cache.end_step(slots, lengths)
+                assert [int(engine.cache.lengths_host()[s]) for s in slots] == lengths
+                assert engine.cache.lengths_dev[slots].tolist() == lengths
+            finally:
+                engine.release(slots)
+            got = {(r, n - 1): logits[i] for i, (r, n) in enumerate(zip(names, lengths)) if names.index(r) == i}
+            check_against_plain(case, got, dtype, f"captured prompts' step {lengths}")
+    assert len(engine._prompt_graphs) <= 10
+    for lengths in shapes + [[200, 131]]:                               # the last one has too many tokens: launch by launch
+        prompts = [case.requests[f"r{n}"] for n in lengths]
+        kw = dict(temperature=0.7, sample_seed=len(lengths)) if len(lengths) % 2 else {}
+        ours = engine.generate_all(prompts, 5, **kw)
+        assert ours == eager.generate_all(prompts, 5, **kw), lengths
+    check_generation(case, [case.requests["r70"], case.requests["r9"]],
+                     list(engine.generate([case.requests["r70"], case.requests["r9"]], 6)), 6, dtype)
+    assert engine.cache.slots.free_count == 9
 
 
 @pytest.mark.parametrize("name,n_seqs", [("A_sharp", 70), ("B", 130), ("C_sharp", 200)])
