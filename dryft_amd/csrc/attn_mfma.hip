@@ -767,7 +767,22 @@ struct HeadRegs {
   float x[4], wt[4], cs[4], sn[4];
 };
 
-__device__ __forceinline__ void head_load(HeadRegs& r, const bf16_t* __restrict__ src, const void* __restrict__ w,
+// Where a row of the fused projection's output lies: as bfloat16 values, or as `parts` float partial sums over K,
+// `part_stride` values apart, which are added up in order here and rounded as the product's own epilogue would.
+struct ProjectedRow {
+  const bf16_t* values;
+  const float* sums;
+  int parts;
+  int64_t part_stride;
+  __device__ __forceinline__ float at(int64_t i) const {
+    if (sums == nullptr) return bf16_to_float(values[i]);
+    float v = sums[i];
+    for (int s = 1; s < parts; ++s) v += sums[s * part_stride + i];
+    return rounded_as<bf16_t>(v);
+  }
+};
+
+__device__ __forceinline__ void head_load(HeadRegs& r, const ProjectedRow& src, int64_t first, const void* __restrict__ w,
                                           int w_f32, int has_norm, const bf16_t* __restrict__ cos_t,
                                           const bf16_t* __restrict__ sin_t, int rot, int pos, int head_dim) {
   const int lane = threadIdx.x % WAVE;
@@ -776,7 +791,7 @@ __device__ __forceinline__ void head_load(HeadRegs& r, const bf16_t* __restrict_
   for (int u = 0; u < 4; ++u) {
     const int i = lane + WAVE * u;
     const bool in = i < head_dim;
-    r.x[u] = in ? bf16_to_float(src[i]) : 0.f;
+    r.x[u] = in ? src.at(first + i) : 0.f;
     r.wt[u] = (in && has_norm) ? load_vector(w, i, w_f32) : 1.f;
     const int j = i < half ? i : i - half;
     r.cs[u] = (in && i < rot) ? bf16_to_float(cos_t[(int64_t)pos * half + j]) : 1.f;
@@ -824,6 +839,8 @@ __device__ __forceinline__ void head_finish(HeadRegs& r, int has_norm, float eps
 struct FusedQKV {
   const bf16_t* qkv;       // [rows, stride]: q heads, k heads, v heads of each row; null: q is given ready
   int64_t stride;
+  int parts;               // > 0: qkv points to float partial sums [parts, rows, stride] instead
+  int64_t part_stride;     // values from one partial sum to the next
   const void* q_w;
   const void* k_w;
   int w_f32, has_norm;
@@ -887,11 +904,15 @@ __global__ __launch_bounds__(64 * SPLIT_WAVES, 2) void attn_split_kernel(
     // them into its operands itself, so nothing has to wait for memory. The loads of a wave's first head are
     // issued before those of its first page of keys and waited for first, so the two latencies overlap.
     float* tmp = &merge_o[wave][0][0];                          // free until the merge
-    const bf16_t* src_row = fused.qkv + row * fused.stride;
+    ProjectedRow src_row;
+    src_row.values = fused.parts > 0 ? nullptr : fused.qkv + row * fused.stride;
+    src_row.sums = fused.parts > 0 ? (const float*)fused.qkv + row * fused.stride : nullptr;
+    src_row.parts = fused.parts;
+    src_row.part_stride = fused.part_stride;
     HeadRegs first;
     const bool has_first = slot >= 0 && wave < group;
     if (has_first)
-      head_load(first, src_row + (int64_t)(kvh * group + wave) * head_dim, fused.q_w, fused.w_f32, fused.has_norm,
+      head_load(first, src_row, (int64_t)(kvh * group + wave) * head_dim, fused.q_w, fused.w_f32, fused.has_norm,
                 fused.cos_t, fused.sin_t, fused.rot, pos, head_dim);
     if (page >= 0) load_page_k<KB, FULL>(kf, k_pages + ((int64_t)page * n_kv + kvh) * page_elems, head_dim);
     if (has_first)
@@ -899,7 +920,7 @@ __global__ __launch_bounds__(64 * SPLIT_WAVES, 2) void attn_split_kernel(
     if (slot >= 0) {
       for (int r = wave + SPLIT_WAVES; r < group; r += SPLIT_WAVES) {
         HeadRegs more;
-        head_load(more, src_row + (int64_t)(kvh * group + r) * head_dim, fused.q_w, fused.w_f32, fused.has_norm,
+        head_load(more, src_row, (int64_t)(kvh * group + r) * head_dim, fused.q_w, fused.w_f32, fused.has_norm,
                   fused.cos_t, fused.sin_t, fused.rot, pos, head_dim);
         head_finish(more, fused.has_norm, fused.eps, fused.rot, head_dim, tmp, &q_lds[r][0], nullptr);
       }
@@ -910,15 +931,15 @@ __global__ __launch_bounds__(64 * SPLIT_WAVES, 2) void attn_split_kernel(
         const bool store = fused.write_kv && page_last >= 0;
         if (wave == SPLIT_WAVES - 1) {
           HeadRegs key;
-          head_load(key, src_row + (int64_t)(n_heads + kvh) * head_dim, fused.k_w, fused.w_f32, fused.has_norm,
+          head_load(key, src_row, (int64_t)(n_heads + kvh) * head_dim, fused.k_w, fused.w_f32, fused.has_norm,
                     fused.cos_t, fused.sin_t, fused.rot, pos, head_dim);
           head_finish(key, fused.has_norm, fused.eps, fused.rot, head_dim, tmp, &kv_new[0][0],
                       store ? k_pages_w + base + (int64_t)at * head_dim : nullptr);
         }
         if (wave == SPLIT_WAVES - 2) {
-          const bf16_t* vs = src_row + (int64_t)(n_heads + n_kv + kvh) * head_dim;
+          const int64_t vs = (int64_t)(n_heads + n_kv + kvh) * head_dim;
           for (int i = lane; i < head_dim; i += WAVE) {
-            const bf16_t v = vs[i];
+            const bf16_t v = float_to_bf16(src_row.at(vs + i));
             kv_new[1][i] = v;
             if (store) v_pages_w[base + (int64_t)i * PAGE_TOKENS + value_column(at)] = v;
           }
@@ -1223,17 +1244,20 @@ DRYFT_API int dryft_attn_split_bf16(const void* q, const void* k_pages, const vo
 }
 
 // The same with the work of the norm/rotation/append kernel folded in: `qkv` is the fused projection's output
-// for one row per sequence. Takes kv groups of at most 16 query heads.
-DRYFT_API int dryft_attn_decode_fused_bf16(const void* qkv, int64_t qkv_stride, const void* q_w, const void* k_w,
+// for one row per sequence, as bfloat16 [rows, qkv_stride] (qkv_parts 0) or as qkv_parts float partial sums over K,
+// [qkv_parts, rows, qkv_stride] with qkv_part_stride values from one to the next, which the kernel adds up in order
+// and rounds on its way in. Takes kv groups of at most 16 query heads.
+DRYFT_API int dryft_attn_decode_fused_bf16(const void* qkv, int64_t qkv_stride, int qkv_parts, int64_t qkv_part_stride,
+                                           const void* q_w, const void* k_w,
                                            int w_f32, int has_norm, float eps, const void* cos_t, const void* sin_t,
                                            int rot, int write_kv, void* k_pages, void* v_pages, const int* page_table,
                                            int max_pages, const int* seq_slot, const int* cu_rows, const int* kv_len,
                                            int n_seqs, float* part_o, float* part_ml, int n_splits, void* out,
                                            int n_heads, int n_kv, int head_dim, float scale, int window,
                                            hipStream_t stream) {
-  if (qkv == nullptr) return -1;
-  FusedQKV fused = {(const bf16_t*)qkv, qkv_stride, q_w, k_w, w_f32, has_norm, eps, (const bf16_t*)cos_t,
-                    (const bf16_t*)sin_t, rot, write_kv};
+  if (qkv == nullptr || qkv_parts < 0) return -1;
+  FusedQKV fused = {(const bf16_t*)qkv, qkv_stride, qkv_parts, qkv_part_stride, q_w, k_w, w_f32, has_norm, eps,
+                    (const bf16_t*)cos_t, (const bf16_t*)sin_t, rot, write_kv};
   return launch_split(nullptr, k_pages, v_pages, page_table, max_pages, seq_slot, cu_rows, kv_len, n_seqs, part_o,
                       part_ml, n_splits, out, n_heads, n_kv, head_dim, scale, window, fused, stream);
 }

@@ -33,7 +33,7 @@ _SIGNATURES = {
                                                        _I, _P, _I, _I, _I, _F, _I, _I, _P],
                   "dryft_attn_split_bf16": [_P, _P, _P, _P, _I, _P, _P, _P, _I, _P, _P, _I, _P, _I, _I, _I, _F, _I,
                                             _P],
-                  "dryft_attn_decode_fused_bf16": [_P, _L, _P, _P, _I, _I, _F, _P, _P, _I, _I, _P, _P, _P, _I, _P, _P,
+                  "dryft_attn_decode_fused_bf16": [_P, _L, _I, _L, _P, _P, _I, _I, _F, _P, _P, _I, _I, _P, _P, _P, _I, _P, _P,
                                                    _P, _I, _P, _P, _I, _P, _I, _I, _I, _F, _I, _P]},
     "gemm": {"dryft_gemm_tiled": [_P, _L, _P, _P, _I, _I, _I, _I, _I, _P],
              "dryft_gemm_stream_bf16": [_P, _L, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
@@ -400,17 +400,27 @@ def attn_split_bf16(q, k_pages, v_pages, page_table, seq_slot, cu_rows, kv_len, 
 
 def attn_decode_fused_bf16(qkv, q_weight, k_weight, eps: float, cos, sin, rot: int, write_kv: bool, k_pages, v_pages,
                            page_table, seq_slot, cu_rows, kv_len, n_seqs: int, part_o, part_ml, n_splits: int, out,
-                           n_heads: int, n_kv: int, head_dim: int, scale: float, window: int) -> None:
+                           n_heads: int, n_kv: int, head_dim: int, scale: float, window: int, qkv_parts: int = 0) -> None:
     """One row per sequence: q/k norm, rotation, append to the cache and attention in one kernel (plus the combine).
 
     ``qkv`` is the fused projection's output ``[n_seqs rows, (heads + 2 kv heads) * head_dim]``; row ``i`` belongs to
-    sequence ``i`` (``cu_rows[i] == i``).
+    sequence ``i`` (``cu_rows[i] == i``). It may also be that product left as float32 partial sums over K,
+    ``[parts, rows, width]`` (``qkv_parts`` of them): the kernel adds them up in order and rounds the sum to bfloat16
+    as the product would have.
     """
-    _gpu(qkv, "qkv", torch.bfloat16)
     _gpu(out, "out", torch.bfloat16)
     need_cols = (n_heads + 2 * n_kv) * head_dim
-    if not (qkv.dim() == 2 and qkv.stride(1) == 1 and qkv.shape[1] >= need_cols and qkv.shape[0] >= n_seqs):
-        raise KernelError(f"attn_decode_fused: qkv must be [rows >= {n_seqs}, >= {need_cols}]")
+    if qkv_parts:
+        _gpu(qkv, "qkv", torch.float32)
+        if not (qkv.dim() == 3 and qkv.is_contiguous() and qkv.shape[0] >= qkv_parts and qkv.shape[1] >= n_seqs
+                and qkv.shape[2] >= need_cols):
+            raise KernelError(f"attn_decode_fused: partial sums must be [>= {qkv_parts}, rows >= {n_seqs}, >= {need_cols}]")
+        row_stride, part_stride = qkv.stride(1), qkv.stride(0)
+    else:
+        _gpu(qkv, "qkv", torch.bfloat16)
+        if not (qkv.dim() == 2 and qkv.stride(1) == 1 and qkv.shape[1] >= need_cols and qkv.shape[0] >= n_seqs):
+            raise KernelError(f"attn_decode_fused: qkv must be [rows >= {n_seqs}, >= {need_cols}]")
+        row_stride, part_stride = qkv.stride(0), 0
     if not (out.is_contiguous() and out.numel() >= n_seqs * n_heads * head_dim):
         raise KernelError("attn_decode_fused: out too small")
     if not (n_heads // n_kv <= 16):
@@ -443,7 +453,8 @@ def attn_decode_fused_bf16(qkv, q_weight, k_weight, eps: float, cos, sin, rot: i
     if part_o.numel() < entries * head_dim or part_ml.numel() < entries * 2:
         raise KernelError("attn_decode_fused: partial buffers too small")
     _check(_fn("attn_mfma", "dryft_attn_decode_fused_bf16")(
-        _ptr(qkv), qkv.stride(0), _ptr(q_weight), _ptr(k_weight), w_f32, int(has_norm), float(eps), _ptr(cos), _ptr(sin),
+        _ptr(qkv), row_stride, int(qkv_parts), part_stride, _ptr(q_weight), _ptr(k_weight), w_f32, int(has_norm),
+        float(eps), _ptr(cos), _ptr(sin),
         int(rot), int(write_kv), _ptr(k_pages), _ptr(v_pages), _ptr(page_table), page_table.shape[1], _ptr(seq_slot),
         _ptr(cu_rows), _ptr(kv_len), n_seqs, _ptr(part_o), _ptr(part_ml), n_splits, _ptr(out), n_heads, n_kv, head_dim,
         float(scale), int(window), _stream()), "attn_decode_fused_bf16")

@@ -24,11 +24,12 @@ from ..csrc import ops
 from ..limits import MATRIX_CORE_HEAD_STEP, MAX_HEAD_DIM
 from ..weights.spec import VECTOR
 from . import register_part
-from .base import Mixer, StepContext, matrix
+from .base import Mixer, Partials, StepContext, matrix
 from .linear import linear
 
 _RESIDENT_WORKGROUPS = 512     # of the split kernel: two per compute unit (its registers allow no more)
 _MAX_SPLITS = 32
+_QKV_PARTIAL_ROWS = 32         # decoding steps of up to so many rows take the projection as partial sums over K
 
 
 class GQAAttention(Mixer):
@@ -74,7 +75,15 @@ class GQAAttention(Mixer):
 
     def forward(self, h: torch.Tensor, ctx: StepContext, line: KVLine, writes_cache: bool):
         rows = h.shape[0]
-        qkv = linear(h, self.w_qkv)
+        # bfloat16 on the matrix cores where they take the head size; float32 and the other head sizes on the plain kernel
+        matrix_cores = h.dtype == torch.bfloat16 and self.head_dim % MATRIX_CORE_HEAD_STEP == 0
+        decoding = matrix_cores and ctx.max_q_len == 1
+        fused_decoding = decoding and self.n_heads // self.n_kv <= 16
+        # The kernel that norms, rotates, appends and attends in one adds up partial sums of the projection on its way
+        # in, so K may be split over workgroups. Measured on Qwen3-4B's sizes, a decoding step with the split against
+        # without: 2.980 against 3.008 ms at 8 sequences, 4.63 against 4.74 at 32, and level with the vendor library's
+        # product at 64 (6.88 against 6.86), where it therefore stays.
+        qkv = linear(h, self.w_qkv, allow_partials=fused_decoding, partial_rows=_QKV_PARTIAL_ROWS)
         cos = sin = None
         if self.positions:
             table = ctx.positions[self.positions]
@@ -86,19 +95,17 @@ class GQAAttention(Mixer):
         # so for those the rows are cleared beforehand wherever the step may hold such sequences.
         make = torch.zeros if ctx.max_q_len > 1 and ctx.some_sit_out() else torch.empty
         out = make((rows, self.n_heads, self.head_dim), dtype=h.dtype, device=h.device)
-        # bfloat16 on the matrix cores where they take the head size; float32 and the other head sizes on the plain kernel
-        matrix_cores = h.dtype == torch.bfloat16 and self.head_dim % MATRIX_CORE_HEAD_STEP == 0
-        decoding = matrix_cores and ctx.max_q_len == 1
         if decoding:
             splits = self.decode_splits(ctx.n_seqs, ctx.max_kv_len)
             part_o = torch.empty((ctx.n_seqs, self.n_heads, splits, self.head_dim), dtype=torch.float32, device=h.device)
             part_ml = torch.empty((ctx.n_seqs, self.n_heads, splits, 2), dtype=torch.float32, device=h.device)
-        if decoding and self.n_heads // self.n_kv <= 16:
+        if fused_decoding:
             # one token per sequence: norm, rotation, append and attention in one kernel
-            ops.attn_decode_fused_bf16(qkv, self.q_norm, self.k_norm, self.qk_norm_eps or 0.0, cos, sin, self.rotary_dim,
+            parts = qkv.count if isinstance(qkv, Partials) else 0
+            ops.attn_decode_fused_bf16(qkv.data if parts else qkv, self.q_norm, self.k_norm, self.qk_norm_eps or 0.0, cos, sin, self.rotary_dim,
                                        writes_cache, line.k, line.v, line.page_table, ctx.seq_slot, ctx.cu_rows,
                                        ctx.kv_len, ctx.n_seqs, part_o, part_ml, splits, out, self.n_heads, self.n_kv,
-                                       self.head_dim, self.scale, window)
+                                       self.head_dim, self.scale, window, qkv_parts=parts)
             return linear(out.view(rows, self.q_dim), self.w_o, allow_partials=True)
         if matrix_cores and not decoding and cos is not None and \
                 ops.attn_causal_takes_projection(self.head_dim, self.rotary_dim):

@@ -105,9 +105,13 @@ def within_direct_reach(x: torch.Tensor, w: torch.Tensor) -> bool:
         x.shape[0] * x.stride(0) * x.element_size() < ops.DIRECT_REACH
 
 
-def linear(x: torch.Tensor, w: torch.Tensor, *, out_dtype: torch.dtype | None = None, allow_partials: bool = False):
-    """Returns ``[rows, out]`` in ``out_dtype`` (default: the dtype of ``x``), or ``Partials``."""
+def linear(x: torch.Tensor, w: torch.Tensor, *, out_dtype: torch.dtype | None = None, allow_partials: bool = False,
+           partial_rows: int | None = None):
+    """Returns ``[rows, out]`` in ``out_dtype`` (default: the dtype of ``x``), or, where the caller allows it and a
+    split of K pays, ``Partials`` (``partial_rows``: only for steps of at most so many rows)."""
     m, k = x.shape
+    if partial_rows is not None and m > partial_rows:
+        allow_partials = False
     n = w.shape[0]
     out_dtype = out_dtype or x.dtype
     if x.dtype == torch.float32:

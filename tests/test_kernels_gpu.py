@@ -487,6 +487,18 @@ def test_attn_decode_fused_equals_the_two_kernels(n_heads, n_kv, D, splits, wind
     o.attn_decode_fused_bf16(qkv, wq, wk, 1e-6, cos, sin, D, False, k3, v3, table, seq_slot, cu, kv_len, B, po, pml,
                              splits, out3, n_heads, n_kv, D, scale, window)
     assert torch.equal(k3, k1) and torch.equal(v3, v1) and torch.equal(out3, out2)
+    # the projection handed over as float partial sums over K: the kernel adds them up in order and rounds, so it
+    # gives what it gives for the rounded sum, bit for bit
+    parts = torch.randn(3, B, qkv.shape[1], device=DEV)
+    summed = ((parts[0] + parts[1]) + parts[2]).to(torch.bfloat16)
+    k4, v4, k5, v5 = k0.clone(), v0.clone(), k0.clone(), v0.clone()
+    out4, out5 = torch.zeros_like(out2), torch.zeros_like(out2)
+    o.attn_decode_fused_bf16(summed, wq, wk, 1e-6, cos, sin, D, True, k4, v4, table, seq_slot, cu, kv_len, B, po, pml,
+                             splits, out4, n_heads, n_kv, D, scale, window)
+    o.attn_decode_fused_bf16(parts, wq, wk, 1e-6, cos, sin, D, True, k5, v5, table, seq_slot, cu, kv_len, B, po, pml,
+                             splits, out5, n_heads, n_kv, D, scale, window, qkv_parts=3)
+    assert torch.equal(k4, k5) and torch.equal(v4, v5) and torch.equal(out4, out5), "partial sums of the projection"
+    assert not torch.equal(out4, out2)
 
 
 @pytest.mark.parametrize("heads", [(8, 2), (16, 2), (10, 2), (4, 2), (3, 3)])       # 4, 8, 5, 2 and 1 to a kv head
