@@ -1,6 +1,7 @@
 """Decode and prefill throughput of the Qwen3 engine on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--preset qwen3-4b] [--batch 8] [--layers L]
+                    [--prompt-len 2048] [--slot-len 4096]
 
 The workload is the one named for the reference's headline metric: Qwen3-4B layer sizes with
 random weights in bfloat16, prompts of 2,048 uniform random token ids in 4,096-token cache
@@ -8,7 +9,9 @@ slots, greedy decoding. A step is one decode step of the whole batch through the
 machinery (graph replay, token choice, token hand-back). One JSON line is printed:
 decoded tokens per second at the main batch size, the prefill rate of one 2,048-token prompt
 with its fraction of the bf16 matrix-core peak, the decode step's fraction of the HBM
-roofline, and decode rates at batch 1 and 64. Timing protocol after the reference's harness
+roofline (with the bytes, the time and the peak it is made of), and as further points the
+decode rates at batch 1 and 64 and the rate of eight 2,048-token prompts prefilled in one
+step. Timing protocol after the reference's harness
 (agent/bench.py:96-126): untimed warm-up, synchronise on both sides of the timed region.
 """
 
@@ -39,6 +42,7 @@ def prefill_flops(engine, tokens: int) -> float:
 
 
 def main() -> int:
+    global PROMPT, SLOT
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=128)
@@ -54,7 +58,11 @@ def main() -> int:
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-tune", action="store_true",
                     help="keep the vendor library's default kernels for the prompt's matrix products")
+    ap.add_argument("--prompt-len", type=int, default=PROMPT, help="tokens of every prompt (the context decoding starts at)")
+    ap.add_argument("--slot-len", type=int, default=None, help="tokens a cache slot holds (default: twice the prompt)")
     args = ap.parse_args()
+    PROMPT = args.prompt_len
+    SLOT = args.slot_len or max(SLOT, 2 * PROMPT)
     if args.gpus != 1:
         print(f"bench.py measures one GPU only (asked for {args.gpus}); this library has no multi-GPU path")
         return 2
@@ -72,8 +80,10 @@ def main() -> int:
     if args.layers:
         raw["num_hidden_layers"] = args.layers
     max_batch = args.batch if args.no_points else max(args.batch, 64)
+    # the cache holds what the largest batch needs at the end of its run, no more (long contexts at small batches)
     engine = Engine(config=raw, seed=args.seed, dtype=args.dtype, max_batch=max_batch, max_len=SLOT,
-                    use_graph=not args.no_graph, verbose=True)
+                    max_tokens=max_batch * (PROMPT + 2 * (args.steps + args.warmup) + 192), use_graph=not args.no_graph,
+                    verbose=True)
     cfg = engine.config
     vocab = engine.model.plan.vocab_size
     if not args.no_tune and args.dtype == "bfloat16":
@@ -108,11 +118,12 @@ def main() -> int:
         context = PROMPT + warmup + (steps + 1) / 2.0
         return batch * steps / dt, dt / steps * 1e3, context
 
-    def prefill_rate(repeats: int = 3):
+    def prefill_rate(n_prompts: int = 1, repeats: int = 3):
+        """(tokens/s, ms) of `n_prompts` prompts prefilled in one step: the best of `repeats` runs."""
         best = None
         for _ in range(repeats + 1):                       # the first run warms libraries up
-            slots = engine.acquire(1)
-            p = prompts(1)
+            slots = engine.acquire(n_prompts)
+            p = prompts(n_prompts)
             sync()
             t0 = time.perf_counter()
             engine.start(slots, p, 0)
@@ -120,17 +131,18 @@ def main() -> int:
             dt = time.perf_counter() - t0
             engine.release(slots)
             best = dt if best is None else min(best, dt)
-        return PROMPT / best, best * 1e3
+        return n_prompts * PROMPT / best, best * 1e3
 
-    tok_s = ms_step = achieved = pf_tok_s = pf_ms = pf_frac = 0.0
+    tok_s = ms_step = achieved = need = pf_tok_s = pf_ms = pf_frac = pf_flops = 0.0
+    peak = PEAK_FLOPS["bf16" if args.dtype == "bfloat16" else "fp32"]
     if args.phase in ("all", "decode"):
         tok_s, ms_step, context = decode_rate(args.batch, args.steps, args.warmup)
         need = decode_bytes(engine, args.batch, context)
         achieved = need / (ms_step * 1e-3) / 1e9
     if args.phase in ("all", "prefill"):
         pf_tok_s, pf_ms = prefill_rate()
-        peak = PEAK_FLOPS["bf16" if args.dtype == "bfloat16" else "fp32"]
-        pf_frac = prefill_flops(engine, PROMPT) / (pf_ms * 1e-3) / peak
+        pf_flops = prefill_flops(engine, PROMPT)
+        pf_frac = pf_flops / (pf_ms * 1e-3) / peak
     points, points_frac = {}, {}
     if not args.no_points and args.phase == "all":
         for b in (1, 64):
@@ -138,8 +150,13 @@ def main() -> int:
             points[f"decode_b{b}"] = round(rate, 1)
             # the same roofline as the main batch: bytes the step has to read / its time / the HBM peak
             points_frac[f"decode_b{b}"] = round(decode_bytes(engine, b, ctx) / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
+        # eight prompts in one step: tokens a second, and the step's flops / time / peak
+        if 8 * (PROMPT + 64) <= engine.max_tokens:
+            rate, ms = prefill_rate(8, repeats=2)
+            points["prefill_b8"] = round(rate, 1)
+            points_frac["prefill_b8"] = round(engine.model.step_flops([(0, PROMPT)] * 8, 8) / (ms * 1e-3) / peak, 4)
     line = {
-        "metric": f"decode tok/s ({args.preset} layer sizes, 2,048-token prompts, 4,096-token slots)",
+        "metric": f"decode tok/s ({args.preset} layer sizes, {PROMPT:,}-token prompts, {SLOT:,}-token slots)",
         "value": round(tok_s, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic (random weights, uniform random token ids)",
@@ -150,9 +167,11 @@ def main() -> int:
             "library_tuned": not args.no_tune,
             **{k: v for k, v in asdict(cfg).items() if isinstance(v, (bool, int, float, str))},
         },
-        "prefill": {"value": round(pf_tok_s, 1), "tokens": PROMPT, "ms": round(pf_ms, 3), "frac": round(pf_frac, 4)},
+        "prefill": {"value": round(pf_tok_s, 1), "tokens": PROMPT, "ms": round(pf_ms, 3), "frac": round(pf_frac, 4),
+                    "tflop": round(pf_flops / 1e12, 3), "peak_tflops": peak / 1e12},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4)},
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "gbytes": round(need / 1e9, 4),
+                     "ms": round(ms_step, 4)},
         "points": points,
         "points_frac": points_frac,
     }

@@ -212,6 +212,55 @@ def cmd_profile(args) -> int:
     return 0
 
 
+def cmd_kernel_table(args) -> int:
+    """Reduces a ``rocprofv3 --kernel-trace`` recording of this library at work (its ``*_results.db``) to one table:
+    the kernels of a step, how often each runs in it and for how long. Steps are told apart by the kernel that
+    opens every step (``prepare_batch``); ``--kind decode`` keeps the steps that hold no prompt attention,
+    ``--kind prompt`` those that do, and the last ``--steps`` of them are averaged."""
+    import re
+    import sqlite3
+    import statistics
+
+    cur = sqlite3.connect(args.database).cursor()
+    tables = [r[0] for r in cur.execute("select name from sqlite_master where type='table'")]
+    dispatches = next(t for t in tables if t.startswith("rocpd_kernel_dispatch"))
+    symbols = next(t for t in tables if t.startswith("rocpd_info_kernel_symbol"))
+    launches = cur.execute(f"select d.start, d.end, s.kernel_name from {dispatches} d join {symbols} s "
+                           f"on d.kernel_id = s.id order by d.start").fetchall()
+    opens = [i for i, (_, _, name) in enumerate(launches) if "prepare_batch" in name]
+    steps = []
+    for a, b in zip(opens[:-1], opens[1:]):
+        step = launches[a:b]
+        has_prompt = any("attn_causal" in name for _, _, name in step)
+        if len(step) >= args.min_kernels and has_prompt == (args.kind == "prompt"):
+            steps.append(step)
+    steps = steps[-args.steps:]
+    if not steps:
+        print("no step of that kind in the recording", file=sys.stderr)
+        return 1
+
+    def plain_name(name: str) -> str:
+        name = re.sub(r"\.kd$", "", re.sub(r"^_Z\d+", "", name))
+        m = re.match(r"([a-z_0-9]+kernel)(I.*?E)?Ev", name)
+        return (m.group(1) + (" <" + m.group(2)[1:-1] + ">" if m.group(2) else "")) if m else name[:64]
+
+    per_kernel: dict[str, list[float]] = {}
+    for step in steps:
+        for start, end, name in step:
+            entry = per_kernel.setdefault(plain_name(name), [0, 0.0])
+            entry[0] += 1
+            entry[1] += (end - start) / 1e3
+    n = len(steps)
+    busy = statistics.median(sum(e - s for s, e, _ in step) / 1e3 for step in steps)
+    span = statistics.median((step[-1][1] - step[0][0]) / 1e3 for step in steps)
+    print(f"{args.kind} steps averaged: {n}; kernels in a step: {len(steps[-1])}; "
+          f"median time inside kernels {busy:.0f} us, median first start to last end {span:.0f} us")
+    print(f"{'kernel':70s} {'in a step':>9s} {'us a step':>10s} {'us each':>8s} {'of the step':>11s}")
+    for name, (count, us) in sorted(per_kernel.items(), key=lambda kv: -kv[1][1]):
+        print(f"{name:70s} {count / n:9.1f} {us / n:10.1f} {us / count:8.2f} {us / n / busy:11.1%}")
+    return 0
+
+
 def cmd_attention(args) -> int:
     """Times the bfloat16 prompt-attention kernel alone: for each ``BxL`` (B sequences of L new positions each, nothing
     cached before them) and each way of running it (``ops.attn_causal_bf16``'s ``mode``), the best of four timings
@@ -306,6 +355,13 @@ def main(argv=None) -> int:
     pr.add_argument("--rows", type=int, default=20, help="kernels to list")
     pr.add_argument("--seed", type=int, default=0)
     pr.set_defaults(fn=cmd_profile)
+
+    kt = sub.add_parser("kernel-table", help="per-step kernel table from a rocprofv3 --kernel-trace recording (no GPU)")
+    kt.add_argument("database", help="the recording's *_results.db")
+    kt.add_argument("--kind", choices=["decode", "prompt"], default="decode")
+    kt.add_argument("--steps", type=int, default=32, help="average over the last so many steps of that kind")
+    kt.add_argument("--min-kernels", type=int, default=50, help="ignore stretches with fewer launches (warm-up odds and ends)")
+    kt.set_defaults(fn=cmd_kernel_table)
 
     at = sub.add_parser("attention", help="time the prompt-attention kernel alone, in each way of running it")
     at.add_argument("--shapes", default="1x2048,1x4096,8x2048", help="BxL,...: B sequences of L positions each")
