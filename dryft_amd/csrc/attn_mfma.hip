@@ -894,6 +894,7 @@ __global__ __launch_bounds__(64 * SPLIT_WAVES, 2) void attn_split_kernel(
   PageV<KB> vf;
   int page = pg <= pg1 ? table[pg] : -1;
   RowBlock<KB> st;
+  bool values_asked = false;                      // the values of the wave's first page are on their way already
   const bool fused_on = fused.qkv != nullptr;
   // exactly one split has the row's own page among its pages (splits past the sequence's end have none)
   const bool owns_last = fused_on && slot >= 0 && pg_first <= pg_hi && pg1 == pg_hi;
@@ -914,7 +915,12 @@ __global__ __launch_bounds__(64 * SPLIT_WAVES, 2) void attn_split_kernel(
     if (has_first)
       head_load(first, src_row, (int64_t)(kvh * group + wave) * head_dim, fused.q_w, fused.w_f32, fused.has_norm,
                 fused.cos_t, fused.sin_t, fused.rot, pos, head_dim);
-    if (page >= 0) load_page_k<KB, FULL>(kf, k_pages + ((int64_t)page * n_kv + kvh) * page_elems, head_dim);
+    if (page >= 0) {
+      // the first page's values too: asked for behind the barrier below they would cost a trip to memory of their own
+      load_page_k<KB, FULL>(kf, k_pages + ((int64_t)page * n_kv + kvh) * page_elems, head_dim);
+      load_page_v<KB, FULL>(vf, v_pages + ((int64_t)page * n_kv + kvh) * page_elems, head_dim);
+      values_asked = true;
+    }
     if (has_first)
       head_finish(first, fused.has_norm, fused.eps, fused.rot, head_dim, tmp, &q_lds[wave][0], nullptr);
     if (slot >= 0) {
@@ -956,7 +962,8 @@ __global__ __launch_bounds__(64 * SPLIT_WAVES, 2) void attn_split_kernel(
     const int pg_next = pg + SPLIT_WAVES;
     const int page_next = pg_next <= pg1 ? table[pg_next] : -1;
     if (page >= 0) {
-      load_page_v<KB, FULL>(vf, v_pages + ((int64_t)page * n_kv + kvh) * page_elems, head_dim);
+      if (!values_asked) load_page_v<KB, FULL>(vf, v_pages + ((int64_t)page * n_kv + kvh) * page_elems, head_dim);
+      values_asked = false;
       if (fused_on && fused.write_kv && pg == pg_hi) {
         // this page holds the row's own position, whose key and value may not have reached memory yet: take them
         // from LDS. Key `at` is row at%16 of key tile at/16; as a value it is one element of one lane group.
@@ -1039,7 +1046,9 @@ __global__ __launch_bounds__(64 * SPLIT_WAVES, 2) void attn_split_kernel(
 
 // out[seq_row, head, :] = sum_s w_s o_s / sum_s w_s l_s,  w_s = 2^(m_s - max m)  (attn_decode.py:102-118)
 #define COMBINE_MAX_SPLITS 64
-__global__ __launch_bounds__(128) void attn_combine_kernel(const float* __restrict__ part_o,
+#define COMBINE_THREADS 128          // head sizes up to 256: two features a thread
+template <int COMBINE_HELD>          // how many splits a thread asks for before it knows their weights
+__global__ __launch_bounds__(COMBINE_THREADS) void attn_combine_kernel(const float* __restrict__ part_o,
                                                            const float* __restrict__ part_ml,
                                                            const int* __restrict__ seq_slot,
                                                            const int* __restrict__ cu_rows, bf16_t* __restrict__ out,
@@ -1052,6 +1061,16 @@ __global__ __launch_bounds__(128) void attn_combine_kernel(const float* __restri
   const float* ml = part_ml + ((int64_t)seq * n_heads + head) * n_splits * 2;
   const float* po = part_o + ((int64_t)seq * n_heads + head) * n_splits * head_dim;
   const bool live = seq_slot[seq] >= 0;
+  // The partial outputs are asked for before the weights are known, so that one trip to memory serves both (the
+  // kernel moves almost nothing: what it costs is its trips to memory one after the other). A thread holds the first
+  // COMBINE_HELD splits of its (at most two) features; further splits are read after the weights.
+  float held[2][COMBINE_HELD];
+#pragma unroll
+  for (int k = 0; k < 2; ++k) {
+    const int d = min(tid + k * COMBINE_THREADS, head_dim - 1);        // every load unconditional, from a valid place
+#pragma unroll
+    for (int s = 0; s < COMBINE_HELD; ++s) held[k][s] = po[min(s, n_splits - 1) * head_dim + d];
+  }
   if (tid < WAVE) {                       // the first wave turns (m_s, l_s) into weights
     const float ms = (live && tid < n_splits) ? ml[2 * tid] : -INFINITY;
     const float ls = (live && tid < n_splits) ? ml[2 * tid + 1] : 0.f;
@@ -1062,10 +1081,15 @@ __global__ __launch_bounds__(128) void attn_combine_kernel(const float* __restri
     if (tid == 0) inv_l = l > 0.f ? 1.f / l : 0.f;
   }
   __syncthreads();
-  for (int d = tid; d < head_dim; d += blockDim.x) {
+#pragma unroll
+  for (int k = 0; k < 2; ++k) {
+    const int d = tid + k * COMBINE_THREADS;
+    if (d >= head_dim) continue;
     float num = 0.f;
-#pragma unroll 8
-    for (int s = 0; s < n_splits; ++s) num += wgt[s] * po[s * head_dim + d];
+#pragma unroll
+    for (int s = 0; s < COMBINE_HELD; ++s)
+      if (s < n_splits) num += wgt[s] * held[k][s];      // a split without keys has weight 0 and holds finite values
+    for (int s = COMBINE_HELD; s < n_splits; ++s) num += wgt[s] * po[s * head_dim + d];
     o[d] = float_to_bf16(num * inv_l);
   }
 }
@@ -1229,8 +1253,14 @@ static int launch_split(const void* q, const void* k_pages, const void* v_pages,
 #undef LAUNCH_SPLIT
   int rc = DRYFT_LAUNCH_CHECK();
   if (rc || n_splits == 1) return rc;
-  hipLaunchKernelGGL(attn_combine_kernel, dim3(n_seqs, n_heads), dim3(128), 0, stream, part_o, part_ml, seq_slot,
-                     cu_rows, (bf16_t*)out, n_heads, head_dim, n_splits);
+#define COMBINE(HELD)                                                                                              \
+  hipLaunchKernelGGL(attn_combine_kernel<HELD>, dim3(n_seqs, n_heads), dim3(COMBINE_THREADS), 0, stream, part_o,   \
+                     part_ml, seq_slot, cu_rows, (bf16_t*)out, n_heads, head_dim, n_splits)
+  if (n_splits <= 4) COMBINE(4);
+  else if (n_splits <= 8) COMBINE(8);
+  else if (n_splits <= 16) COMBINE(16);
+  else COMBINE(32);
+#undef COMBINE
   return DRYFT_LAUNCH_CHECK();
 }
 

@@ -43,7 +43,8 @@ __global__ void add_rmsnorm_kernel(const T* __restrict__ res, const D* __restric
 
 // The same for rows whose width is a multiple of 8 and at most 8 * 8 * blockDim: a thread owns runs of 8
 // contiguous values, reads them with 16-byte loads issued together, and keeps them in registers between the
-// two passes. This is the kernel that decoding steps use: few rows, so latency rather than bandwidth counts.
+// two passes. This is the kernel that decoding steps use: few rows, so latency rather than bandwidth counts: the
+// weights are asked for together with the row, so that nothing has to come from memory after the reduction.
 #define NORM_VEC_RUNS 8   // runs of 8 values a thread may hold
 
 template <typename T, typename D, int RUNS>
@@ -55,13 +56,15 @@ __global__ __launch_bounds__(512) void add_rmsnorm_vec_kernel(const T* __restric
   __shared__ float scratch[16];
   const int64_t row = blockIdx.x;
   const int64_t base = row * width;
-  float v[RUNS][8];
+  float v[RUNS][8], wv[RUNS][8];
   float ss = 0.f;
 #pragma unroll
   for (int r = 0; r < RUNS; ++r) {
     const int i = (r * blockDim.x + threadIdx.x) * 8;
     if (i < width) {
       load8_as_float(res + base + i, v[r]);
+      if (w_f32) load8_as_float((const float*)w + i, wv[r]);
+      else load8_as_float((const bf16_t*)w + i, wv[r]);
       if (n_partials > 0) {
         float d[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
         int p = 0;
@@ -96,7 +99,7 @@ __global__ __launch_bounds__(512) void add_rmsnorm_vec_kernel(const T* __restric
     if (i < width) {
       float o[8];
 #pragma unroll
-      for (int j = 0; j < 8; ++j) o[j] = rounded_as<T>(v[r][j] * inv) * load_vector(w, i + j, w_f32);
+      for (int j = 0; j < 8; ++j) o[j] = rounded_as<T>(v[r][j] * inv) * wv[r][j];
       store8_from_float(y + base + i, o);
     }
   }
@@ -130,7 +133,7 @@ DRYFT_API int dryft_add_rmsnorm(const void* res, const void* delta, int delta_ki
   const int threads = width >= 2048 ? 512 : 256;
   dim3 grid(n_rows), block(threads);
   if (delta_kind == 0) n_partials = 0;
-  const bool aligned = (((uintptr_t)res | (uintptr_t)delta | (uintptr_t)res_out | (uintptr_t)y) & 15) == 0 &&
+  const bool aligned = (((uintptr_t)res | (uintptr_t)delta | (uintptr_t)res_out | (uintptr_t)y | (uintptr_t)w) & 15) == 0 &&
                        (partial_stride % 4) == 0;
   if (width % 8 == 0 && width <= 8 * NORM_VEC_RUNS * 512 && aligned) {
     if (is_f32)
