@@ -29,7 +29,7 @@ from .linear import linear
 
 _RESIDENT_WORKGROUPS = 512     # of the split kernel: two per compute unit (its registers allow no more)
 _MAX_SPLITS = 32
-_QKV_PARTIAL_ROWS = 32         # decoding steps of up to so many rows take the projection as partial sums over K
+_QKV_PARTIAL_ROWS = 64         # decoding steps of up to so many rows take the projection as partial sums over K
 
 
 class GQAAttention(Mixer):
@@ -81,8 +81,8 @@ class GQAAttention(Mixer):
         fused_decoding = decoding and self.n_heads // self.n_kv <= 16
         # The kernel that norms, rotates, appends and attends in one adds up partial sums of the projection on its way
         # in, so K may be split over workgroups. Measured on Qwen3-4B's sizes, a decoding step with the split against
-        # without: 2.980 against 3.008 ms at 8 sequences, 4.63 against 4.74 at 32, and level with the vendor library's
-        # product at 64 (6.88 against 6.86), where it therefore stays.
+        # without: 2.980 against 3.008 ms at 8 sequences, 4.63 against 4.74 at 32; from 33 rows on the split product is
+        # the kernel that brings its operands straight into LDS (6.75 against 6.86 ms at 64 sequences for q/k/v alone).
         qkv = linear(h, self.w_qkv, allow_partials=fused_decoding, partial_rows=_QKV_PARTIAL_ROWS)
         cos = sin = None
         if self.positions:

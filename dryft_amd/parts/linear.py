@@ -12,7 +12,10 @@ engine/dryft_qwen3/model.py:153, 179-180, 237, 258-261). Here:
   as float32 partial sums over K for the consumer to add;
 * bfloat16, at most 64 rows, the fused gate/up product with its activation: this library's kernel that brings
   its operands straight into LDS (``panel_swiglu_ok``; K a multiple of 128, else the two kernels below);
-* bfloat16, 17 to 64 rows: this library's shared-activation kernel where the consumer adds
+* bfloat16, 33 to 64 rows, where the consumer adds partial sums (q/k/v of decoding steps, the projections back to
+  the hidden width) and K is a multiple of 64: this library's kernel that splits K and brings its operands straight
+  into LDS (``small_mid_plan``);
+* bfloat16, 17 to 64 rows otherwise: this library's shared-activation kernel where the consumer adds
   partial sums (the projections back to the hidden width, which give the vendor library too
   few tiles to fill the chip), where the result is wanted in float32 (the output head) and
   for sizes the vendor library does not take;
@@ -38,6 +41,7 @@ from .base import Partials
 
 STREAM_ROWS = 16                # the most rows the line-staging kernel takes; up to here it beats the vendor library
 WIDE_ROWS = 64                  # the most rows the shared-activation kernel takes
+SMALL_MID_ROWS = 32             # above so many rows (and up to WIDE_ROWS) split products go to the direct-to-LDS kernel
 _STREAM_BLOCKS_PER_WAVE = 5     # measured on the projection shapes of 4B to 32B models inside captured graphs:
 _STREAM_WORKGROUPS = 1536       # short walks over K, as long as the launch stays under about six workgroups a unit
 _COMPUTE_UNITS = 256            # of the MI355X
@@ -80,6 +84,16 @@ def mid_plan(n: int, k: int) -> int:
     if splits >= 1 and groups // max(splits, 1) > 64:
         splits *= 2
     return ops.gemm_mid_splits(k, min(splits, 16)) if splits > 1 else 1
+
+
+def small_mid_plan(n: int, k: int) -> int:
+    """Splits of K across workgroups for the kernel that brings its operands straight into LDS, at 33 to 64 rows (64
+    outputs a workgroup): as many as give every compute unit one workgroup. Measured on Qwen3-4B's sizes, a decoding
+    step with it against the shared-activation kernel (o, down) and the vendor library (q/k/v): 6.64 against 6.86 ms at
+    64 sequences, 5.92 against 6.09 at 48, 5.67 against 5.83 at 40; level at 32 (4.54 against 4.57) and behind at 24,
+    where it is not used."""
+    blocks = (n + 63) // 64
+    return ops.gemm_mid_splits(k, max(1, min(16, _COMPUTE_UNITS // blocks)))
 
 
 def few_rows_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
@@ -133,6 +147,13 @@ def linear(x: torch.Tensor, w: torch.Tensor, *, out_dtype: torch.dtype | None = 
         out = torch.empty((m, n), dtype=out_dtype, device=x.device)
         ops.gemm_stream_bf16(x, w, out, None, group, 1, depth)
         return out
+    if SMALL_MID_ROWS < m <= WIDE_ROWS and allow_partials and few_ok and k % ops.MID_GROUP == 0 and \
+            within_direct_reach(x, w):
+        splits = small_mid_plan(n, k)
+        if splits > 1:
+            partials = torch.empty((splits, m, n), dtype=torch.float32, device=x.device)
+            ops.gemm_mid_bf16(x, w, partials, splits)
+            return Partials(partials, splits)
     if m <= WIDE_ROWS and few_ok:
         splits, group, depth = wide_plan(n, k, allow_partials)
         if splits > 1:

@@ -700,7 +700,7 @@ def test_gemm_panel_swiglu(m, inter, k):
         ops().gemm_panel_swiglu_bf16(x.to(DEV)[:, :64].contiguous(), w.to(DEV)[:, :64].contiguous(), out)
 
 
-@pytest.mark.parametrize("m", [1, 65, 128, 129, 192, 193, 256])
+@pytest.mark.parametrize("m", [1, 17, 32, 33, 48, 64, 65, 128, 129, 192, 193, 256])
 @pytest.mark.parametrize("n,k,splits", [(2560, 4096, 6), (77, 64, 1), (100, 192, 3), (136, 640, 4), (64, 1024, 16),
                                          (130, 9728, 6)])
 def test_gemm_mid(m, n, k, splits):
@@ -803,7 +803,7 @@ def test_linear_dispatch_matches_everywhere():
     torch.manual_seed(5)
     for n, k in ((384, 96), (100, 2560), (331, 72)):           # 331 outputs: no size the vendor library takes
         w = (torch.randn(n, k) / math.sqrt(k)).to(torch.bfloat16).to(DEV)
-        for m in (1, 7, 16, 17, 64, 65, 130, 256, 257, 300):
+        for m in (1, 7, 16, 17, 32, 33, 40, 64, 65, 130, 256, 257, 300):
             x = torch.randn(m, k).to(torch.bfloat16).to(DEV)
             want = x.double().cpu() @ w.double().cpu().T
             close(linear(x, w), want, torch.bfloat16, ulps=1.0, what=f"linear m={m}")
