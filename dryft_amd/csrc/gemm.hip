@@ -885,7 +885,9 @@ DRYFT_API int dryft_gemm_mid_bf16(const void* x, int64_t x_stride, const void* w
   const int groups = K / MID_GROUP, per = (groups + splits - 1) / splits;
   if ((groups + per - 1) / per != splits) return -1;       // a run would be empty
   if (M <= 32) return launch_mid<2>(x, x_stride, w, partials, M, N, K, splits, per, stream);
+  if (M <= 48) return launch_mid<3>(x, x_stride, w, partials, M, N, K, splits, per, stream);
   if (M <= 64) return launch_mid<4>(x, x_stride, w, partials, M, N, K, splits, per, stream);
+  if (M <= 96) return launch_mid<6>(x, x_stride, w, partials, M, N, K, splits, per, stream);
   if (M <= 128) return launch_mid<8>(x, x_stride, w, partials, M, N, K, splits, per, stream);
   if (M <= 192) return launch_mid<12>(x, x_stride, w, partials, M, N, K, splits, per, stream);
   return launch_mid<16>(x, x_stride, w, partials, M, N, K, splits, per, stream);

@@ -29,7 +29,7 @@ from .linear import linear
 
 _RESIDENT_WORKGROUPS = 512     # of the split kernel: two per compute unit (its registers allow no more)
 _MAX_SPLITS = 32
-_QKV_PARTIAL_ROWS = 64         # decoding steps of up to so many rows take the projection as partial sums over K
+_QKV_PARTIAL_ROWS = 128         # decoding steps of up to so many rows take the projection as partial sums over K
 
 
 class GQAAttention(Mixer):
@@ -82,7 +82,8 @@ class GQAAttention(Mixer):
         # The kernel that norms, rotates, appends and attends in one adds up partial sums of the projection on its way
         # in, so K may be split over workgroups. Measured on Qwen3-4B's sizes, a decoding step with the split against
         # without: 2.980 against 3.008 ms at 8 sequences, 4.63 against 4.74 at 32; from 33 rows on the split product is
-        # the kernel that brings its operands straight into LDS (6.75 against 6.86 ms at 64 sequences for q/k/v alone).
+        # the kernel that brings its operands straight into LDS (6.75 against 6.86 ms at 64 sequences for q/k/v alone,
+        # 8.92 against 9.04 ms at 96; at 256 sequences the vendor library's product is ahead, 19.0 against 19.3 ms).
         qkv = linear(h, self.w_qkv, allow_partials=fused_decoding, partial_rows=_QKV_PARTIAL_ROWS)
         cos = sin = None
         if self.positions:

@@ -700,7 +700,7 @@ def test_gemm_panel_swiglu(m, inter, k):
         ops().gemm_panel_swiglu_bf16(x.to(DEV)[:, :64].contiguous(), w.to(DEV)[:, :64].contiguous(), out)
 
 
-@pytest.mark.parametrize("m", [1, 17, 32, 33, 48, 64, 65, 128, 129, 192, 193, 256])
+@pytest.mark.parametrize("m", [1, 17, 32, 33, 48, 49, 64, 65, 96, 97, 128, 129, 192, 193, 256])
 @pytest.mark.parametrize("n,k,splits", [(2560, 4096, 6), (77, 64, 1), (100, 192, 3), (136, 640, 4), (64, 1024, 16),
                                          (130, 9728, 6)])
 def test_gemm_mid(m, n, k, splits):
