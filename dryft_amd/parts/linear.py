@@ -41,6 +41,7 @@ from .base import Partials
 
 STREAM_ROWS = 16                # the most rows the line-staging kernel takes; up to here it beats the vendor library
 WIDE_ROWS = 64                  # the most rows the shared-activation kernel takes
+_SMALL_MID_BYTES = 48 << 20     # the largest matrix that goes there
 SMALL_MID_ROWS = 32             # above so many rows (and up to WIDE_ROWS) split products go to the direct-to-LDS kernel
 _STREAM_BLOCKS_PER_WAVE = 5     # measured on the projection shapes of 4B to 32B models inside captured graphs:
 _STREAM_WORKGROUPS = 1536       # short walks over K, as long as the launch stays under about six workgroups a unit
@@ -88,10 +89,14 @@ def mid_plan(n: int, k: int) -> int:
 
 def small_mid_plan(n: int, k: int) -> int:
     """Splits of K across workgroups for the kernel that brings its operands straight into LDS, at 33 to 64 rows (64
-    outputs a workgroup): as many as give every compute unit one workgroup. Measured on Qwen3-4B's sizes, a decoding
-    step with it against the shared-activation kernel (o, down) and the vendor library (q/k/v): 6.64 against 6.86 ms at
-    64 sequences, 5.92 against 6.09 at 48, 5.67 against 5.83 at 40; level at 32 (4.54 against 4.57) and behind at 24,
-    where it is not used."""
+    outputs a workgroup): as many as give every compute unit one workgroup; 1 where the product stays with the
+    shared-activation kernel or the vendor library. Measured alone in a captured graph at 64 rows, us, against the
+    better of those two: Qwen3-4B's q/k/v 11.7 (13.7), o 8.1 (10.2), down 14.3 (15.6); Qwen3-8B's 16.0 (17.8), 9.9 (11.6),
+    23.3 (25.5); and a decoding step of 64 sequences with it 6.28 against 6.50 ms (Qwen3-4B), 7.58 against 7.71
+    (Qwen3-8B). On larger matrices the same kernel is ahead alone (Qwen3-14B's q/k/v 20.5 against 25.0) and behind in
+    the step (11.27 against 11.18 ms; Qwen3-32B 21.9 against 21.5), so matrices beyond 48 MiB stay where they were."""
+    if n * k * 2 > _SMALL_MID_BYTES:
+        return 1
     blocks = (n + 63) // 64
     return ops.gemm_mid_splits(k, max(1, min(16, _COMPUTE_UNITS // blocks)))
 

@@ -27,7 +27,7 @@ def test_plans_split_k_only_where_partial_sums_are_taken():
     from dryft_amd.parts.linear import mid_plan, small_mid_plan, stream_plan, wide_plan
     # 33 to 64 rows: one workgroup of 64 outputs a compute unit, and no run of K left empty
     assert small_mid_plan(6144, 2560) == 2 and small_mid_plan(2560, 4096) == 6 and small_mid_plan(2560, 9728) == 6
-    assert small_mid_plan(25600, 5120) == 1 and small_mid_plan(64, 64) == 1
+    assert small_mid_plan(5120, 25600) == 1 and small_mid_plan(64, 64) == 1          # beyond 48 MiB; one group of K
     assert stream_plan(6144, 2560, may_split=False)[0] == 1
     assert stream_plan(2560, 9728, may_split=True)[0] > 1
     assert wide_plan(6144, 2560, may_split=False)[0] == 1
