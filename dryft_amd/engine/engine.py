@@ -71,10 +71,10 @@ def require_gpu(device) -> torch.device:
 class PendingStep:
     """A launched decoding step: where its chosen tokens will be, and when."""
 
-    def __init__(self, n: int, device: torch.device):
+    def __init__(self, n: int, chosen: torch.Tensor):
         self.n = n                                            # how many of the entries are the batch's own
-        self.chosen = torch.empty(n, dtype=torch.int32, device=device)
-        self.host = torch.empty(n, dtype=torch.int32).pin_memory()
+        self.chosen = chosen                                  # on the device: where the captured step reads its tokens
+        self.host = torch.empty(chosen.numel(), dtype=torch.int32).pin_memory()
         self.done = torch.cuda.Event()
         self.sampler_state = None
 
@@ -254,8 +254,9 @@ class Engine:
         else:
             logits = graph.replay(slots, list(tokens) + [0] * (width - n))
         self.cache.end_step(live, [1] * len(live))
-        pending = PendingStep(width, self.device)
-        pending.n = n
+        # the tokens are chosen straight into the place the next step reads them from; the copy for the host is
+        # queued before that step, which is the next to write there
+        pending = PendingStep(n, graph.tokens)
         pending.sampler_state = self._sampler.state()
         uniforms = None
         if not self._sampler.greedy:                          # the dead rows of the bucket draw nothing

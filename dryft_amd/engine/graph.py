@@ -41,6 +41,7 @@ class DecodeGraph:
         # take turns, and a step is only launched once the step before the previous one has been waited for.
         self._stages = [torch.zeros(2 * self.batch, dtype=torch.int32).pin_memory() for _ in range(4)]
         self._turn = 0
+        self._slots_there: list[int] | None = None          # the slots the device holds, when known
 
     def _body(self) -> torch.Tensor:
         hidden = self.stepper.run(self.buf, self.ctx)
@@ -48,7 +49,14 @@ class DecodeGraph:
 
     def capture(self, warm_runs: int = 2) -> None:
         self.buf.seq_slot.fill_(-1)
+        self._slots_there = None
         self.graph, self.logits = capture_body(self._body, self.stepper.device, self.pool, warm_runs)
+
+    @property
+    def tokens(self) -> torch.Tensor:
+        """Where the step reads its tokens (int32, on the device): whoever chooses a step's tokens may write them
+        here for the next step and hand this very tensor to ``replay``, which then copies nothing."""
+        return self.buf.tokens
 
     def replay(self, slots: list[int], tokens: list[int] | torch.Tensor) -> torch.Tensor:
         """Logits ``[batch, vocab]`` of one more token each; rows of dead sequences hold nothing of use.
@@ -58,13 +66,17 @@ class DecodeGraph:
         n = self.batch
         stage = self._stages[self._turn]
         self._turn = (self._turn + 1) % len(self._stages)
-        stage[n:] = torch.from_numpy(np.asarray(slots, dtype=np.int32))
         if isinstance(tokens, torch.Tensor):
-            self.buf.tokens.copy_(tokens, non_blocking=True)
+            if tokens.data_ptr() != self.buf.tokens.data_ptr():
+                self.buf.tokens.copy_(tokens, non_blocking=True)
         else:
             stage[:n] = torch.from_numpy(np.asarray(tokens, dtype=np.int32))
             self.buf.tokens.copy_(stage[:n], non_blocking=True)
-        self.buf.seq_slot.copy_(stage[n:], non_blocking=True)
+        slots = list(slots)
+        if slots != self._slots_there:                        # between two steps of a batch they rarely change
+            stage[n:] = torch.from_numpy(np.asarray(slots, dtype=np.int32))
+            self.buf.seq_slot.copy_(stage[n:], non_blocking=True)
+            self._slots_there = slots
         self.graph.replay()
         return self.logits
 
