@@ -563,6 +563,36 @@ __device__ __forceinline__ void panel_wait() {
   asm volatile("" ::: "memory");
 }
 
+// silu for the epilogues whose result is rounded to bfloat16 at once: the hardware's exp2 and reciprocal (about an
+// ulp of float each) instead of the library's exp and an exact division, a fifth of the instructions; the ends of
+// the range come out right (exp2 = inf gives -0, exp2 = 0 gives g).
+__device__ __forceinline__ float silu_for_bf16(float g) {
+  return g * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(g * -1.4426950408889634f));
+}
+
+// The end of the fused gate/up products: of one row, a lane with g < 2 holds the gates of four neighbouring outputs
+// n .. n + 3 (n = first + 4 g), the lane 32 further on their ups. The two lanes share the work: the first takes
+// outputs n and n + 1, the second n + 2 and n + 3, each after one exchange of two values.
+// y[n + i] = T(T(silu(gate)) * up), two values in one store where N is even.
+__device__ __forceinline__ void swiglu_store4(bf16_t* __restrict__ y_row, int first, int N, int g, const f32x4& acc,
+                                              bool row_there) {
+  const bool second = g >= 2;
+  const float got0 = __shfl_xor(second ? acc[0] : acc[2], 32, WAVE);
+  const float got1 = __shfl_xor(second ? acc[1] : acc[3], 32, WAVE);
+  const float gate0 = second ? got0 : acc[0], gate1 = second ? got1 : acc[1];
+  const float up0 = second ? acc[2] : got0, up1 = second ? acc[3] : got1;
+  const int n = first + 4 * (g & 1) + (second ? 2 : 0);
+  const bf16_t v0 = float_to_bf16(rounded_as<bf16_t>(silu_for_bf16(rounded_as<bf16_t>(gate0))) * rounded_as<bf16_t>(up0));
+  const bf16_t v1 = float_to_bf16(rounded_as<bf16_t>(silu_for_bf16(rounded_as<bf16_t>(gate1))) * rounded_as<bf16_t>(up1));
+  if (!row_there || n >= N) return;
+  if (N % 2 == 0) {                                        // then n + 1 < N too, and the address is a multiple of 4
+    *(uint32_t*)(y_row + n) = (uint32_t)v0.bits | ((uint32_t)v1.bits << 16);
+    return;
+  }
+  y_row[n] = v0;
+  if (n + 1 < N) y_row[n + 1] = v1;
+}
+
 #define PANEL_GROUP 128                      // values of K in a group; K must be a multiple of it
 #define PANEL_STAGES 3
 
@@ -667,15 +697,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_panel_swiglu_kernel(const bf1
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
     const int m = 16 * mt + c;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const float up = __shfl_xor(acc[mt][i], 32, WAVE);
-      const int n = n0 + 4 * g + i;
-      if (g >= 2 || m >= M || n >= N) continue;
-      const float gv = rounded_as<bf16_t>(acc[mt][i]), uv = rounded_as<bf16_t>(up);
-      const float sv = rounded_as<bf16_t>(gv / (1.f + expf(-gv)));
-      store_from_float(y + (int64_t)m * N + n, sv * uv);
-    }
+    swiglu_store4(y + (int64_t)min(m, M - 1) * N, n0, N, g, acc[mt], m < M);
   }
 }
 
@@ -891,6 +913,268 @@ DRYFT_API int dryft_gemm_mid_bf16(const void* x, int64_t x_stride, const void* w
   if (M <= 128) return launch_mid<8>(x, x_stride, w, partials, M, N, K, splits, per, stream);
   if (M <= 192) return launch_mid<12>(x, x_stride, w, partials, M, N, K, splits, per, stream);
   return launch_mid<16>(x, x_stride, w, partials, M, N, K, splits, per, stream);
+}
+
+// -------------------------------------------------------------------------------------------- tall
+// Products of 65 to 256 rows (short prompts, decoding at large batch), cut the other way than the panel and mid
+// products above, whose waves each read every row of x from LDS for only 16 rows of W (one LDS read a matrix
+// instruction). Here a workgroup of eight multiplying waves owns T tiles of 16 rows of W and all rows of x; wave w
+// owns R tiles of 16 rows of x (rows 16 R w ...) and multiplies them with all T tiles of W: R + T reads for R T
+// instructions. Operands go from memory straight into LDS in groups of 64 values of K (rows of 128 bytes, piece p of
+// row r at place p ^ ((r / 2) % 8), as in gemm_mid). Two forms:
+//   the fused gate/up product with its activation (a tile of W is 8 gate rows and the 8 up rows of the same outputs,
+//     as in the panel product, so a workgroup owns 8 T outputs over all of K), rounded to bfloat16;
+//   the plain product as float partial sums over runs of K (a tile is 16 outputs).
+// What bounds it, by the cycle counter inside the kernel at Qwen3-4B's gate/up (100 MB, 244 workgroups of 80 rows
+// of W): the waves never wait for data, they wait to issue loads. A compute unit takes in about 46 bytes a cycle of
+// activations from the L2 on top of the time its share of the weights takes to stream from memory (16.5 us), and
+// every workgroup takes in all of x over its run of K: 1.3 MB at 256 rows, 12 us. So the time grows with the rows
+// (20 us inside the loop at 64 rows, 23 at 128, 29 at 256), deeper rings change nothing, and what pays is fewer
+// bytes of x a compute unit: more rows of W a workgroup, shorter runs of K.
+// x and W within reach of 32-bit offsets.
+#define TALL_GROUP 64
+#define TALL_WAVES 8
+#define TALL_LDS (160 * 1024)
+
+// Weights come from memory (about 2 us away: a compute unit's share of the memory rate wants some 44 KB of them in
+// flight), activations from the L2 (nearer, but 16 R / T times as many bytes): each has a ring of its own in LDS, the
+// activations' of X_STAGES groups, the weights' as deep as the rest of LDS allows. A wave's loads are counted off in
+// the order of their issue, so a wave that fetched both would wait for its newest weights whenever it waits for its
+// activations: a ninth wave fetches the weights and does nothing else, the eight that multiply fetch their own rows
+// of x. The weights' ring is no deeper than the 63 loads a wave can count.
+template <int R, int T>
+struct TallPlan {
+  static constexpr int RB = 2 * TALL_GROUP;                             // bytes of a row in a group
+  static constexpr int W_BYTES = 16 * T * RB, X_BYTES = 16 * R * TALL_WAVES * RB;
+  static constexpr int X_STAGES = R == 1 ? 4 : 3;
+  static constexpr int w_fit = (TALL_LDS - X_STAGES * X_BYTES) / W_BYTES, w_count = 63 / (2 * T) + 2;
+  static constexpr int W_STAGES = w_fit < w_count ? (w_fit < 8 ? w_fit : 8) : (w_count < 8 ? w_count : 8);
+  static constexpr int LDS = W_STAGES * W_BYTES + X_STAGES * X_BYTES;
+  static_assert(W_STAGES >= 3, "two groups of weights in flight at least");
+};
+
+// SWIGLU: y is bf16 [M, N], w is [2N, K]. Otherwise y is float [splits, M, N], w is [N, K], and a workgroup sums
+// over one run of `per` groups of K. Workgroups go to the eight dies in turn, each die with an L2 of its own: the
+// (run, tile) pairs are dealt so that a die gets neighbouring ones, and with them few runs of K, whose columns of x
+// are all of x that its L2 has to hold and to fetch (a prompt's 256 rows of Qwen3-4B's down projection are 5 MB,
+// more than one L2). The grid is 8 * ceil(pairs / 8) workgroups; those beyond the last pair leave at once.
+template <int R, int T, bool SWIGLU>
+__global__ __launch_bounds__(64 * (TALL_WAVES + 1)) void gemm_tall_kernel(
+    const bf16_t* __restrict__ x, int64_t x_stride, const bf16_t* __restrict__ w, void* __restrict__ y, int M, int N,
+    int K, int per, int blocks, int splits) {
+  extern __shared__ __align__(16) unsigned char tall_lds[];
+  using Plan = TallPlan<R, T>;
+  constexpr int WAVES = TALL_WAVES, RB = Plan::RB, W_BYTES = Plan::W_BYTES, X_BYTES = Plan::X_BYTES;
+  constexpr int WS = Plan::W_STAGES, XS = Plan::X_STAGES, DW = WS - 1, DX = XS - 1;
+  constexpr int W_LOADS = 2 * T;                           // 1 KB pieces (8 rows) of W in a group
+  constexpr int X_LOADS = 2 * R;                           // a wave's own 16 R rows of x
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
+  const int lane = threadIdx.x % WAVE, c = lane % 16, g = lane / 16;
+  const int pairs = blocks * splits, a_die = (pairs + 7) / 8;
+  const int pair = (int)(blockIdx.x % 8) * a_die + (int)(blockIdx.x / 8);
+  if (pair >= pairs) return;
+  const int run = pair / blocks, block = pair % blocks;
+  const int tile0 = block * T;                             // first tile of this workgroup
+  const int group0 = run * per;                            // its run of K
+  const int groups = min(per, K / TALL_GROUP - group0);
+  const uint32_t lds0 = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)tall_lds);
+  const int first_group = (int)(((unsigned)block * 5u) % (unsigned)groups);   // workgroups walk K from different places
+  auto group_at = [&](int group) {
+    const int gk = group + first_group;
+    return (int64_t)(group0 + (gk >= groups ? gk - groups : gk)) * RB;
+  };
+  // Nothing is fetched past the end of the run, so near the end fewer loads follow a group's than the waits count on:
+  // there a wave waits for all it has issued.
+  if (wave == WAVES) {                                     // the wave that fetches the weights
+    uint32_t w_from[W_LOADS];
+#pragma unroll
+    for (int i = 0; i < W_LOADS; ++i) {
+      const int r = 8 * i + lane / 8;                      // row among the workgroup's 16 T rows of W
+      int row;
+      if (SWIGLU) {                                        // 0..7: gate rows of the tile's outputs, 8..15: their up rows
+        const int tile = tile0 + r / 16, in_tile = r % 16;
+        row = (in_tile < 8 ? 0 : N) + min(8 * tile + (in_tile & 7), N - 1);
+      } else {
+        row = min(16 * tile0 + r, N - 1);
+      }
+      w_from[i] = (uint32_t)row * (uint32_t)K * 2u + (((lane % 8) ^ ((r >> 1) & 7)) << 4);
+    }
+    auto fetch_w = [&](int group, int stage) {
+      const unsigned char* wb = (const unsigned char*)w + group_at(group);
+#pragma unroll
+      for (int i = 0; i < W_LOADS; ++i) panel_load16(wb, w_from[i], lds0 + stage * W_BYTES + i * 1024);
+    };
+#pragma unroll
+    for (int j = 0; j < DW; ++j)
+      if (j < groups) fetch_w(j, j);
+    int w_stage = 0;
+    for (int group = 0; group < groups; ++group) {
+      if (group + DW <= groups) panel_wait<(DW - 1) * W_LOADS>();      // this group's weights have arrived
+      else panel_wait<0>();
+      __syncthreads();                                     // the others hear of it; they are done with the group before
+      if (group + DW < groups) fetch_w(group + DW, w_stage == 0 ? WS - 1 : w_stage - 1);
+      w_stage = w_stage + 1 == WS ? 0 : w_stage + 1;
+    }
+    return;
+  }
+  uint32_t x_from[X_LOADS];
+#pragma unroll
+  for (int i = 0; i < X_LOADS; ++i) {
+    const int r = 16 * R * wave + 8 * i + lane / 8;        // row of x
+    x_from[i] = (uint32_t)min(r, M - 1) * (uint32_t)x_stride * 2u + (((lane % 8) ^ ((r >> 1) & 7)) << 4);
+  }
+  const uint32_t x_lds0 = lds0 + WS * W_BYTES;
+  auto fetch_x = [&](int group, int stage) {
+    const unsigned char* xb = (const unsigned char*)x + group_at(group);
+#pragma unroll
+    for (int i = 0; i < X_LOADS; ++i) panel_load16(xb, x_from[i], x_lds0 + stage * X_BYTES + (2 * R * wave + i) * 1024);
+  };
+  f32x4 acc[R][T];
+#pragma unroll
+  for (int m = 0; m < R; ++m)
+#pragma unroll
+    for (int t = 0; t < T; ++t) acc[m][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int j = 0; j < DX; ++j)
+    if (j < groups) fetch_x(j, j);
+  int w_stage = 0, x_stage = 0;
+  const int sw = (c >> 1) & 7;                             // row 16 t + c of any tile is swizzled like row c
+  // Operands are read from LDS half a group (32 values of K) ahead of the matrix instructions that use them, into one
+  // of two sets of registers, so that the reads of one half run under the instructions of the half before.
+  bf16x8 a[2][T], b[2][R];
+  auto read_half = [&](int u) {
+    const unsigned char* ws = tall_lds + w_stage * W_BYTES + c * RB;
+    const unsigned char* xs = tall_lds + WS * W_BYTES + x_stage * X_BYTES + (16 * R * wave + c) * RB;
+    const int place = ((4 * u + g) ^ sw) << 4;
+#pragma unroll
+    for (int t = 0; t < T; ++t) a[u][t] = *(const bf16x8*)(ws + 16 * t * RB + place);
+#pragma unroll
+    for (int m = 0; m < R; ++m) b[u][m] = *(const bf16x8*)(xs + 16 * m * RB + place);
+  };
+  auto multiply_half = [&](int u) {
+#pragma unroll
+    for (int m = 0; m < R; ++m)
+#pragma unroll
+      for (int t = 0; t < T; ++t) acc[m][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][t], b[u][m], acc[m][t], 0, 0, 0);
+  };
+  for (int group = 0; group < groups; ++group) {
+    if (group + DX <= groups) panel_wait<(DX - 1) * X_LOADS>();        // this group's rows of x have arrived (nobody
+    else panel_wait<0>();                                              // else reads them)
+    __syncthreads();                                       // its weights too; everybody has read the group before
+    if (group + DX < groups) fetch_x(group + DX, x_stage == 0 ? XS - 1 : x_stage - 1);
+    read_half(0);
+    __builtin_amdgcn_sched_barrier(0);
+    if (group > 0) multiply_half(1);                       // the second half of the group before
+    __builtin_amdgcn_sched_barrier(0);
+    read_half(1);
+    __builtin_amdgcn_sched_barrier(0);
+    multiply_half(0);
+    __builtin_amdgcn_sched_barrier(0);
+    w_stage = w_stage + 1 == WS ? 0 : w_stage + 1;
+    x_stage = x_stage + 1 == XS ? 0 : x_stage + 1;
+  }
+  multiply_half(1);
+  // acc[m][t][i] is row 4g + i of W tile t for activation row 16 (R wave + m) + c
+#pragma unroll
+  for (int m = 0; m < R; ++m) {
+    const int row = 16 * (R * wave + m) + c;
+    if (SWIGLU) {                                          // the gate of output 4g + i of the tile in lanes with g < 2,
+      bf16_t* y_row = (bf16_t*)y + (int64_t)min(row, M - 1) * N;                    // its up 32 lanes further on
+#pragma unroll
+      for (int t = 0; t < T; ++t) swiglu_store4(y_row, 8 * (tile0 + t), N, g, acc[m][t], row < M);
+    } else if (row < M) {
+      float* y_row = (float*)y + ((int64_t)run * M + row) * N;
+#pragma unroll
+      for (int t = 0; t < T; ++t) {
+        const int n = 16 * (tile0 + t) + 4 * g;
+        if (N % 4 == 0) {                                  // then n + 3 < N where n < N, and the address is a multiple of 16
+          if (n < N) *(f32x4*)(y_row + n) = acc[m][t];
+        } else {
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (n + i < N) y_row[n + i] = acc[m][t][i];
+        }
+      }
+    }
+  }
+}
+
+template <int R, int T, bool SWIGLU>
+static int launch_tall(const void* x, int64_t x_stride, const void* w, void* y, int M, int N, int K, int splits, int per,
+                       hipStream_t stream) {
+  constexpr int lds = TallPlan<R, T>::LDS;
+  static_assert(lds <= TALL_LDS, "the rings must fit a compute unit's LDS");
+  static bool raised = false;                              // more dynamic LDS than the default limit allows
+  auto kernel = gemm_tall_kernel<R, T, SWIGLU>;
+  if (lds > 64 * 1024 && !raised) {
+    if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess) return -2;
+    raised = true;
+  }
+  const int outputs = (SWIGLU ? 8 : 16) * T, blocks = (N + outputs - 1) / outputs;
+  dim3 grid(8 * ((blocks * splits + 7) / 8)), block(64 * (TALL_WAVES + 1));
+  hipLaunchKernelGGL(kernel, grid, block, lds, stream, (const bf16_t*)x, x_stride, (const bf16_t*)w, y, M, N, K, per, blocks,
+                     splits);
+  return DRYFT_LAUNCH_CHECK();
+}
+
+// How many tiles of 8 outputs a workgroup of the fused gate/up form gets for N outputs: from four to eight, the count
+// whose workgroups fill whole rounds of the 256 compute units best (one workgroup runs on a unit at a time); among
+// equals the most.
+DRYFT_API int dryft_gemm_tall_tiles(int N) {
+  int best = 4;
+  double best_fill = 0.0;
+  for (int tiles = 4; tiles <= 8; ++tiles) {
+    const int groups = (N + 8 * tiles - 1) / (8 * tiles), rounds = (groups + 255) / 256;
+    const double fill = (double)groups / (256.0 * rounds);
+    if (fill >= best_fill - 1e-9) {
+      best_fill = fill > best_fill ? fill : best_fill;
+      best = tiles;
+    }
+  }
+  return best;
+}
+
+template <int R, bool SWIGLU>
+static int tall_tiles(const void* x, int64_t x_stride, const void* w, void* y, int M, int N, int K, int tiles, int splits,
+                      int per, hipStream_t stream) {
+  switch (tiles) {
+    case 4: return launch_tall<R, 4, SWIGLU>(x, x_stride, w, y, M, N, K, splits, per, stream);
+    case 5: return launch_tall<R, 5, SWIGLU>(x, x_stride, w, y, M, N, K, splits, per, stream);
+    case 6: return launch_tall<R, 6, SWIGLU>(x, x_stride, w, y, M, N, K, splits, per, stream);
+    case 7: return launch_tall<R, 7, SWIGLU>(x, x_stride, w, y, M, N, K, splits, per, stream);
+    case 8: return launch_tall<R, 8, SWIGLU>(x, x_stride, w, y, M, N, K, splits, per, stream);
+    default: return -1;
+  }
+}
+
+static bool tall_operands_ok(const void* x, int64_t x_stride, const void* w, int M, int64_t w_rows, int K) {
+  return M <= 256 && K > 0 && K % TALL_GROUP == 0 && x_stride % 8 == 0 && !(((uintptr_t)x | (uintptr_t)w) & 15) &&
+         w_rows * K * 2 < (int64_t)4 << 30 && (int64_t)M * x_stride * 2 < (int64_t)4 << 30;
+}
+
+// M <= 256. y[M, N] = T(T(silu(x . Wg^T)) * (x . Wu^T)) with W = [Wg; Wu] of 2N rows; K a multiple of 64; x and W
+// within reach of 32-bit byte offsets; tiles: 4 to 8, or 0 for dryft_gemm_tall_tiles' choice.
+DRYFT_API int dryft_gemm_tall_swiglu_bf16(const void* x, int64_t x_stride, const void* w, void* y, int M, int N, int K,
+                                          int tiles, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (!tall_operands_ok(x, x_stride, w, M, (int64_t)2 * N, K)) return -1;
+  if (tiles == 0) tiles = dryft_gemm_tall_tiles(N);
+  const int groups = K / TALL_GROUP;
+  if (M <= 128) return tall_tiles<1, true>(x, x_stride, w, y, M, N, K, tiles, 1, groups, stream);
+  return tall_tiles<2, true>(x, x_stride, w, y, M, N, K, tiles, 1, groups, stream);
+}
+
+// M <= 256. partials[s, M, N] = x . W^T over the s-th of `splits` runs of ceil(K / 64 / splits) groups of K (the last
+// run may be shorter, none may be empty: dryft_gemm_mid_splits gives a count that fits); a workgroup owns 16 `tiles`
+// outputs (tiles 4 to 8); K a multiple of 64; x and W within reach of 32-bit byte offsets.
+DRYFT_API int dryft_gemm_tall_bf16(const void* x, int64_t x_stride, const void* w, float* partials, int M, int N, int K,
+                                   int splits, int tiles, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (!tall_operands_ok(x, x_stride, w, M, N, K) || splits < 1 || ((uintptr_t)partials & 15)) return -1;
+  const int groups = K / TALL_GROUP, per = (groups + splits - 1) / splits;
+  if ((groups + per - 1) / per != splits) return -1;       // a run would be empty
+  if (M <= 128) return tall_tiles<1, false>(x, x_stride, w, partials, M, N, K, tiles, splits, per, stream);
+  return tall_tiles<2, false>(x, x_stride, w, partials, M, N, K, tiles, splits, per, stream);
 }
 
 // ------------------------------------------------------------------------------------------- block

@@ -41,6 +41,9 @@ _SIGNATURES = {
              "dryft_gemm_wide_bf16": [_P, _L, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
              "dryft_gemm_panel_swiglu_bf16": [_P, _L, _P, _P, _I, _I, _I, _I, _P],
              "dryft_gemm_panel_waves": [_I],
+             "dryft_gemm_tall_swiglu_bf16": [_P, _L, _P, _P, _I, _I, _I, _I, _P],
+             "dryft_gemm_tall_bf16": [_P, _L, _P, _P, _I, _I, _I, _I, _I, _P],
+             "dryft_gemm_tall_tiles": [_I],
              "dryft_gemm_mid_bf16": [_P, _L, _P, _P, _I, _I, _I, _I, _P],
              "dryft_gemm_block_bf16": [_P, _L, _P, _P, _I, _I, _I, _I, _I, _I, _P],
              "dryft_gemm_block_f32": [_P, _L, _P, _P, _I, _I, _I, _I, _P],
@@ -600,6 +603,60 @@ def gemm_panel_swiglu_bf16(x, w_gate_up, out, waves: int = 0) -> torch.Tensor:
     _check(_fn("gemm", "dryft_gemm_panel_swiglu_bf16")(_ptr(x), x.stride(0), _ptr(w_gate_up), _ptr(out), m, two_n // 2, k,
                                                        int(waves), _stream()), "gemm_panel_swiglu_bf16")
     return out
+
+
+TALL_ROWS = 256     # the most rows gemm_tall_swiglu takes
+TALL_GROUP = 64     # values of K it moves at a time; K must be a multiple of it
+
+
+def gemm_tall_swiglu_bf16(x, w_gate_up, out, tiles: int = 0) -> torch.Tensor:
+    """``silu(x @ Wg.T) * (x @ Wu.T)`` for ``w_gate_up = [Wg; Wu]``, at most 256 rows, by the kernel whose waves each own
+    rows of x and multiply them with all of the workgroup's rows of W (operands straight into LDS). K must be a multiple
+    of 64. ``tiles`` (4 to 8, 8 outputs each) per workgroup; 0 lets the library choose."""
+    _gpu(x, "x", torch.bfloat16)
+    _gpu(w_gate_up, "w_gate_up", torch.bfloat16)
+    _gpu(out, "out", torch.bfloat16)
+    m, k = x.shape
+    two_n = w_gate_up.shape[0]
+    if not (two_n % 2 == 0 and w_gate_up.shape == (two_n, k) and w_gate_up.is_contiguous() and x.stride(1) == 1):
+        raise KernelError("gemm_tall_swiglu: x [M,K] row-major, w [2N,K] contiguous")
+    if not (m <= TALL_ROWS and k % TALL_GROUP == 0 and x.stride(0) % 8 == 0):
+        raise KernelError(f"gemm_tall_swiglu: needs M <= {TALL_ROWS} and K % {TALL_GROUP} == 0, got M={m} K={k}")
+    if not (x.data_ptr() % 16 == 0 and w_gate_up.data_ptr() % 16 == 0):
+        raise KernelError("gemm_tall_swiglu: operands must be 16-byte aligned")
+    if not (out.shape == (m, two_n // 2) and out.is_contiguous()):
+        raise KernelError(f"gemm_tall_swiglu: out must be [{m},{two_n // 2}]")
+    if not (tiles == 0 or 4 <= tiles <= 8):
+        raise KernelError("gemm_tall_swiglu: tiles 4 to 8, or 0")
+    _check(_fn("gemm", "dryft_gemm_tall_swiglu_bf16")(_ptr(x), x.stride(0), _ptr(w_gate_up), _ptr(out), m, two_n // 2, k,
+                                                      int(tiles), _stream()), "gemm_tall_swiglu_bf16")
+    return out
+
+
+def gemm_tall_bf16(x, w, partials, splits: int, tiles: int) -> torch.Tensor:
+    """Float partial sums ``partials[s] = x @ w.T`` over the s-th run of K, at most 256 rows, by the kernel whose waves
+    each own rows of x (see ``gemm_tall_swiglu_bf16``); a workgroup owns ``16 * tiles`` outputs (tiles 4 to 8). K must
+    be a multiple of 64 and ``splits`` a count ``gemm_mid_splits`` gives."""
+    _gpu(x, "x", torch.bfloat16)
+    _gpu(w, "w", torch.bfloat16)
+    _gpu(partials, "partials", torch.float32)
+    m, k = x.shape
+    n = w.shape[0]
+    if not (w.shape == (n, k) and w.is_contiguous() and x.stride(1) == 1):
+        raise KernelError("gemm_tall: x [M,K] row-major, w [N,K] contiguous")
+    if not (m <= TALL_ROWS and k % TALL_GROUP == 0 and x.stride(0) % 8 == 0):
+        raise KernelError(f"gemm_tall: needs M <= {TALL_ROWS} and K % {TALL_GROUP} == 0, got M={m} K={k}")
+    if not (x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0 and partials.data_ptr() % 16 == 0):
+        raise KernelError("gemm_tall: operands must be 16-byte aligned")
+    if not (partials.shape == (splits, m, n) and partials.is_contiguous()):
+        raise KernelError(f"gemm_tall: partials must be [{splits},{m},{n}]")
+    if not 4 <= tiles <= 8:
+        raise KernelError("gemm_tall: tiles 4 to 8")
+    if gemm_mid_splits(k, splits) != splits:
+        raise KernelError(f"gemm_tall: {splits} runs of K={k} would leave one empty")
+    _check(_fn("gemm", "dryft_gemm_tall_bf16")(_ptr(x), x.stride(0), _ptr(w), _ptr(partials), m, n, k, int(splits),
+                                               int(tiles), _stream()), "gemm_tall_bf16")
+    return partials
 
 
 MID_ROWS = 256      # the most rows gemm_mid takes

@@ -19,8 +19,9 @@ engine/dryft_qwen3/model.py:153, 179-180, 237, 258-261). Here:
   partial sums (the projections back to the hidden width, which give the vendor library too
   few tiles to fill the chip), where the result is wanted in float32 (the output head) and
   for sizes the vendor library does not take;
-* bfloat16, 65 to 256 rows (short prompts), the projections back to the hidden width where the consumer adds
-  partial sums: this library's kernel that splits K and brings its operands straight into LDS (``mid_plan``);
+* bfloat16, 65 to 256 rows (short prompts, decoding at large batch) where the consumer adds partial sums and K is a
+  multiple of 64: this library's kernel whose waves each own rows of x, operands straight into LDS (``tall_plan``);
+  the fused gate/up product of as many rows goes to its other form (``tall_swiglu_ok``);
 * bfloat16, otherwise (prompts, decoding at large batch): the vendor library through
   ``torch.mm``, as in the reference; float32 results of many rows and output sizes the
   library does not take are this library's block kernel (128 x 128 or 256 x 256 outputs
@@ -31,6 +32,7 @@ engine/dryft_qwen3/model.py:153, 179-180, 237, 258-261). Here:
 from __future__ import annotations
 
 import contextlib
+import functools
 import os
 import tempfile
 
@@ -74,17 +76,39 @@ def wide_plan(n: int, k: int, may_split: bool) -> tuple[int, int, int]:
     return (splits, 1, 3) if splits > 1 else (1, 2, 1)
 
 
-def mid_plan(n: int, k: int) -> int:
-    """Splits of K across workgroups for the kernel that takes the projections back to the hidden width at 65 to 256
-    rows (64 outputs a workgroup): as many as give every compute unit one workgroup, twice that where a split would
-    still walk more than 64 groups of K; 1 (not worth it) where the outputs alone fill the chip. Measured on the o
-    and down shapes of 4B, 8B and 32B models at 80, 128 and 192 rows."""
-    blocks = (n + 63) // 64
-    groups = k // ops.MID_GROUP
-    splits = _COMPUTE_UNITS // blocks
-    if splits >= 1 and groups // max(splits, 1) > 64:
-        splits *= 2
-    return ops.gemm_mid_splits(k, min(splits, 16)) if splits > 1 else 1
+def tall_plan(m: int, n: int, k: int) -> tuple[int, int]:
+    return _tall_plan(128 if m <= 128 else 256, n, k)
+
+
+@functools.lru_cache(maxsize=None)
+def _tall_plan(loaded: int, n: int, k: int) -> tuple[int, int]:
+    """(tiles of 16 outputs a workgroup, splits of K across workgroups) for the product of 65 to 256 rows whose waves
+    each own rows of x: the pair with the lowest modelled time. The model, fitted (to 4 % in the mean) to in-graph
+    times on rotating cold weights of the q/k/v, o and down shapes of Qwen3-0.6B, 4B, 8B and 14B at 128 and 256 rows,
+    every tile count with four to five split counts each, in us (the rows counted as the 128 or 256 the kernel loads):
+    3.2 + rounds * (11.1 * MB of x a workgroup takes in + 22.5 * MB of W it takes in) + 0.23 * MB of partial sums
+    + 0.074 * MB of W, rounds being how often the workgroups fill the 256 compute units. (A workgroup takes in all
+    rows of x, 128 or 256 of them, over its run of K: that is what the time goes to, and why a split pays also where
+    the outputs alone would fill the chip.) Its choice is within 5 % of the best measured pair for each of those
+    shapes. Against the kernel it replaces here (64 outputs a workgroup, every wave reading all rows of x from LDS),
+    at 256 rows: Qwen3-4B's down 22.5 against 26.8, Qwen3-8B's 34.7 against 59.8, Qwen3-14B's 55.3 against 96.2."""
+    groups = k // ops.TALL_GROUP
+    best, best_cost = (4, 1), float("inf")
+    for tiles in (4, 5, 6, 7, 8):
+        blocks = -(-n // (16 * tiles))
+        seen = set()
+        for want in range(1, min(groups, 32) + 1):
+            splits = ops.gemm_mid_splits(k, want)
+            if splits in seen:
+                continue
+            seen.add(splits)
+            per = -(-groups // splits)
+            rounds = -(-(blocks * splits) // _COMPUTE_UNITS)
+            cost = 3.2 + rounds * (11.1 * loaded + 22.5 * 16 * tiles) * per * 128e-6 + 0.23e-6 * splits * loaded * n * 4 + \
+                0.074e-6 * n * k * 2
+            if cost < best_cost:
+                best, best_cost = (tiles, splits), cost
+    return best
 
 
 def small_mid_plan(n: int, k: int) -> int:
@@ -115,6 +139,20 @@ def panel_swiglu_ok(x: torch.Tensor, w_gate_up: torch.Tensor) -> bool:
     98.4, 95.0 against 103.8, 97.6 against 100.9, 107.8 against 110.4."""
     m, k = x.shape
     return m <= WIDE_ROWS and k % ops.PANEL_GROUP == 0 and few_rows_ok(x, w_gate_up) and within_direct_reach(x, w_gate_up)
+
+
+_TALL_SWIGLU_BYTES = 256 << 20  # gate/up matrices up to here go to the kernel whose waves own rows of x at 65 to 256 rows
+
+
+def tall_swiglu_ok(x: torch.Tensor, w_gate_up: torch.Tensor) -> bool:
+    """Does the fused gate/up product with its activation go, at 65 to 256 rows, to the kernel whose waves each own
+    rows of x? In-graph times on rotating cold weights, us, against the vendor library plus the activation kernel:
+    Qwen3-4B's sizes 30.0 against 35.6 at 128 rows, 36.3 against 51.0 at 256; Qwen3-8B's 46.8 against 55.5 and 57.9
+    against 66.1; Qwen3-14B's (356 MB) 102 against 100 and 129 against 111, so matrices beyond 256 MiB stay with the
+    library."""
+    m, k = x.shape
+    return WIDE_ROWS < m <= ops.TALL_ROWS and k % ops.TALL_GROUP == 0 and few_rows_ok(x, w_gate_up) and \
+        within_direct_reach(x, w_gate_up) and w_gate_up.numel() * w_gate_up.element_size() <= _TALL_SWIGLU_BYTES
 
 
 def within_direct_reach(x: torch.Tensor, w: torch.Tensor) -> bool:
@@ -169,12 +207,11 @@ def linear(x: torch.Tensor, w: torch.Tensor, *, out_dtype: torch.dtype | None = 
             out = torch.empty((m, n), dtype=out_dtype, device=x.device)
             ops.gemm_wide_bf16(x, w, out, None, group, 1, depth)
             return out
-    if m <= ops.MID_ROWS and allow_partials and few_ok and k % ops.MID_GROUP == 0 and within_direct_reach(x, w):
-        splits = mid_plan(n, k)
-        if splits > 1:
-            partials = torch.empty((splits, m, n), dtype=torch.float32, device=x.device)
-            ops.gemm_mid_bf16(x, w, partials, splits)
-            return Partials(partials, splits)
+    if m <= ops.TALL_ROWS and allow_partials and few_ok and k % ops.TALL_GROUP == 0 and within_direct_reach(x, w):
+        tiles, splits = tall_plan(m, n, k)
+        partials = torch.empty((splits, m, n), dtype=torch.float32, device=x.device)
+        ops.gemm_tall_bf16(x, w, partials, splits, tiles)
+        return Partials(partials, splits)
     if library_ok:
         return torch.mm(x, w.t())
     out = torch.empty((m, n), dtype=out_dtype, device=x.device)

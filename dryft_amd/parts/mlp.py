@@ -11,7 +11,7 @@ import torch
 from ..csrc import ops
 from . import register_part
 from .base import FeedForward, matrix
-from .linear import STREAM_ROWS, few_rows_ok, linear, panel_swiglu_ok
+from .linear import STREAM_ROWS, few_rows_ok, linear, panel_swiglu_ok, tall_swiglu_ok
 
 
 class SwiGLU(FeedForward):
@@ -35,6 +35,8 @@ class SwiGLU(FeedForward):
         act = torch.empty((h.shape[0], self.inter), dtype=h.dtype, device=h.device)
         if h.dtype == torch.bfloat16 and panel_swiglu_ok(h, self.w_gate_up):
             ops.gemm_panel_swiglu_bf16(h, self.w_gate_up, act)        # product and activation in one kernel
+        elif h.dtype == torch.bfloat16 and tall_swiglu_ok(h, self.w_gate_up):
+            ops.gemm_tall_swiglu_bf16(h, self.w_gate_up, act)         # the same at 65 to 256 rows
         elif h.dtype == torch.bfloat16 and h.shape[0] <= STREAM_ROWS and few_rows_ok(h, self.w_gate_up):
             ops.gemm_stream_swiglu_bf16(h, self.w_gate_up, act)       # the same for any K that is a multiple of 8
         else:

@@ -700,6 +700,80 @@ def test_gemm_panel_swiglu(m, inter, k):
         ops().gemm_panel_swiglu_bf16(x.to(DEV)[:, :64].contiguous(), w.to(DEV)[:, :64].contiguous(), out)
 
 
+@pytest.mark.parametrize("m", [1, 65, 100, 128, 129, 200, 256])
+@pytest.mark.parametrize("inter,k,tiles", [(9728, 2560, 0), (224, 128, 4), (136, 384, 5), (37 * 8, 640, 6), (47, 64, 7),
+                                           (49, 256, 8), (700, 192, 0)])
+def test_gemm_tall_swiglu(m, inter, k, tiles):
+    """The gate/up product with its activation for up to 256 rows: row counts on both sides of one tile of 16 a wave
+    and of two, output counts that are no multiple of 8 or of what a workgroup owns, every count of tiles a workgroup,
+    one group of K and many; a row of x strided wider than K."""
+    torch.manual_seed(m + inter)
+    x = torch.randn(m, k).to(torch.bfloat16)
+    w = (torch.randn(2 * inter, k) * 2 / math.sqrt(k)).to(torch.bfloat16)
+    gu = (x.double() @ w.double().T).to(torch.bfloat16).float()            # the unfused path rounds the product first
+    want = (torch.nn.functional.silu(gu[:, :inter]).to(torch.bfloat16).float() * gu[:, inter:]).to(torch.bfloat16)
+    out = torch.full((m, inter), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ops().gemm_tall_swiglu_bf16(x.to(DEV), w.to(DEV), out, tiles)
+    close(out, want, torch.bfloat16, what="tall swiglu")
+    wide = torch.zeros(m, k + 8, dtype=torch.bfloat16, device=DEV)
+    wide[:, :k] = x.to(DEV)
+    out2 = torch.full((m, inter), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ops().gemm_tall_swiglu_bf16(wide[:, :k], w.to(DEV), out2, tiles)
+    assert torch.equal(out, out2)
+
+
+@pytest.mark.parametrize("m", [1, 65, 128, 129, 200, 256])
+@pytest.mark.parametrize("n,k,splits,tiles", [(2560, 4096, 6, 5), (77, 64, 1, 4), (100, 192, 3, 6), (136, 640, 4, 7),
+                                              (64, 1024, 16, 8), (130, 9728, 6, 4), (1000, 1280, 2, 5)])
+def test_gemm_tall(m, n, k, splits, tiles):
+    """Float partial sums over runs of K by the kernel whose waves own rows of x: row counts on both sides of one tile
+    of 16 a wave and of two, output counts that are no multiple of 4 or of what a workgroup owns, every count of tiles,
+    runs of one group (shorter than the rings are deep) and of many, of unequal length; every run against the product
+    over itself; a row of x strided wider than K."""
+    torch.manual_seed(m + n + k)
+    o = ops()
+    assert o.gemm_mid_splits(k, splits) == splits
+    x, w = torch.randn(m, k).to(torch.bfloat16), (torch.randn(n, k) / math.sqrt(k)).to(torch.bfloat16)
+    parts = torch.full((splits, m, n), float("nan"), dtype=torch.float32, device=DEV)
+    o.gemm_tall_bf16(x.to(DEV), w.to(DEV), parts, splits, tiles)
+    groups = k // 64
+    per = -(-groups // splits)
+    for s in range(splits):
+        a, b = 64 * per * s, min(k, 64 * per * (s + 1))
+        close(parts[s], x[:, a:b].double() @ w[:, a:b].double().T, torch.float32, what=f"tall, run {s}")
+    close(parts.sum(0), x.double() @ w.double().T, torch.float32, what="tall, sum")
+    wide = torch.zeros(m, k + 8, dtype=torch.bfloat16, device=DEV)
+    wide[:, :k] = x.to(DEV)
+    parts2 = torch.full((splits, m, n), float("nan"), dtype=torch.float32, device=DEV)
+    o.gemm_tall_bf16(wide[:, :k], w.to(DEV), parts2, splits, tiles)
+    assert torch.equal(parts, parts2)
+
+
+def test_gemm_tall_refuses():
+    o = ops()
+    w = torch.zeros(64, 128, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(Exception, match="M <= 256"):
+        o.gemm_tall_bf16(torch.zeros(257, 128, dtype=torch.bfloat16, device=DEV), w,
+                         torch.empty(1, 257, 64, dtype=torch.float32, device=DEV), 1, 4)
+    with pytest.raises(Exception, match="leave one empty"):
+        o.gemm_tall_bf16(torch.zeros(80, 256, dtype=torch.bfloat16, device=DEV), torch.zeros(64, 256, dtype=torch.bfloat16, device=DEV),
+                         torch.empty(3, 80, 64, dtype=torch.float32, device=DEV), 3, 4)
+    with pytest.raises(Exception, match="tiles 4 to 8"):
+        o.gemm_tall_bf16(torch.zeros(80, 128, dtype=torch.bfloat16, device=DEV), w,
+                         torch.empty(1, 80, 64, dtype=torch.float32, device=DEV), 1, 3)
+
+
+def test_gemm_tall_swiglu_refuses():
+    o = ops()
+    w = torch.zeros(64, 128, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(Exception, match="M <= 256"):
+        o.gemm_tall_swiglu_bf16(torch.zeros(257, 128, dtype=torch.bfloat16, device=DEV), w,
+                                torch.empty(257, 32, dtype=torch.bfloat16, device=DEV))
+    with pytest.raises(Exception, match="K % 64"):
+        o.gemm_tall_swiglu_bf16(torch.zeros(80, 96, dtype=torch.bfloat16, device=DEV), w[:, :96].contiguous(),
+                                torch.empty(80, 32, dtype=torch.bfloat16, device=DEV))
+
+
 @pytest.mark.parametrize("m", [1, 17, 32, 33, 48, 49, 64, 65, 96, 97, 128, 129, 192, 193, 256])
 @pytest.mark.parametrize("n,k,splits", [(2560, 4096, 6), (77, 64, 1), (100, 192, 3), (136, 640, 4), (64, 1024, 16),
                                          (130, 9728, 6)])
