@@ -25,7 +25,10 @@ _SIGNATURES = {
              "dryft_add_rows": [_P, _P, _P, _L, _I, _P]},
     "activation": {"dryft_silu_mul": [_P, _P, _I, _I, _L, _I, _P]},
     "rope_kv": {"dryft_qk_norm_rope_kv": [_P, _L, _P, _P, _I, _I, _F, _P, _P, _I, _P, _P, _P, _P, _P, _P, _I, _I,
-                                          _I, _I, _I, _I, _I, _P]},
+                                          _I, _I, _I, _I, _I, _P],
+                "dryft_rows_to_cache_takes": [_I, _I, _I, _I],
+                "dryft_rows_to_cache_parts": [_P, _I, _L, _P, _P, _I, _I, _F, _P, _P, _I, _P, _P, _P, _P, _P, _P, _I, _I,
+                                              _I, _I, _I, _P]},
     "attn_rows": {"dryft_attn_rows": [_P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _F, _I, _I, _P]},
     "attn_mfma": {"dryft_attn_causal_bf16": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _P, _I, _I, _I, _F, _I, _I, _P],
                   "dryft_attn_causal_takes_projection": [_I, _I],
@@ -267,6 +270,57 @@ def qk_norm_rope_kv(qkv: torch.Tensor, q_weight, k_weight, eps: float, cos, sin,
         _ptr(sin), int(rot), _ptr(row_slot), _ptr(row_pos), _ptr(q_out), _ptr(k_pages), _ptr(v_pages),
         _ptr(page_table), max_pages, int(write_kv), rows, n_heads, n_kv, head_dim, is_f32, _stream()),
         "qk_norm_rope_kv")
+
+
+def rows_to_cache_takes(n_rows: int, head_dim: int, rot: int, write_kv: bool) -> bool:
+    """Can ``rows_to_cache_from_partials`` take a step of so many rows, heads of this size rotated over ``rot``
+    features?"""
+    return bool(_fn("rope_kv", "dryft_rows_to_cache_takes")(int(n_rows), int(head_dim), int(rot), int(write_kv)))
+
+
+def rows_to_cache_from_partials(parts: torch.Tensor, q_weight, k_weight, eps: float, cos, sin, rot: int, row_slot,
+                                row_pos, q_out, k_pages, v_pages, page_table, n_heads: int, n_kv: int,
+                                head_dim: int) -> None:
+    """``qk_norm_rope_kv`` for a bfloat16 step whose projection was left as float partial sums ``parts`` [count, rows,
+    columns]: each value is the sum of its parts rounded to bfloat16, then normed, rotated and written as there (queries
+    to ``q_out``, or nowhere if it is None; keys and values to the cache)."""
+    _gpu(parts, "parts", torch.float32)
+    if not (parts.dim() == 3 and parts.is_contiguous()):
+        raise KernelError("rows_to_cache_from_partials: parts must be [count, rows, columns], contiguous")
+    count, rows, cols = parts.shape
+    if not (cols >= (n_heads + 2 * n_kv) * head_dim and cols % 8 == 0):
+        raise KernelError(f"rows_to_cache_from_partials: parts need {(n_heads + 2 * n_kv) * head_dim} columns, a multiple "
+                          f"of 8; have {cols}")
+    if not rows_to_cache_takes(rows, head_dim, rot, True):
+        raise KernelError(f"rows_to_cache_from_partials: takes steps of at least 64 rows, a full rotation and head sizes "
+                          f"32, 64, 128, 256; got {rows} rows, head size {head_dim}, rotation over {rot}")
+    has_norm = q_weight is not None
+    w_f32 = 0
+    if has_norm:
+        for name, w in (("q_weight", q_weight), ("k_weight", k_weight)):
+            _gpu(w, name)
+            if not (w.shape == (head_dim,) and w.is_contiguous()):
+                raise KernelError(f"{name}: must be [{head_dim}]")
+        if not (q_weight.dtype == k_weight.dtype):
+            raise KernelError("q_weight and k_weight must share a dtype")
+        w_f32 = _float_flag(q_weight, "q_weight")
+    for name, t in (("cos", cos), ("sin", sin)):
+        _gpu(t, name, torch.bfloat16)
+        if not (t.dim() == 2 and t.shape[1] == rot // 2 and t.is_contiguous()):
+            raise KernelError(f"{name}: must be [positions, {rot // 2}]")
+    for name, t in (("row_slot", row_slot), ("row_pos", row_pos)):
+        _gpu(t, name, torch.int32)
+        if not (t.numel() >= rows and t.is_contiguous()):
+            raise KernelError(f"{name}: needs {rows} entries")
+    if q_out is not None:
+        _gpu(q_out, "q_out", torch.bfloat16)
+        if not (q_out.is_contiguous() and q_out.numel() == rows * n_heads * head_dim):
+            raise KernelError("q_out: must be [rows, heads, head_dim]")
+    _check_pages(k_pages, v_pages, page_table, n_kv, head_dim, torch.bfloat16)
+    _check(_fn("rope_kv", "dryft_rows_to_cache_parts")(
+        _ptr(parts), int(count), cols, _ptr(q_weight), _ptr(k_weight), w_f32, int(has_norm), float(eps), _ptr(cos),
+        _ptr(sin), int(rot), _ptr(row_slot), _ptr(row_pos), _ptr(q_out), _ptr(k_pages), _ptr(v_pages),
+        _ptr(page_table), page_table.shape[1], rows, n_heads, n_kv, head_dim, _stream()), "rows_to_cache_parts")
 
 
 def _check_pages(k_pages, v_pages, page_table, n_kv: int, head_dim: int, dtype) -> None:

@@ -14,6 +14,28 @@
 
 #define MAX_HEAD_DIM 512
 
+// Eight values of the projection's output at element `at`: from the output itself, or, where the product was left as
+// `parts` float partial sums (each `part_stride` elements after the other, `qkv` pointing at the first), their sum
+// rounded as the output would have been.
+template <typename T>
+__device__ __forceinline__ void load8_projected(const T* __restrict__ qkv, int64_t at, int parts, int64_t part_stride,
+                                                float (&v)[8]) {
+  if (parts == 0) {
+    load8_as_float(qkv + at, v);
+    return;
+  }
+  const float* f = (const float*)qkv + at;
+  load8_as_float(f, v);
+  for (int s = 1; s < parts; ++s) {
+    float more[8];
+    load8_as_float(f + s * part_stride, more);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] += more[j];
+  }
+#pragma unroll
+  for (int j = 0; j < 8; ++j) v[j] = rounded_as<T>(v[j]);
+}
+
 template <typename T>
 __global__ void qk_norm_rope_kv_kernel(const T* __restrict__ qkv, int64_t qkv_stride, const void* __restrict__ q_w,
                                        const void* __restrict__ k_w, int w_f32, int has_norm, float eps,
@@ -181,7 +203,8 @@ __device__ __forceinline__ void qk_norm_rope_row(int64_t row, const T* __restric
                                                  const T* __restrict__ sin_t, const int* __restrict__ row_slot,
                                                  const int* __restrict__ row_pos, T* __restrict__ q_out,
                                                  T* __restrict__ k_pages, const int* __restrict__ page_table,
-                                                 int max_pages, int write_kv, int n_heads, int n_kv) {
+                                                 int max_pages, int write_kv, int n_heads, int n_kv, int parts,
+                                                 int64_t part_stride) {
   constexpr int D = 8 * LPH, PER = 256 / LPH;           // heads a workgroup handles side by side
   const int part = threadIdx.x % LPH, lane_head = threadIdx.x / LPH;
   const int slot = row_slot[row], pos = row_pos[row];
@@ -207,12 +230,12 @@ __device__ __forceinline__ void qk_norm_rope_row(int64_t row, const T* __restric
   }
   const int page = write_kv ? page_of(page_table, max_pages, slot, pos) : -1;
   const int jobs = n_heads + (page >= 0 ? n_kv : 0);    // q heads, then k heads
-  const T* src = qkv + row * qkv_stride + 8 * part;
+  const int64_t src = row * qkv_stride + 8 * part;
   for (int j0 = (q_out != nullptr ? 0 : n_heads) + lane_head; j0 < jobs; j0 += 4 * PER) {   // without q_out: keys only
     float v[4][8];
 #pragma unroll
     for (int u = 0; u < 4; ++u)
-      if (j0 + u * PER < jobs) load8_as_float(src + (int64_t)(j0 + u * PER) * D, v[u]);
+      if (j0 + u * PER < jobs) load8_projected(qkv, src + (int64_t)(j0 + u * PER) * D, parts, part_stride, v[u]);
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       const int job = j0 + u * PER;                      // the same for the LPH lanes that share a head
@@ -256,7 +279,7 @@ __device__ __forceinline__ void v_tile_write(int tile_index, int kvh, const T* _
                                              int v_col0, const int* __restrict__ row_slot,
                                              const int* __restrict__ row_pos, T* __restrict__ v_pages,
                                              const int* __restrict__ page_table, int max_pages, int n_rows, int n_kv,
-                                             int head_dim) {
+                                             int head_dim, int parts, int64_t part_stride) {
   __shared__ int64_t base[V_TILE_ROWS];                     // start of the row's page for this kv head, or -1
   __shared__ int in_page[V_TILE_ROWS];                      // the row's position within its page
   __shared__ int block_ok[V_TILE_ROWS / 32];
@@ -267,7 +290,7 @@ __device__ __forceinline__ void v_tile_write(int tile_index, int kvh, const T* _
   for (int e = threadIdx.x; e < V_TILE_ROWS * chunks; e += blockDim.x) {
     const int t = e / chunks, ch = e % chunks;
     float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    if (t < rows) load8_as_float(qkv + (int64_t)(r0 + t) * qkv_stride + v_col0 + kvh * head_dim + 8 * ch, v);
+    if (t < rows) load8_projected(qkv, (int64_t)(r0 + t) * qkv_stride + v_col0 + kvh * head_dim + 8 * ch, parts, part_stride, v);
 #pragma unroll
     for (int j = 0; j < 8; ++j) store_from_float(tile + (8 * ch + j) * V_TILE_LD + t, v[j]);
   }
@@ -322,7 +345,7 @@ __global__ __launch_bounds__(256) void v_tile_write_kernel(const T* __restrict__
                                                            const int* __restrict__ page_table, int max_pages,
                                                            int n_rows, int n_kv, int head_dim) {
   v_tile_write<T>(blockIdx.x, blockIdx.y, qkv, qkv_stride, v_col0, row_slot, row_pos, v_pages, page_table, max_pages,
-                  n_rows, n_kv, head_dim);
+                  n_rows, n_kv, head_dim, 0, 0);
 }
 
 // One launch for a step of many rows: the first workgroups turn the tiles of values (few, and waiting on memory
@@ -336,15 +359,17 @@ __global__ __launch_bounds__(256) void rows_to_cache_kernel(const T* __restrict_
                                                             const int* __restrict__ row_pos, T* __restrict__ q_out,
                                                             T* __restrict__ k_pages, T* __restrict__ v_pages,
                                                             const int* __restrict__ page_table, int max_pages,
-                                                            int write_kv, int n_rows, int n_heads, int n_kv, int v_tiles) {
+                                                            int write_kv, int n_rows, int n_heads, int n_kv, int v_tiles,
+                                                            int parts, int64_t part_stride) {
   const int v_blocks = v_tiles * n_kv;                      // none when nothing is cached
   if ((int)blockIdx.x < v_blocks) {
     v_tile_write<T>(blockIdx.x % v_tiles, blockIdx.x / v_tiles, qkv, qkv_stride, (n_heads + n_kv) * 8 * LPH, row_slot,
-                    row_pos, v_pages, page_table, max_pages, n_rows, n_kv, 8 * LPH);
+                    row_pos, v_pages, page_table, max_pages, n_rows, n_kv, 8 * LPH, parts, part_stride);
     return;
   }
   qk_norm_rope_row<T, LPH>((int64_t)blockIdx.x - v_blocks, qkv, qkv_stride, q_w, k_w, w_f32, has_norm, eps, cos_t, sin_t,
-                           row_slot, row_pos, q_out, k_pages, page_table, max_pages, write_kv, n_heads, n_kv);
+                           row_slot, row_pos, q_out, k_pages, page_table, max_pages, write_kv, n_heads, n_kv, parts,
+                           part_stride);
 }
 
 template <typename T>
@@ -352,7 +377,7 @@ static int launch_rows_to_cache(const void* qkv, int64_t qkv_stride, const void*
                                 int has_norm, float eps, const void* cos_t, const void* sin_t, const int* row_slot,
                                 const int* row_pos, void* q_out, void* k_pages, void* v_pages, const int* page_table,
                                 int max_pages, int write_kv, int n_rows, int n_heads, int n_kv, int head_dim,
-                                hipStream_t stream) {
+                                hipStream_t stream, int parts = 0, int64_t part_stride = 0) {
   const int v_tiles = write_kv ? (n_rows + V_TILE_ROWS - 1) / V_TILE_ROWS : 0;
   const size_t lds = (size_t)head_dim * V_TILE_LD * sizeof(T);
 #define ROWS(LPHV)                                                                                                     \
@@ -363,7 +388,8 @@ static int launch_rows_to_cache(const void* qkv, int64_t qkv_stride, const void*
       return -2;                                                                                                       \
     hipLaunchKernelGGL(kernel, dim3(v_tiles * n_kv + n_rows), dim3(256), lds, stream, (const T*)qkv, qkv_stride, q_w,  \
                        k_w, w_f32, has_norm, eps, (const T*)cos_t, (const T*)sin_t, row_slot, row_pos, (T*)q_out,       \
-                       (T*)k_pages, (T*)v_pages, page_table, max_pages, write_kv, n_rows, n_heads, n_kv, v_tiles);      \
+                       (T*)k_pages, (T*)v_pages, page_table, max_pages, write_kv, n_rows, n_heads, n_kv, v_tiles,       \
+                       parts, part_stride);                                                                            \
   }
   switch (head_dim) {
     case 32: ROWS(4); break;
@@ -373,6 +399,29 @@ static int launch_rows_to_cache(const void* qkv, int64_t qkv_stride, const void*
   }
 #undef ROWS
   return DRYFT_LAUNCH_CHECK();
+}
+
+// The many-row form of dryft_qk_norm_rope_kv below for a projection left as `parts` float partial sums
+// [parts, n_rows, qkv_stride] (bfloat16 activations, weights and cache): every value is the sum of its parts rounded
+// to bfloat16, then treated as there. For steps of at least 64 rows that write the cache, a full rotation and a head
+// size of 32, 64, 128 or 256: dryft_rows_to_cache_takes says whether a step qualifies.
+DRYFT_API int dryft_rows_to_cache_takes(int n_rows, int head_dim, int rot, int write_kv) {
+  return write_kv && n_rows >= 64 && rot == head_dim && (head_dim == 32 || head_dim == 64 || head_dim == 128 || head_dim == 256);
+}
+
+DRYFT_API int dryft_rows_to_cache_parts(const float* qkv_parts, int parts, int64_t qkv_stride, const void* q_w,
+                                        const void* k_w, int w_f32, int has_norm, float eps, const void* cos_t,
+                                        const void* sin_t, int rot, const int* row_slot, const int* row_pos, void* q_out,
+                                        void* k_pages, void* v_pages, const int* page_table, int max_pages, int n_rows,
+                                        int n_heads, int n_kv, int head_dim, hipStream_t stream) {
+  if (n_rows <= 0) return 0;
+  if (parts < 1 || !dryft_rows_to_cache_takes(n_rows, head_dim, rot, 1)) return -1;
+  if ((((uintptr_t)qkv_parts | (uintptr_t)q_out | (uintptr_t)k_pages | (uintptr_t)v_pages | (uintptr_t)cos_t |
+        (uintptr_t)sin_t) & 15) || qkv_stride % 8)
+    return -1;
+  return launch_rows_to_cache<bf16_t>(qkv_parts, qkv_stride, q_w, k_w, w_f32, has_norm, eps, cos_t, sin_t, row_slot,
+                                      row_pos, q_out, k_pages, v_pages, page_table, max_pages, 1, n_rows, n_heads, n_kv,
+                                      head_dim, stream, parts, (int64_t)n_rows * qkv_stride);
 }
 
 DRYFT_API int dryft_qk_norm_rope_kv(const void* qkv, int64_t qkv_stride, const void* q_w, const void* k_w, int w_f32,

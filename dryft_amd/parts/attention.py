@@ -30,6 +30,7 @@ from .linear import linear
 _RESIDENT_WORKGROUPS = 512     # of the split kernel: two per compute unit (its registers allow no more)
 _MAX_SPLITS = 32
 _QKV_PARTIAL_ROWS = 128         # decoding steps of up to so many rows take the projection as partial sums over K
+_PROMPT_PARTIAL_ROWS = (64, 256)     # and so do prompt steps of more than so many and at most so many rows
 
 
 class GQAAttention(Mixer):
@@ -84,18 +85,29 @@ class GQAAttention(Mixer):
         # without: 2.980 against 3.008 ms at 8 sequences, 4.63 against 4.74 at 32; from 33 rows on the split product is
         # the kernel that brings its operands straight into LDS (6.75 against 6.86 ms at 64 sequences for q/k/v alone,
         # 8.92 against 9.04 ms at 96; at 256 sequences the vendor library's product is ahead, 19.0 against 19.3 ms).
-        qkv = linear(h, self.w_qkv, allow_partials=fused_decoding, partial_rows=_QKV_PARTIAL_ROWS)
         cos = sin = None
         if self.positions:
             table = ctx.positions[self.positions]
             cos, sin = table.cos, table.sin
             if ctx.max_kv_len > table.n_positions:
                 raise ValueError(f"position tables cover {table.n_positions} positions, the step reaches {ctx.max_kv_len}")
+        # So does the kernel that takes a short prompt's keys and values to the cache (and its queries out): at 65 to
+        # 256 rows the split product is ahead of the vendor library's (Qwen3-4B's q/k/v at 256 rows: 17.9 against 31.0 us).
+        prompt_parts = matrix_cores and not decoding and writes_cache and cos is not None and \
+            _PROMPT_PARTIAL_ROWS[0] < rows <= _PROMPT_PARTIAL_ROWS[1] and \
+            ops.rows_to_cache_takes(rows, self.head_dim, self.rotary_dim, True)
+        if prompt_parts:
+            qkv = linear(h, self.w_qkv, allow_partials=True)
+        else:
+            qkv = linear(h, self.w_qkv, allow_partials=fused_decoding, partial_rows=_QKV_PARTIAL_ROWS)
         window = self.window or 0
-        # Every kernel leaves the rows of sequences that sit out at zero; the tiled prompt kernels never visit them,
-        # so for those the rows are cleared beforehand wherever the step may hold such sequences.
-        make = torch.zeros if ctx.max_q_len > 1 and ctx.some_sit_out() else torch.empty
-        out = make((rows, self.n_heads, self.head_dim), dtype=h.dtype, device=h.device)
+        # The tiled prompt kernels never visit the rows of sequences that sit out, and the projection after them reads
+        # every row: where the step may hold such sequences the output lives in a tensor that started as zeros, so
+        # that those rows hold zeros or an earlier layer's or step's output, never what memory happened to hold.
+        if ctx.max_q_len > 1 and ctx.some_sit_out():
+            out = ctx.kept_zeros((rows, self.n_heads, self.head_dim), h.dtype)
+        else:
+            out = torch.empty((rows, self.n_heads, self.head_dim), dtype=h.dtype, device=h.device)
         if decoding:
             splits = self.decode_splits(ctx.n_seqs, ctx.max_kv_len)
             part_o = torch.empty((ctx.n_seqs, self.n_heads, splits, self.head_dim), dtype=torch.float32, device=h.device)
@@ -107,6 +119,16 @@ class GQAAttention(Mixer):
                                        writes_cache, line.k, line.v, line.page_table, ctx.seq_slot, ctx.cu_rows,
                                        ctx.kv_len, ctx.n_seqs, part_o, part_ml, splits, out, self.n_heads, self.n_kv,
                                        self.head_dim, self.scale, window, qkv_parts=parts)
+            return linear(out.view(rows, self.q_dim), self.w_o, allow_partials=True)
+        if prompt_parts and isinstance(qkv, Partials):
+            q = torch.empty((rows, self.n_heads, self.head_dim), dtype=h.dtype, device=h.device)
+            ops.rows_to_cache_from_partials(qkv.data, self.q_norm, self.k_norm, self.qk_norm_eps or 0.0, cos, sin,
+                                            self.rotary_dim, ctx.row_slot, ctx.row_pos, q, line.k, line.v,
+                                            line.page_table, self.n_heads, self.n_kv, self.head_dim)
+            tile_cu, max_tiles = ctx.tiles(ops.ATTN_ROW_TILE)
+            ops.attn_causal_bf16(q, line.k, line.v, line.page_table, ctx.seq_slot, ctx.cu_rows, tile_cu,
+                                 ctx.seq_start, ctx.n_seqs, max_tiles, out, self.n_heads, self.n_kv,
+                                 self.head_dim, self.scale, window)
             return linear(out.view(rows, self.q_dim), self.w_o, allow_partials=True)
         if matrix_cores and not decoding and cos is not None and \
                 ops.attn_causal_takes_projection(self.head_dim, self.rotary_dim):

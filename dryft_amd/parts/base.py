@@ -58,6 +58,7 @@ class StepContext:
     host: HostBatch | None = None
     positions: dict[str, Any] = field(default_factory=dict)   # name -> position encoding, tables ready
     _tiles: dict[int, tuple[torch.Tensor, int]] = field(default_factory=dict, repr=False)
+    _kept: dict[Any, torch.Tensor] = field(default_factory=dict, repr=False)
 
     def tiles(self, rows_per_tile: int) -> tuple[torch.Tensor, int]:
         """For kernels that walk the step tile by tile: ``(tile_cu, bound)``. ``tile_cu`` (int32, device,
@@ -74,6 +75,19 @@ class StepContext:
             else:
                 bound = self.n_seqs * -(-self.max_q_len // rows_per_tile)
             found = self._tiles[rows_per_tile] = (tile_cu, bound)
+        return found
+
+    def kept_zeros(self, shape: tuple[int, ...], dtype: torch.dtype) -> torch.Tensor:
+        """A tensor that starts as zeros and lives as long as the context, one per shape and dtype, shared by every
+        part that asks: for an output of which a kernel writes only the rows of sequences that take part, while the
+        other rows must hold something finite (zeros, or what an earlier step or layer left there) because products
+        and norms downstream read whole rows. Cleared once, not once a layer. A part that hands such a tensor on must
+        be done with it before the next part of the step asks for the same shape (the parts of a step run one after
+        another on one stream, so a mixer's output that the same mixer's projection consumes qualifies)."""
+        key = (tuple(shape), dtype)
+        found = self._kept.get(key)
+        if found is None:
+            found = self._kept[key] = torch.zeros(shape, dtype=dtype, device=self.device)
         return found
 
     def forget_derived(self) -> None:

@@ -722,6 +722,47 @@ def test_gemm_tall_swiglu(m, inter, k, tiles):
     assert torch.equal(out, out2)
 
 
+@pytest.mark.parametrize("n_heads,n_kv,head_dim,rows,count", [(8, 2, 128, 200, 4), (3, 1, 64, 64, 1), (4, 4, 32, 130, 3),
+                                                                  (2, 1, 256, 97, 2)])
+def test_rows_to_cache_from_partial_sums(n_heads, n_kv, head_dim, rows, count):
+    """A projection left as float partial sums goes to the cache and to the queries exactly as its rounded sum does:
+    the parts are made so that their sums are exact in float32 whatever the order."""
+    torch.manual_seed(rows + count)
+    o = ops()
+    cols = (n_heads + 2 * n_kv) * head_dim
+    parts = (torch.randint(-64, 65, (count, rows, cols)).float() / 16).to(DEV)
+    whole = parts.sum(0).to(torch.bfloat16)
+    n_slots, max_pages = 3, 4
+    n_pages = n_slots * max_pages
+    table = torch.randperm(n_pages, dtype=torch.int32).view(n_slots, max_pages).to(DEV)
+    row_slot = torch.tensor([0] * 70 + [-1] * 5 + [2] * (rows - 75) if rows > 75 else [1] * rows, dtype=torch.int32, device=DEV)
+    row_pos = torch.cat([torch.arange(70), torch.zeros(5), torch.arange(3, 3 + rows - 75)]).int().to(DEV) if rows > 75 \
+        else torch.arange(5, 5 + rows, dtype=torch.int32, device=DEV)
+    cos = torch.randn(256, head_dim // 2, device=DEV).to(torch.bfloat16)
+    sin = torch.randn(256, head_dim // 2, device=DEV).to(torch.bfloat16)
+    qw, kw = (1 + 0.1 * torch.randn(head_dim, device=DEV)).to(torch.bfloat16), (1 + 0.1 * torch.randn(head_dim, device=DEV)).to(torch.bfloat16)
+    got, want = [], []
+    for source, into in ((parts, got), (whole, want)):
+        k = torch.zeros(n_pages, n_kv, 64, head_dim, dtype=torch.bfloat16, device=DEV)
+        v = torch.zeros(n_pages, n_kv, head_dim, 64, dtype=torch.bfloat16, device=DEV)
+        q = torch.full((rows, n_heads, head_dim), float("nan"), dtype=torch.bfloat16, device=DEV)
+        if source is parts:
+            assert o.rows_to_cache_takes(rows, head_dim, head_dim, True)
+            o.rows_to_cache_from_partials(parts, qw, kw, 1e-6, cos, sin, head_dim, row_slot, row_pos, q, k, v, table,
+                                          n_heads, n_kv, head_dim)
+        else:
+            o.qk_norm_rope_kv(whole, qw, kw, 1e-6, cos, sin, head_dim, row_slot, row_pos, q, k, v, table, True, n_heads,
+                              n_kv, head_dim)
+        into.extend([q, k, v])
+    for a, b, what in zip(got, want, ("q", "k", "v")):
+        assert torch.equal(a, b), what
+    assert got[1].any() and got[2].any()
+    assert not o.rows_to_cache_takes(63, head_dim, head_dim, True) and not o.rows_to_cache_takes(rows, head_dim, head_dim // 2, True)
+    with pytest.raises(Exception, match="at least 64 rows"):
+        o.rows_to_cache_from_partials(parts[:, :10].contiguous(), qw, kw, 1e-6, cos, sin, head_dim, row_slot, row_pos, None,
+                                      got[1], got[2], table, n_heads, n_kv, head_dim)
+
+
 @pytest.mark.parametrize("m", [1, 65, 128, 129, 200, 256])
 @pytest.mark.parametrize("n,k,splits,tiles", [(2560, 4096, 6, 5), (77, 64, 1, 4), (100, 192, 3, 6), (136, 640, 4, 7),
                                               (64, 1024, 16, 8), (130, 9728, 6, 4), (1000, 1280, 2, 5)])
