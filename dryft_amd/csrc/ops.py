@@ -292,8 +292,8 @@ def rows_to_cache_from_partials(parts: torch.Tensor, q_weight, k_weight, eps: fl
         raise KernelError(f"rows_to_cache_from_partials: parts need {(n_heads + 2 * n_kv) * head_dim} columns, a multiple "
                           f"of 8; have {cols}")
     if not rows_to_cache_takes(rows, head_dim, rot, True):
-        raise KernelError(f"rows_to_cache_from_partials: takes steps of at least 64 rows, a full rotation and head sizes "
-                          f"32, 64, 128, 256; got {rows} rows, head size {head_dim}, rotation over {rot}")
+        raise KernelError(f"rows_to_cache_from_partials: takes a full rotation and head sizes 32, 64, 128, 256; got head "
+                          f"size {head_dim}, rotation over {rot}")
     has_norm = q_weight is not None
     w_f32 = 0
     if has_norm:

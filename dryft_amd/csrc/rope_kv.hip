@@ -403,10 +403,10 @@ static int launch_rows_to_cache(const void* qkv, int64_t qkv_stride, const void*
 
 // The many-row form of dryft_qk_norm_rope_kv below for a projection left as `parts` float partial sums
 // [parts, n_rows, qkv_stride] (bfloat16 activations, weights and cache): every value is the sum of its parts rounded
-// to bfloat16, then treated as there. For steps of at least 64 rows that write the cache, a full rotation and a head
-// size of 32, 64, 128 or 256: dryft_rows_to_cache_takes says whether a step qualifies.
+// to bfloat16, then treated as there. For steps that write the cache, a full rotation and a head size of 32, 64, 128
+// or 256: dryft_rows_to_cache_takes says whether a step qualifies.
 DRYFT_API int dryft_rows_to_cache_takes(int n_rows, int head_dim, int rot, int write_kv) {
-  return write_kv && n_rows >= 64 && rot == head_dim && (head_dim == 32 || head_dim == 64 || head_dim == 128 || head_dim == 256);
+  return write_kv && n_rows >= 1 && rot == head_dim && (head_dim == 32 || head_dim == 64 || head_dim == 128 || head_dim == 256);
 }
 
 DRYFT_API int dryft_rows_to_cache_parts(const float* qkv_parts, int parts, int64_t qkv_stride, const void* q_w,

@@ -29,8 +29,8 @@ from .linear import linear
 
 _RESIDENT_WORKGROUPS = 512     # of the split kernel: two per compute unit (its registers allow no more)
 _MAX_SPLITS = 32
-_QKV_PARTIAL_ROWS = 128         # decoding steps of up to so many rows take the projection as partial sums over K
-_PROMPT_PARTIAL_ROWS = (64, 256)     # and so do prompt steps of more than so many and at most so many rows
+_QKV_PARTIAL_ROWS = 256         # decoding steps of up to so many rows take the projection as partial sums over K
+_PROMPT_PARTIAL_ROWS = 256      # and so do prompt steps of at most so many rows
 
 
 class GQAAttention(Mixer):
@@ -82,19 +82,19 @@ class GQAAttention(Mixer):
         fused_decoding = decoding and self.n_heads // self.n_kv <= 16
         # The kernel that norms, rotates, appends and attends in one adds up partial sums of the projection on its way
         # in, so K may be split over workgroups. Measured on Qwen3-4B's sizes, a decoding step with the split against
-        # without: 2.980 against 3.008 ms at 8 sequences, 4.63 against 4.74 at 32; from 33 rows on the split product is
-        # the kernel that brings its operands straight into LDS (6.75 against 6.86 ms at 64 sequences for q/k/v alone,
-        # 8.92 against 9.04 ms at 96; at 256 sequences the vendor library's product is ahead, 19.0 against 19.3 ms).
+        # without: 2.980 against 3.008 ms at 8 sequences, 4.63 against 4.74 at 32, 6.75 against 6.86 at 64, 8.92 against
+        # 9.04 at 96 and, since the product whose waves own rows of x, 5.89 against 5.97 at 192.
         cos = sin = None
         if self.positions:
             table = ctx.positions[self.positions]
             cos, sin = table.cos, table.sin
             if ctx.max_kv_len > table.n_positions:
                 raise ValueError(f"position tables cover {table.n_positions} positions, the step reaches {ctx.max_kv_len}")
-        # So does the kernel that takes a short prompt's keys and values to the cache (and its queries out): at 65 to
-        # 256 rows the split product is ahead of the vendor library's (Qwen3-4B's q/k/v at 256 rows: 17.9 against 31.0 us).
+        # So does the kernel that takes a short prompt's keys and values to the cache (and its queries out): up to 256
+        # rows the split product is ahead of the vendor library's (Qwen3-4B's q/k/v: 11.7 against 15.2 us at 64 rows,
+        # 17.9 against 31.0 at 256).
         prompt_parts = matrix_cores and not decoding and writes_cache and cos is not None and \
-            _PROMPT_PARTIAL_ROWS[0] < rows <= _PROMPT_PARTIAL_ROWS[1] and \
+            rows <= _PROMPT_PARTIAL_ROWS and \
             ops.rows_to_cache_takes(rows, self.head_dim, self.rotary_dim, True)
         if prompt_parts:
             qkv = linear(h, self.w_qkv, allow_partials=True)

@@ -723,7 +723,7 @@ def test_gemm_tall_swiglu(m, inter, k, tiles):
 
 
 @pytest.mark.parametrize("n_heads,n_kv,head_dim,rows,count", [(8, 2, 128, 200, 4), (3, 1, 64, 64, 1), (4, 4, 32, 130, 3),
-                                                                  (2, 1, 256, 97, 2)])
+                                                                  (2, 1, 256, 97, 2), (8, 2, 128, 5, 2), (4, 2, 64, 33, 6)])
 def test_rows_to_cache_from_partial_sums(n_heads, n_kv, head_dim, rows, count):
     """A projection left as float partial sums goes to the cache and to the queries exactly as its rounded sum does:
     the parts are made so that their sums are exact in float32 whatever the order."""
@@ -757,10 +757,10 @@ def test_rows_to_cache_from_partial_sums(n_heads, n_kv, head_dim, rows, count):
     for a, b, what in zip(got, want, ("q", "k", "v")):
         assert torch.equal(a, b), what
     assert got[1].any() and got[2].any()
-    assert not o.rows_to_cache_takes(63, head_dim, head_dim, True) and not o.rows_to_cache_takes(rows, head_dim, head_dim // 2, True)
-    with pytest.raises(Exception, match="at least 64 rows"):
-        o.rows_to_cache_from_partials(parts[:, :10].contiguous(), qw, kw, 1e-6, cos, sin, head_dim, row_slot, row_pos, None,
-                                      got[1], got[2], table, n_heads, n_kv, head_dim)
+    assert not o.rows_to_cache_takes(rows, 48, 48, True) and not o.rows_to_cache_takes(rows, head_dim, head_dim // 2, True)
+    with pytest.raises(Exception, match="a full rotation"):
+        o.rows_to_cache_from_partials(parts, qw, kw, 1e-6, cos[:, :head_dim // 4].contiguous(), sin[:, :head_dim // 4].contiguous(),
+                                      head_dim // 2, row_slot, row_pos, None, got[1], got[2], table, n_heads, n_kv, head_dim)
 
 
 @pytest.mark.parametrize("m", [1, 65, 128, 129, 200, 256])
