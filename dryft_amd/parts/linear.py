@@ -141,6 +141,11 @@ def panel_swiglu_ok(x: torch.Tensor, w_gate_up: torch.Tensor) -> bool:
     return m <= WIDE_ROWS and k % ops.PANEL_GROUP == 0 and few_rows_ok(x, w_gate_up) and within_direct_reach(x, w_gate_up)
 
 
+_TALL_SMALL_BYTES = 128 << 20   # matrices from here on go to the kernel whose waves own rows of x already at 33 to 64 rows.
+# Whole decoding steps, ms, against the shared-activation kernel or the vendor library there: Qwen3-14B (down, 178 MB) 10.99
+# against 11.19 at 64 sequences, the same at 48. With every matrix beyond 48 MiB sent there Qwen3-14B gains more (10.89; 9.97
+# against 10.09 at 48), Qwen3-32B a little (20.35 against 20.63; 19.01 against 19.10), and Qwen3-8B (q/k/v 50 MB, down 100 MB)
+# loses (7.60 against 7.54 at 64), though each of its products alone is faster: so only the large ones.
 _TALL_SWIGLU_BYTES = 256 << 20  # gate/up matrices up to here go to the kernel whose waves own rows of x at 65 to 256 rows
 
 
@@ -196,6 +201,11 @@ def linear(x: torch.Tensor, w: torch.Tensor, *, out_dtype: torch.dtype | None = 
         if splits > 1:
             partials = torch.empty((splits, m, n), dtype=torch.float32, device=x.device)
             ops.gemm_mid_bf16(x, w, partials, splits)
+            return Partials(partials, splits)
+        if n * k * 2 >= _TALL_SMALL_BYTES:
+            tiles, splits = tall_plan(m, n, k)
+            partials = torch.empty((splits, m, n), dtype=torch.float32, device=x.device)
+            ops.gemm_tall_bf16(x, w, partials, splits, tiles)
             return Partials(partials, splits)
     if m <= WIDE_ROWS and few_ok:
         splits, group, depth = wide_plan(n, k, allow_partials)
