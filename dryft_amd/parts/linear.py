@@ -90,7 +90,9 @@ def _tall_plan(loaded: int, n: int, k: int) -> tuple[int, int]:
     + 0.074 * MB of W, rounds being how often the workgroups fill the 256 compute units. (A workgroup takes in all
     rows of x, 128 or 256 of them, over its run of K: that is what the time goes to, and why a split pays also where
     the outputs alone would fill the chip.) Its choice is within 5 % of the best measured pair for each of those
-    shapes. Against the kernel it replaces here (64 outputs a workgroup, every wave reading all rows of x from LDS),
+    shapes. The choice itself counts 0.42 us a MB of partial sums: the kernel that adds them up on its way in takes
+    0.19 us a MB more to read them (the norm after o and down at 256 rows: 6.9 us with eight parts, 21 MB; the
+    cache writer after q/k/v 12.0 us with four parts, 7.8 without). Against the kernel it replaces here (64 outputs a workgroup, every wave reading all rows of x from LDS),
     at 256 rows: Qwen3-4B's down 22.5 against 26.8, Qwen3-8B's 34.7 against 59.8, Qwen3-14B's 55.3 against 96.2."""
     groups = k // ops.TALL_GROUP
     best, best_cost = (4, 1), float("inf")
@@ -104,7 +106,7 @@ def _tall_plan(loaded: int, n: int, k: int) -> tuple[int, int]:
             seen.add(splits)
             per = -(-groups // splits)
             rounds = -(-(blocks * splits) // _COMPUTE_UNITS)
-            cost = 3.2 + rounds * (11.1 * loaded + 22.5 * 16 * tiles) * per * 128e-6 + 0.23e-6 * splits * loaded * n * 4 + \
+            cost = 3.2 + rounds * (11.1 * loaded + 22.5 * 16 * tiles) * per * 128e-6 + 0.42e-6 * splits * loaded * n * 4 + \
                 0.074e-6 * n * k * 2
             if cost < best_cost:
                 best, best_cost = (tiles, splits), cost
