@@ -777,7 +777,8 @@ DRYFT_API int dryft_gemm_panel_swiglu_bf16(const void* x, int64_t x_stride, cons
 // products with many outputs (q/k/v, gate/up). Measured, weights from memory, us at 80 / 128 / 192 rows against the
 // vendor library: Qwen3-4B's o 10.9 / 12.8 / 17.3 (21 / 25 / 19), down 19.1 / 21.0 / 28.5 (27 / 53 / 34); Qwen3-8B's o
 // 13.5 / 15.4 / 20.6 (21 / 25 / 34), down 29 / 38 / 53 (38 / 67 / 90); Qwen3-32B's o 26 / 29 / 39 (30 / 45 / 61), down
-// 72 / 88 / 111 (173 / 181 / 209).
+// 72 / 88 / 111 (173 / 181 / 209). Since the tall product below took the steps of 65 to 256 rows (its workgroups take
+// in fewer bytes of x for a row of W), this one serves those of 33 to 64 rows.
 #define MID_GROUP 64
 #define MID_STAGES 3
 #define MID_WAVES 4
