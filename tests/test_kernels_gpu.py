@@ -790,6 +790,30 @@ def test_gemm_tall(m, n, k, splits, tiles):
     assert torch.equal(parts, parts2)
 
 
+def test_gemm_tall_at_random_sizes():
+    """Forty shapes drawn with a fixed seed: any row count up to 256, output counts from 1, K of 1 to 40 groups,
+    every tile count, any split that leaves no run empty; both forms of the kernel."""
+    import random
+    rng = random.Random(7)
+    o = ops()
+    for case in range(40):
+        m, n, groups, tiles = rng.randint(1, 256), rng.randint(1, 700), rng.randint(1, 40), rng.randint(4, 8)
+        k = 64 * groups
+        splits = o.gemm_mid_splits(k, rng.randint(1, min(groups, 12)))
+        torch.manual_seed(case)
+        x, w = torch.randn(m, k).to(torch.bfloat16), (torch.randn(n, k) / math.sqrt(k)).to(torch.bfloat16)
+        parts = torch.full((splits, m, n), float("nan"), dtype=torch.float32, device=DEV)
+        o.gemm_tall_bf16(x.to(DEV), w.to(DEV), parts, splits, tiles)
+        close(parts.sum(0), x.double() @ w.double().T, torch.float32, what=f"tall, case {case}: {m}x{n}x{k}, {tiles} tiles, {splits} runs")
+        inter = max(1, n // 2)
+        w2 = (torch.randn(2 * inter, k) * 2 / math.sqrt(k)).to(torch.bfloat16)
+        gu = (x.double() @ w2.double().T).to(torch.bfloat16).float()
+        want = (torch.nn.functional.silu(gu[:, :inter]).to(torch.bfloat16).float() * gu[:, inter:]).to(torch.bfloat16)
+        out = torch.full((m, inter), float("nan"), dtype=torch.bfloat16, device=DEV)
+        o.gemm_tall_swiglu_bf16(x.to(DEV), w2.to(DEV), out, tiles)
+        close(out, want, torch.bfloat16, what=f"tall swiglu, case {case}: {m}x{inter}x{k}, {tiles} tiles")
+
+
 def test_gemm_tall_refuses():
     o = ops()
     w = torch.zeros(64, 128, dtype=torch.bfloat16, device=DEV)
