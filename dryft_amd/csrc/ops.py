@@ -20,7 +20,7 @@ _P, _I, _L, _F = c_void_p, c_int, c_int64, c_float
 _SIGNATURES = {
     "batch": {"dryft_prepare_batch": [_P, _P, _P, _I, _I, _P, _P, _P, _P, _P, _P, _P],
               "dryft_tile_prefix": [_P, _P, _I, _I, _P, _P]},
-    "embed": {"dryft_embed_rows": [_P, _P, _P, _I, _I, _I, _I, _P]},
+    "embed": {"dryft_embed_rows": [_P, _P, _P, _I, _I, _I, _I, _I, _P]},
     "norm": {"dryft_add_rmsnorm": [_P, _P, _I, _I, _L, _P, _I, _P, _P, _I, _I, _F, _I, _P],
              "dryft_add_rows": [_P, _P, _P, _L, _I, _P]},
     "activation": {"dryft_silu_mul": [_P, _P, _I, _I, _L, _I, _P]},
@@ -142,15 +142,20 @@ def tile_prefix(seq_slot, q_len, n_seqs: int, tile_rows: int, tile_cu) -> None:
 
 # ------------------------------------------------------------------------------------------- embed
 def embed_rows(tokens: torch.Tensor, table: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """``out[r] = table[tokens[r]]`` for a table ``[vocab, hidden]``; for several tables ``[tables, vocab, hidden]`` the same
+    rows of each, ``out[t, r] = table[t, tokens[r]]``."""
     _gpu(tokens, "tokens", torch.int32)
     _gpu(table, "table")
     _gpu(out, "out", table.dtype)
-    n, (vocab, hidden) = tokens.numel(), table.shape
-    if not (table.is_contiguous() and out.is_contiguous() and tokens.is_contiguous()):
-        raise KernelError("embed_rows: contiguous operands")
-    if not (out.shape == (n, hidden)):
-        raise KernelError(f"embed_rows: out is {tuple(out.shape)}, expected {(n, hidden)}")
-    _check(_fn("embed", "dryft_embed_rows")(_ptr(tokens), _ptr(table), _ptr(out), n, hidden, vocab,
+    n = tokens.numel()
+    tables = table.shape[0] if table.dim() == 3 else 1
+    vocab, hidden = table.shape[-2:]
+    if not (table.dim() in (2, 3) and table.is_contiguous() and out.is_contiguous() and tokens.is_contiguous()):
+        raise KernelError("embed_rows: contiguous operands, the table [vocab, hidden] or [tables, vocab, hidden]")
+    want = (n, hidden) if table.dim() == 2 else (tables, n, hidden)
+    if not (out.shape == want):
+        raise KernelError(f"embed_rows: out is {tuple(out.shape)}, expected {want}")
+    _check(_fn("embed", "dryft_embed_rows")(_ptr(tokens), _ptr(table), _ptr(out), n, hidden, vocab, tables,
                                             _float_flag(table, "table"), _stream()), "embed_rows")
     return out
 

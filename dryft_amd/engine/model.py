@@ -164,10 +164,8 @@ def _pick_rows(x, rows: torch.Tensor):
     if x is None:
         return None
     if isinstance(x, Partials):
-        count, n, width = x.count, x.data.shape[1], x.data.shape[2]
-        table = x.data[:count].reshape(count * n, width)
-        index = (rows[None, :] + n * torch.arange(count, dtype=torch.int32, device=rows.device)[:, None]).reshape(-1)
-        picked = torch.empty((count * rows.numel(), width), dtype=table.dtype, device=table.device)
-        return Partials(ops.embed_rows(index.contiguous(), table, picked).view(count, rows.numel(), width), count)
+        parts = x.data[:x.count]
+        picked = torch.empty((x.count, rows.numel(), parts.shape[2]), dtype=parts.dtype, device=parts.device)
+        return Partials(ops.embed_rows(rows, parts, picked), x.count)
     picked = torch.empty((rows.numel(), x.shape[1]), dtype=x.dtype, device=x.device)
     return ops.embed_rows(rows, x, picked)

@@ -37,6 +37,13 @@ def test_embed_rows(dtype):
     out = torch.empty(7, 100, dtype=dtype, device=DEV)
     ops().embed_rows(tokens.to(DEV), table.to(DEV), out)
     assert torch.equal(out.cpu(), table[tokens.long()])
+    # the same rows of each of several tables (the wanted rows of a product left as partial sums)
+    tables = torch.randn(5, 331, 100).to(dtype)
+    outs = torch.full((5, 7, 100), float("nan"), dtype=dtype, device=DEV)
+    ops().embed_rows(tokens.to(DEV), tables.to(DEV), outs)
+    assert torch.equal(outs.cpu(), tables[:, tokens.long()])
+    with pytest.raises(Exception, match="expected"):
+        ops().embed_rows(tokens.to(DEV), tables.to(DEV), out)
 
 
 # -------------------------------------------------------------------------------------------- norm
